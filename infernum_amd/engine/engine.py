@@ -1,0 +1,211 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step takes any mix of portions of prompts and single decoded tokens, cut
+anywhere, runs only those tokens against what earlier steps left in the cache,
+and returns fp32 logits at the wanted places.  The reference has two calls for
+this, one whole prompt of one request (``forward_prefill``, infernum/src/model.rs:
+96-103, whose start position the CUDA engine ignores,
+infernum-cuda/src/inner/cuda_graph_engine.rs:1318,1363) and one token of each of B
+requests (``forward_batch_decode``, model.rs:121-132); here they are one.
+
+The engine owns the model and the cache manager.  It packs the batch into one
+int32 buffer, copies it to the device once, and runs the model's forward pass.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheConfig, CacheManager
+from ..models.model import DecoderModel
+from ..parts.base import Runtime, StepContext
+
+PREFILL_TILE_ROWS = 64      # query rows per workgroup of the tiled prefill attention
+
+
+class OutOfPages(RuntimeError):
+    """The pool has too few free pages (or state slots) for this step; nothing was changed."""
+
+
+class StepError(ValueError):
+    """A step's entries are malformed (unknown place wanted, token outside the vocabulary, ...)."""
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)     # places among ``tokens`` whose logits are wanted
+
+
+def _align4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, cache_config: CacheConfig):
+        self.model = model
+        self.rt: Runtime = model.rt
+        self.spec = model.spec
+        self.cache = CacheManager(model.cache_needs(), [e.cache_of for e in model.spec.schedule], cache_config,
+                                  dtype=self.rt.dtype, device=self.rt.device)
+        self.views = self.cache.views()
+        self.steps_run = 0
+
+    # ---- building ------------------------------------------------------------------
+    @staticmethod
+    def runtime(dtype: Any = "bfloat16", device: Any = "cuda:0", max_tokens_per_step: int = 8192) -> Runtime:
+        from ..kernels.api import KernelError
+        dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+              "f32": torch.float32, torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}.get(dtype)
+        if dt is None:
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
+        dev = torch.device(device)
+        if dev.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError("infernum_amd runs on a gfx950 GPU only: no GPU is visible (there is no CPU fallback)")
+        return Runtime(dev, dt, max_tokens_per_step)
+
+    @classmethod
+    def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", cache_config: Optional[CacheConfig] = None,
+                        device: Any = "cuda:0", **runtime_kw: Any) -> "Engine":
+        """Model class by config.json's model_type, weights from the folder's safetensors."""
+        from .. import models  # noqa: F401  (registers the architectures)
+        from ..config.registry import load_config, model_spec_for
+        from ..weights.loader import load_weights
+        from ..kernels.api import load_library
+        rt = cls.runtime(dtype, device, **runtime_kw)
+        load_library("core")
+        config = load_config(model_dir)
+        model = DecoderModel(model_spec_for(config), rt)
+        load_weights(model, model_dir)
+        eng = cls(model, cache_config or CacheConfig())
+        eng.config = config
+        return eng
+
+    @classmethod
+    def from_config(cls, config: Any, seed: int = 0, dtype: Any = "bfloat16",
+                    cache_config: Optional[CacheConfig] = None, device: Any = "cuda:0",
+                    spec_kw: Optional[Dict[str, Any]] = None, **runtime_kw: Any) -> "Engine":
+        """Random weights made on the device from (config, seed); nothing is read or written."""
+        from .. import models  # noqa: F401
+        from ..config.registry import model_spec_for
+        from ..weights.random_init import random_weights_on_device
+        from ..kernels.api import load_library
+        rt = cls.runtime(dtype, device, **runtime_kw)
+        load_library("core")
+        model = DecoderModel(model_spec_for(config, **(spec_kw or {})), rt)
+        random_weights_on_device(model, seed)
+        eng = cls(model, cache_config or CacheConfig())
+        eng.config = config
+        return eng
+
+    # ---- the step ------------------------------------------------------------------
+    def pages_short(self, entries: Sequence[StepEntry]) -> bool:
+        """True when the pool cannot hold this step's new tokens."""
+        for g in self.cache.groups:
+            need = 0
+            for e in entries:
+                if self.cache.has(e.request):
+                    need += g.pages_missing(e.request, len(e.tokens))
+                else:
+                    need += (len(e.tokens) + g.page_size - 1) // g.page_size
+            if need > g.allocator.num_free:
+                return True
+        new = sum(1 for e in entries if not self.cache.has(e.request))
+        return new > self.cache.slots.num_free
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns logits [sum(len(want)), vocab] fp32 in the order of entries and of ``want``."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        V = self.spec.vocab_size
+        if not entries:
+            return torch.empty((0, V), dtype=torch.float32, device=self.rt.device)
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} stands twice in one step")
+            seen.add(e.request)
+            if len(e.tokens) == 0:
+                raise StepError(f"request {e.request!r} brings no tokens")
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+        total = sum(len(e.tokens) for e in entries)
+        if total > self.rt.max_tokens_per_step:
+            raise StepError(f"a step of {total} tokens is above max_tokens_per_step {self.rt.max_tokens_per_step}")
+        if self.pages_short(entries):
+            raise OutOfPages(f"not enough free pages or state slots for a step of {total} tokens")
+        cache = self.cache
+        for e in entries:
+            if not cache.has(e.request):
+                cache.admit(e.request)
+            ok = cache.reserve(e.request, len(e.tokens))
+            assert ok
+
+        # single tokens first, portions of prompts after them
+        order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
+        batch = [entries[i] for i in order]
+        B = len(batch)
+        num_decode = sum(1 for e in batch if len(e.tokens) == 1)
+        q_lens = [len(e.tokens) for e in batch]
+        ctx_lens = [cache.num_tokens(e.request) for e in batch]
+        starts = np.zeros(B + 1, dtype=np.int32)
+        starts[1:] = np.cumsum(q_lens)
+        N = int(starts[-1])
+        start_of = {e.request: int(starts[i]) for i, e in enumerate(batch)}
+
+        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in batch])
+        if token_ids.min() < 0 or token_ids.max() >= V:
+            raise StepError(f"token id outside the vocabulary [0, {V})")
+        positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(ctx_lens, q_lens)])
+        token_seq = np.repeat(np.arange(B, dtype=np.int32), q_lens)
+        logit_rows = np.asarray([start_of[e.request] + w for e in entries for w in e.want], dtype=np.int32)
+        state_slots = np.asarray([cache.state_slot(e.request) for e in batch], dtype=np.int32)
+        reqs = [e.request for e in batch]
+        tiles = [(s, r) for s in range(num_decode, B) for r in range(0, q_lens[s], PREFILL_TILE_ROWS)]
+        tiles_np = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+
+        segs: List[np.ndarray] = [token_ids.astype(np.int32), positions, token_seq, starts,
+                                  np.asarray(ctx_lens, dtype=np.int32), state_slots, logit_rows, tiles_np.reshape(-1)]
+        bt_shapes = []
+        for g in cache.groups:
+            bt = cache.block_table_rows(g.index, reqs)
+            bt_shapes.append(bt.shape)
+            segs.append(np.concatenate([cache.token_slots(g.index, r, c, q)
+                                        for r, c, q in zip(reqs, ctx_lens, q_lens)]))
+            segs.append(bt.reshape(-1))
+        offs, total_ints = [], 0
+        for s in segs:
+            offs.append(total_ints)
+            total_ints += _align4(max(s.size, 1))
+        host = np.zeros(total_ints, dtype=np.int32)
+        for o, s in zip(offs, segs):
+            host[o:o + s.size] = s
+        dev = torch.from_numpy(host).to(self.rt.device)
+
+        def seg(i: int) -> torch.Tensor:
+            return dev[offs[i]:offs[i] + segs[i].size]
+
+        ctx = StepContext(
+            num_tokens=N, num_seqs=B, num_decode=num_decode,
+            token_ids=seg(0), positions=seg(1), token_seq=seg(2), seq_starts=seg(3), seq_ctx=seg(4),
+            state_slots=seg(5), logit_rows=seg(6),
+            block_tables=[seg(9 + 2 * gi).view(bt_shapes[gi]) for gi in range(len(cache.groups))],
+            slots=[seg(8 + 2 * gi) for gi in range(len(cache.groups))],
+            q_lens=q_lens, ctx_lens=ctx_lens, max_q_len=max(q_lens),
+            max_total_len=max(c + q for c, q in zip(ctx_lens, q_lens)),
+            prefill_tiles=seg(7).view(-1, 2), num_prefill_tiles=len(tiles),
+        )
+        logits = self.model.forward(ctx, self.views)
+        for e in batch:
+            cache.commit(e.request, len(e.tokens))
+        self.steps_run += 1
+        return logits
+
+    def end(self, request: Hashable) -> None:
+        """The request is finished: its pages and its state slot are given back."""
+        if self.cache.has(request):
+            self.cache.release(request)

@@ -1,0 +1,274 @@
+"""Python face of the HIP kernels: shape checks on the host, then one C call.
+
+Every function checks that its operands are what the kernel and its grid assume
+(device, dtype, contiguity, sizes) before anything is launched, and launches on
+torch's current stream, so that calls order with torch's own work and can be
+captured into a HIP graph.  There is no fallback: without a GPU or without the
+built library a call raises :class:`KernelError`.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import build as _build
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+_libs: Dict[str, ctypes.CDLL] = {}
+
+_ERRORS = {10001: "bad argument", 10002: "size not supported by this kernel"}
+
+
+def load_library(name: str) -> ctypes.CDLL:
+    lib = _libs.get(name)
+    if lib is None:
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: infernum_amd runs on a gfx950 GPU only (there is no CPU fallback)")
+        try:
+            path = _build.ensure(name)
+            lib = ctypes.CDLL(path)
+        except (OSError, _build.BuildError) as e:
+            raise KernelError(f"the HIP kernel library '{name}' could not be built or loaded: {e}") from e
+        _libs[name] = lib
+    return lib
+
+
+def _core() -> ctypes.CDLL:
+    return load_library("core")
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ok(code: int, what: str) -> None:
+    if code != 0:
+        why = _ERRORS.get(code, f"HIP error {code}")
+        raise KernelError(f"{what}: {why}")
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "operand is not on the GPU")
+            _need(t.is_contiguous(), "operand is not contiguous")
+
+
+def _i32(t: torch.Tensor, n: int, what: str) -> None:
+    _need(t.dtype == torch.int32 and t.is_cuda and t.is_contiguous() and t.numel() >= n,
+          f"{what}: needs a contiguous int32 GPU tensor of at least {n} elements")
+
+
+# --------------------------------------------------------------------------- rows
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n, :] = float(table[ids[n], :]); out is fp32 [N, H]."""
+    _dev(table, ids, out)
+    V, H = table.shape
+    N = ids.numel()
+    _need(table.dtype in DTYPE_CODE, f"embed: table dtype {table.dtype}")
+    _i32(ids, N, "embed ids")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == (N, H), f"embed: out must be fp32 [{N}, {H}]")
+    _ok(_core().ia_embed(_p(table), DTYPE_CODE[table.dtype], _p(ids), _p(out), N, H, V, _stream()), "embed")
+    return out
+
+
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h += delta (fp32, in place); out = h * rsqrt(mean(h^2) + eps) * weight.
+
+    With ``rows`` the norm is taken of the selected rows only and h stays as it is.
+    """
+    _dev(h, delta, weight, out, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "add_rmsnorm: h must be fp32 [N, H]")
+    H = h.shape[1]
+    n_out = rows.numel() if rows is not None else h.shape[0]
+    _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (n_out, H), f"add_rmsnorm: out must be [{n_out}, {H}]")
+    if delta is not None:
+        _need(delta.dtype == out.dtype and tuple(delta.shape) == tuple(h.shape),
+              "add_rmsnorm: delta must have h's shape and out's dtype")
+    _need(weight.dtype in DTYPE_CODE and weight.numel() == H, f"add_rmsnorm: weight must hold {H} values")
+    if rows is not None:
+        _i32(rows, n_out, "add_rmsnorm rows")
+    _ok(_core().ia_add_rmsnorm(_p(h), _p(delta), DTYPE_CODE[out.dtype], _p(weight), DTYPE_CODE[weight.dtype],
+                               _p(out), _p(rows), n_out, H, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _dev(h, delta)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and tuple(delta.shape) == tuple(h.shape)
+          and delta.dtype in DTYPE_CODE, "residual_add: h fp32 [N, H], delta of the same shape")
+    _ok(_core().ia_residual_add(_p(h), _p(delta), DTYPE_CODE[delta.dtype], h.shape[0], h.shape[1], _stream()),
+        "residual_add")
+    return h
+
+
+def rope_kv_append(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], nh: int, nkv: int,
+                   d: int, rot: int, slots: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
+                   v_pages: Optional[torch.Tensor] = None) -> None:
+    """Rotate q (in place) and k, and write k and v to their page slots.
+
+    qkv is [N, (nh + 2 nkv) d] (or [N, nh d] when no pages are given).  Pages are
+    [num_pages, nkv, page_size, d].
+    """
+    _dev(qkv, positions, inv_freq, slots, k_pages, v_pages)
+    write = k_pages is not None
+    N, row = qkv.shape
+    _need(qkv.dtype in DTYPE_CODE, "rope: dtype")
+    _need(row >= (nh + (2 * nkv if write else 0)) * d, "rope: row of qkv is too short for its heads")
+    _i32(positions, N, "rope positions")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2 and rot % 2 == 0 and 0 < rot <= d,
+              "rope: inv_freq must hold rot/2 fp32 values, rot even and at most the head size")
+    page_size = num_pages = 0
+    if write:
+        _need(v_pages is not None and slots is not None, "rope: k_pages, v_pages and slots go together")
+        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "rope: pages must have qkv's dtype")
+        _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
+              and tuple(v_pages.shape) == tuple(k_pages.shape), "rope: pages must be [num_pages, nkv, page_size, d]")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+        _i32(slots, N, "rope slots")
+    _ok(_core().ia_rope_kv_append(_p(qkv), DTYPE_CODE[qkv.dtype], _p(positions), _p(slots), _p(inv_freq),
+                                  _p(k_pages), _p(v_pages), N, row, nh, nkv, d, rot if inv_freq is not None else 0,
+                                  page_size, num_pages, 1 if write else 0, _stream()), "rope_kv_append")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+    _dev(gate_up, out)
+    N, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (N, two_i // 2) and out.dtype == gate_up.dtype
+          and out.dtype in DTYPE_CODE, "swiglu: gate_up [N, 2I] and out [N, I] of one dtype")
+    _ok(_core().ia_swiglu(_p(gate_up), _p(out), DTYPE_CODE[out.dtype], N, two_i // 2, _stream()), "swiglu")
+    return out
+
+
+# ------------------------------------------------------------------ matrix products
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T with fp32 multiply-adds in the order of k."""
+    _dev(w, out)
+    _need(a.is_cuda and a.dim() == 2 and a.stride(1) == 1, "gemm: a must be a GPU matrix with unit inner stride")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.dim() == 2 and w.shape[1] == K, f"gemm: weight must be [N, {K}], got {tuple(w.shape)}")
+    _need(a.dtype == w.dtype and a.dtype in DTYPE_CODE and out.dtype in DTYPE_CODE, "gemm: dtypes")
+    _need(tuple(out.shape) == (M, N), f"gemm: out must be [{M}, {N}]")
+    lda = a.stride(0) if M > 1 else K
+    _need(lda >= K, "gemm: a's rows overlap")
+    _ok(_core().ia_gemm_generic(_p(a), _p(w), _p(out), DTYPE_CODE[a.dtype], DTYPE_CODE[out.dtype], M, N, K, lda, K, N,
+                                _stream()), "gemm_generic")
+    return out
+
+
+SKINNY_MAX_M = 64
+
+
+def gemm_skinny_supported(M: int, N: int, K: int) -> bool:
+    return 0 < M <= SKINNY_MAX_M and K % 32 == 0 and K >= 32 and N >= 1
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """bf16 out[M, N] (or fp32) = a[M, K] @ w[N, K]^T for M <= 64 on MFMA, weights streamed once."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in DTYPE_CODE, "gemm_skinny: bf16 in")
+    _need(w.dim() == 2 and w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_skinny: shapes")
+    _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 64, K % 32 == 0)")
+    _ok(_core().ia_gemm_skinny(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, _stream()), "gemm_skinny")
+    return out
+
+
+# ------------------------------------------------------------------------ attention
+def _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, what):
+    _dev(qkv, k_pages, v_pages, out, block_tables)
+    _need(qkv.dtype == out.dtype == k_pages.dtype == v_pages.dtype and qkv.dtype in DTYPE_CODE,
+          f"{what}: q, pages and out must share one dtype")
+    _need(qkv.dim() == 2 and qkv.shape[1] >= nh * d, f"{what}: q rows must hold nh*d values")
+    _need(out.dim() == 2 and out.shape[1] == nh * d and out.shape[0] == qkv.shape[0],
+          f"{what}: out must be [N, nh*d]")
+    _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
+          and tuple(v_pages.shape) == tuple(k_pages.shape), f"{what}: pages must be [num_pages, nkv, page_size, d]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, f"{what}: block_tables int32 [B, MB]")
+    _need(nh % nkv == 0, f"{what}: nh must be a multiple of nkv")
+
+
+def attention_generic(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                      token_seq: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor, nh: int,
+                      nkv: int, d: int, scale: float, window: int = 0) -> None:
+    """Causal paged attention, one wave per (token, head), fp32 arithmetic.
+
+    qkv [N, >= nh*d]: the q heads of token n are the first nh*d values of row n.
+    token_seq[n] is the row of block_tables of token n; positions[n] its position.
+    """
+    _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, "attention")
+    N = out.shape[0]
+    _i32(token_seq, N, "attention token_seq")
+    _i32(positions, N, "attention positions")
+    _need(0 < d <= 256, "attention: head size must be at most 256")
+    _ok(_core().ia_attention_generic(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d,
+                                     DTYPE_CODE[out.dtype], _p(token_seq), _p(positions), _p(block_tables),
+                                     block_tables.shape[1], N, nh, nkv, d, k_pages.shape[2], k_pages.shape[0],
+                                     ctypes.c_float(scale), int(window), _stream()), "attention_generic")
+
+
+# ------------------------------------------------------------------------- sampling
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(logits, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "argmax: logits must be fp32")
+    _i32(out, R, "argmax out")
+    _ok(_core().ia_argmax(_p(logits), V, _p(out), R, V, _stream()), "argmax")
+    return out
+
+
+def repetition_penalty(logits: torch.Tensor, recent: torch.Tensor, counts: torch.Tensor,
+                       penalty: torch.Tensor) -> None:
+    _dev(logits, recent, counts, penalty)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "penalty: logits must be fp32")
+    _need(recent.dtype == torch.int32 and recent.dim() == 2 and recent.shape[0] == R, "penalty: recent int32 [R, W]")
+    _i32(counts, R, "penalty counts")
+    _need(penalty.dtype == torch.float32 and penalty.numel() == R, "penalty: one fp32 factor per row")
+    _ok(_core().ia_repetition_penalty(_p(logits), V, _p(recent), recent.shape[1], _p(counts), _p(penalty), R, V,
+                                      _stream()), "repetition_penalty")
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
+           u: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(logits, work, temperature, top_p, u, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and work.dtype == torch.float32 and work.numel() >= R * V,
+          "sample: logits fp32 [R, V] and fp32 work space of the same size")
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("u", u)):
+        _need(t.dtype == torch.float32 and t.numel() == R, f"sample: {name} must hold one fp32 value per row")
+    _i32(out, R, "sample out")
+    _ok(_core().ia_sample(_p(logits), V, _p(work), _p(temperature), _p(top_p), _p(u), _p(out), R, V, _stream()),
+        "sample")
+    return out
+
+
+# ------------------------------------------------------- which fast kernels are built
+_has: Dict[str, bool] = {}
+
+
+def gemm_skinny_available() -> bool:
+    if "skinny" not in _has:
+        _has["skinny"] = hasattr(_core(), "ia_gemm_skinny")
+    return _has["skinny"]

@@ -1,0 +1,106 @@
+"""A decoder built from a :class:`ModelSpec`: the parts, their weights' names,
+and the forward pass of one step over the schedule of layer runs.
+
+This file holds no architecture: which parts a model has, and in which order
+its layers run, is data (the reference builds the same sequence as a graph,
+infernum-llama/src/graph_builder.rs:399-549 for whole prompts and :756-921 for
+batched decoding; here one forward serves both).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..parts.base import (Block, CacheSpec, CacheView, ModelSpec, Part, PartSpec, Runtime, StateSpec, StepContext,
+                          WeightSpec, block_factory, make_part)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, rt: Runtime):
+        self.spec = spec
+        self.rt = rt
+        self._parts: List[Tuple[str, Part]] = []        # (prefix, part) of everything that has weights
+        self.embedding = self._make("embedding", spec.embedding)
+        self.blocks: List[Block] = []
+        for ls in spec.layers:
+            mixer = self._make("mixer", ls.mixer)
+            ff = self._make("feed_forward", ls.feed_forward)
+            n1 = self._make("norm", ls.mixer_norm)
+            n2 = self._make("norm", ls.feed_forward_norm)
+            extra = {name: self._make("norm", ps) for name, ps in ls.extra.items()}
+            self.blocks.append(block_factory(ls.block)(rt, mixer, ff, n1, n2, extra))
+        self.final_norm = self._make("norm", spec.final_norm) if spec.final_norm is not None else None
+        self.head = self._make("head", spec.head)
+        self._check_schedule()
+
+    def _make(self, category: str, ps: PartSpec) -> Part:
+        part = make_part(category, ps, self.rt)
+        self._parts.append((ps.prefix, part))
+        return part
+
+    def _check_schedule(self) -> None:
+        n_layers = len(self.spec.layers)
+        for i, e in enumerate(self.spec.schedule):
+            if not 0 <= e.layer < n_layers:
+                raise ValueError(f"schedule entry {i} names layer {e.layer}, but there are {n_layers} layers")
+            if e.cache_of is not None:
+                if not 0 <= e.cache_of < i:
+                    raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_of}, which does not run before it")
+                if self.spec.schedule[e.cache_of].cache_of is not None:
+                    raise ValueError(f"schedule entry {i} reads entry {e.cache_of}, which has no cache of its own")
+                a = self.blocks[e.layer].mixer.cache_spec()
+                b = self.blocks[self.spec.schedule[e.cache_of].layer].mixer.cache_spec()
+                if a != b:
+                    raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_of}: {a} != {b}")
+
+    # ---- weights -------------------------------------------------------------
+    def expected_weights(self) -> Dict[str, WeightSpec]:
+        """Full tensor name -> what is expected of it."""
+        out: Dict[str, WeightSpec] = {}
+        for prefix, part in self._parts:
+            for local, ws in part.weights().items():
+                name = prefix + local
+                if name in out and out[name] != ws:
+                    raise ValueError(f"two parts want tensor {name!r} differently")
+                out[name] = ws
+        return out
+
+    def load_weights(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """``tensors``: full name -> device tensor, already checked and converted."""
+        for prefix, part in self._parts:
+            wanted = part.weights()
+            if wanted:
+                part.load({local: tensors[prefix + local] for local in wanted})
+
+    # ---- cache needs ---------------------------------------------------------
+    def cache_needs(self) -> List[Tuple[Optional[CacheSpec], Optional[StateSpec]]]:
+        """Per schedule entry: the pages and the per-request state its mixer wants
+        (None, None for an entry that reads another entry's)."""
+        needs = []
+        for e in self.spec.schedule:
+            if e.cache_of is not None:
+                needs.append((None, None))
+            else:
+                m = self.blocks[e.layer].mixer
+                needs.append((m.cache_spec(), m.state_spec()))
+        return needs
+
+    # ---- one step --------------------------------------------------------------
+    def forward(self, ctx: StepContext, views: List[CacheView]) -> torch.Tensor:
+        """Runs the tokens of ``ctx`` and returns fp32 logits [R, V] at ctx.logit_rows."""
+        h = self.embedding.forward(ctx)
+        pending: Optional[torch.Tensor] = None
+        for e, view in zip(self.spec.schedule, views):
+            pending = self.blocks[e.layer].forward(h, pending, ctx, view)
+        rows = ctx.logit_rows
+        if rows.numel() == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
+        if self.final_norm is not None:
+            f = self.final_norm.forward(h, pending, rows=rows)
+        else:
+            from ..kernels import api as K
+            if pending is not None:
+                K.residual_add(h, pending)
+            f = h.index_select(0, rows.long()).to(self.rt.dtype)
+        return self.head.forward(f)

@@ -1,0 +1,104 @@
+"""Grouped-query attention over the paged cache.
+
+q = x Wq^T, k = x Wk^T, v = x Wv^T without bias; heads are consecutive within a
+row; q and k are rotated, then k and v are written to the pages at the tokens'
+positions; query head h reads key/value head h // (nh / nkv); scores are
+scale * <q, k_j> over the keys 0 .. p of the same request (the last ``window``
+of them when a window is set), softmax with the maximum subtracted, output
+sum_j w_j v_j; then the output projection.  (infernum-llama/src/graph_builder.rs:
+456-483 and 819-867; infernum-cuda/kernels/paged_decode_attention.cu:319-430;
+kernels/flash_prefill_attention_v2.cu:85-88 for the causal range with a window.)
+
+The three projections are kept as one [ (nh + 2 nkv) d, H ] matrix (row-wise
+concatenation, as the reference's optional fused weight,
+infernum-cuda/src/inner/weights/generic_impl.rs:153-180).
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import api as K
+from .base import (CacheSpec, CacheView, Mixer, PartSpec, Runtime, StepContext, WeightSpec, make_part,
+                   register_part)
+from .linear import linear
+
+
+class Attention(Mixer):
+    def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[Mapping[str, Any]] = None, window: Optional[int] = None,
+                 scale: Optional[float] = None, kernels: str = "auto", init_std: float = 0.02):
+        super().__init__(rt)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        if head_dim > 256:
+            raise ValueError(f"head size {head_dim} is above 256, the largest the attention kernels take")
+        self.hidden_size, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.window = int(window) if window else 0
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.kernels = kernels
+        self.init_std = init_std
+        pos_spec = PartSpec(**position) if isinstance(position, Mapping) else (position or PartSpec("none"))
+        self.position = make_part("position", pos_spec, rt)
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+        if kernels not in ("auto", "generic"):
+            raise ValueError("kernels must be 'auto' or 'generic'")
+        self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and self.d % 16 == 0)
+
+    # ---- what it needs ---------------------------------------------------
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec("window" if self.window else "full", self.nkv, self.d, self.window)
+
+    def weights(self) -> Dict[str, WeightSpec]:
+        nh, nkv, d, H = self.nh, self.nkv, self.d, self.hidden_size
+        init = ("normal", self.init_std)
+        return {
+            "q_proj.weight": WeightSpec((nh * d, H), init),
+            "k_proj.weight": WeightSpec((nkv * d, H), init),
+            "v_proj.weight": WeightSpec((nkv * d, H), init),
+            "o_proj.weight": WeightSpec((H, nh * d), init),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
+        self.w_qkv = self.w_qkv.contiguous()
+        self.w_o = tensors["o_proj.weight"].contiguous()
+
+    # ---- one step --------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView) -> torch.Tensor:
+        nh, nkv, d = self.nh, self.nkv, self.d
+        if cache.k_pages is None:
+            raise K.KernelError("attention needs pages of the cache")
+        g = cache.group
+        if cache.writable:
+            qkv = linear(x, self.w_qkv)
+            K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
+                             ctx.slots[g], cache.k_pages, cache.v_pages)
+        else:
+            # keys and values of another run of a layer: only queries are made here
+            qkv = linear(x, self.w_qkv[: nh * d])
+            K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim)
+        out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+        self.attend(qkv, out, ctx, cache)
+        return linear(out, self.w_o)
+
+    def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
+        nh, nkv, d = self.nh, self.nkv, self.d
+        bt = ctx.block_tables[cache.group]
+        if not self.use_mfma:
+            K.attention_generic(qkv, cache.k_pages, cache.v_pages, out, ctx.token_seq, ctx.positions, bt, nh, nkv, d,
+                                self.scale, self.window)
+            return
+        nd = ctx.num_decode
+        if nd > 0:
+            K.attention_decode(qkv[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.positions[:nd], bt[:nd], nh, nkv,
+                               d, self.scale, self.window, ctx.max_total_len, ctx.extras.get("decode_workspace"))
+        if ctx.num_seqs > nd:
+            K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
+                                ctx.prefill_tiles, ctx.num_prefill_tiles, nh, nkv, d, self.scale, self.window)
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,293 @@
+"""What a model is put together from: part specifications, the registry of part
+kinds, and the interfaces that a mixer, a feed-forward, a norm, a position
+encoding and a block arrangement have to keep.
+
+A part is made from a :class:`PartSpec` (its kind and its own sizes and
+constants) and knows nothing about the model it sits in: not its name, not its
+other layers, not the names of its weights in a file (those are given to it as a
+prefix).  The reference gets the same separation from its ``define_block!``
+macro (infernum-macros/src/lib.rs:32-106) and builds a layer from such blocks in
+infernum-llama/src/graph_builder.rs:446-507.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Mapping, Optional, Sequence, Tuple
+
+import torch
+
+# ----------------------------------------------------------------------- specs
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """Kind of a part, its parameters, and the prefix of its weights' names."""
+
+    kind: str
+    params: Mapping[str, Any] = field(default_factory=dict)
+    prefix: str = ""
+
+    def with_prefix(self, prefix: str) -> "PartSpec":
+        return PartSpec(self.kind, self.params, prefix)
+
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One tensor a part wants: its shape, how random weights are drawn for it,
+    whether it is a matrix that follows the compute dtype, and the full name of
+    another tensor that stands in when the file does not hold this one."""
+
+    shape: Tuple[int, ...]
+    init: Tuple = ("normal", 0.02)          # ("normal", std) | ("ones",) | ("uniform", lo, hi) | ("zeros",)
+    follows_compute_dtype: bool = True      # False: kept as stored (fp32 stays fp32, integers become int32)
+    fallback: Optional[str] = None          # full tensor name used when this one is absent
+    write_when_random: bool = True          # False: random-weights mode leaves it out (e.g. a tied head)
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer needs of the paged cache: keys and values of all positions
+    ('full') or of the last ``window`` positions ('window')."""
+
+    kind: str                      # "full" | "window"
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+    def group_key(self) -> Tuple:
+        """Layers with equal keys share page tables (one group of the cache manager)."""
+        return (self.kind, self.window)
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state per request that a mixer keeps between steps (fp32 unless said)."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer: how its parts are arranged (``block``) and the parts themselves."""
+
+    block: str
+    mixer: PartSpec
+    feed_forward: PartSpec
+    mixer_norm: PartSpec
+    feed_forward_norm: PartSpec
+    extra: Mapping[str, PartSpec] = field(default_factory=dict)   # further norms of other arrangements
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    """One run of a layer.  ``cache_of`` names an earlier entry of the schedule
+    whose keys and values (or state) this run reads instead of writing its own."""
+
+    layer: int
+    cache_of: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    """A whole decoder as data: embedding, layers, the order they run in, head."""
+
+    vocab_size: int
+    hidden_size: int
+    embedding: PartSpec
+    layers: Sequence[LayerSpec]
+    schedule: Sequence[ScheduleEntry]
+    final_norm: Optional[PartSpec]
+    head: PartSpec
+    max_position: int = 0
+    bos_token_id: Optional[int] = None
+    eos_token_id: Optional[int] = None
+
+
+# -------------------------------------------------------------------- run time
+
+
+@dataclass
+class Runtime:
+    """Where and in what precision a model runs."""
+
+    device: torch.device
+    dtype: torch.dtype                       # torch.bfloat16 or torch.float32: activations, matrices, cache
+    max_tokens_per_step: int = 8192
+
+    @property
+    def is_fp32(self) -> bool:
+        return self.dtype == torch.float32
+
+
+@dataclass
+class CacheView:
+    """What one run of a layer sees of the cache.
+
+    k_pages/v_pages: [num_pages, nkv, page_size, d] of its schedule entry (or of
+    the entry it reads); ``group`` indexes the step's block tables and slots;
+    ``writable`` is False when the pages belong to another entry.  ``state`` is
+    the entry's [num_slots, *shape] tensor when the mixer declared a StateSpec.
+    """
+
+    group: int = -1
+    k_pages: Optional[torch.Tensor] = None
+    v_pages: Optional[torch.Tensor] = None
+    writable: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+@dataclass
+class StepContext:
+    """One step's batch, as the parts see it (all tensors on the device).
+
+    Tokens of one request are consecutive rows.  Requests that bring a single
+    token come first (``num_decode`` of them, rows 0 .. num_decode-1), requests
+    that bring a portion of a prompt after them.
+    """
+
+    num_tokens: int
+    num_seqs: int
+    num_decode: int
+    token_ids: torch.Tensor                 # [N] int32
+    positions: torch.Tensor                 # [N] int32 position of each token in its request
+    token_seq: torch.Tensor                 # [N] int32 index of each token's request in this batch
+    seq_starts: torch.Tensor                # [B+1] int32 first row of each request
+    seq_ctx: torch.Tensor                   # [B] int32 tokens each request had in the cache before this step
+    state_slots: torch.Tensor               # [B] int32 slot of each request's fixed-size state
+    block_tables: List[torch.Tensor]        # per cache group: [B, MB] int32, -1 where no page is held
+    slots: List[torch.Tensor]               # per cache group: [N] int32 page*page_size+offset of each token
+    logit_rows: torch.Tensor                # [R] int32 rows whose logits are wanted
+    # host copies, for choosing kernels and grids without reading the device
+    q_lens: Sequence[int] = ()
+    ctx_lens: Sequence[int] = ()
+    max_q_len: int = 0
+    max_total_len: int = 0                  # largest ctx + q over the batch
+    prefill_tiles: Optional[torch.Tensor] = None   # [n_tiles, 2] int32 (request, first row) for tiled attention
+    num_prefill_tiles: int = 0
+    extras: Dict[str, Any] = field(default_factory=dict)
+
+
+# ------------------------------------------------------------------ interfaces
+
+
+class Part:
+    """Base of all parts.  ``weights`` lists what it wants; ``load`` receives them."""
+
+    category = "part"
+
+    def __init__(self, rt: Runtime, **params: Any):
+        self.rt = rt
+
+    def weights(self) -> Dict[str, WeightSpec]:
+        """Local tensor name (appended to the spec's prefix) -> WeightSpec."""
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take the tensors of ``weights`` (by local name), already on the device."""
+
+
+class Norm(Part):
+    category = "norm"
+
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """h [N, H] fp32 += delta (in place, when given); returns norm(h) in the compute dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    category = "position"
+
+
+class Mixer(Part):
+    category = "mixer"
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView) -> torch.Tensor:
+        """x [N, H] in the compute dtype -> [N, H]; reads and writes its cache view."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    category = "feed_forward"
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    category = "embedding"
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """-> the residual stream h [N, H] in fp32."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    category = "head"
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [R, H] -> logits [R, V] fp32."""
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of a layer's parts around the residual stream.
+
+    ``forward`` takes the fp32 residual stream ``h`` and a ``pending`` delta that
+    has not been added to it yet (so that the add can be fused into the next
+    norm), and returns the next pending delta.
+    """
+
+    category = "block"
+
+    def __init__(self, rt: Runtime, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
+                 feed_forward_norm: Norm, extra: Mapping[str, Part]):
+        self.rt = rt
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+        self.extra = dict(extra)
+
+    def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
+                cache: CacheView) -> torch.Tensor:
+        raise NotImplementedError
+
+
+# -------------------------------------------------------------------- registry
+
+_REGISTRY: Dict[Tuple[str, str], Callable[..., Any]] = {}
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Any], replace: bool = False) -> None:
+    """Make ``kind`` available for specs of ``category`` ('mixer', 'feed_forward',
+    'norm', 'position', 'embedding', 'head', 'block')."""
+    key = (category, kind)
+    if key in _REGISTRY and not replace and _REGISTRY[key] is not factory:
+        raise ValueError(f"{category} kind {kind!r} is registered already")
+    _REGISTRY[key] = factory
+
+
+def part_kinds(category: str) -> List[str]:
+    return sorted(k for (c, k) in _REGISTRY if c == category)
+
+
+def make_part(category: str, spec: PartSpec, rt: Runtime) -> Any:
+    factory = _REGISTRY.get((category, spec.kind))
+    if factory is None:
+        raise KeyError(f"no {category} of kind {spec.kind!r}; registered: {part_kinds(category)}")
+    return factory(rt, **dict(spec.params))
+
+
+def block_factory(kind: str) -> Callable[..., Block]:
+    factory = _REGISTRY.get(("block", kind))
+    if factory is None:
+        raise KeyError(f"no block arrangement {kind!r}; registered: {part_kinds('block')}")
+    return factory

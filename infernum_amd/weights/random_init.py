@@ -1,0 +1,89 @@
+"""Random weights from a configuration and a seed.
+
+Every tensor is drawn from its own generator, seeded from (seed, tensor name),
+so values do not depend on the order in which tensors are made.  Matrices and
+the embedding are N(0, std), norm weights are what the spec says (ones, or a
+uniform range).  ``write_random_model`` writes a model folder (config.json,
+model.safetensors) that loads like any other; ``random_weights_on_device``
+fills a model directly, for runs whose weights are too large to write first.
+The reference has no such mode (its tests download checkpoints).
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+from typing import Any, Dict, Iterator, Optional, Tuple
+
+import torch
+
+from ..parts.base import Runtime, WeightSpec
+
+
+def _tensor_seed(seed: int, name: str) -> int:
+    digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+    return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
+
+
+def draw(spec: WeightSpec, seed: int, name: str, device: torch.device) -> torch.Tensor:
+    """An fp32 tensor of the spec's shape on ``device``."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(_tensor_seed(seed, name))
+    kind = spec.init[0]
+    if kind == "normal":
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
+        return t.normal_(0.0, float(spec.init[1]), generator=gen)
+    if kind == "uniform":
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
+        return t.uniform_(float(spec.init[1]), float(spec.init[2]), generator=gen)
+    if kind == "ones":
+        return torch.ones(spec.shape, dtype=torch.float32, device=device)
+    if kind == "zeros":
+        return torch.zeros(spec.shape, dtype=torch.float32, device=device)
+    raise ValueError(f"unknown init {spec.init!r} for {name}")
+
+
+def _cpu_model(config: Any, dtype: torch.dtype, **spec_kw: Any):
+    from ..config.registry import model_spec_for
+    from ..models.model import DecoderModel
+    spec = model_spec_for(config, **spec_kw)
+    return DecoderModel(spec, Runtime(torch.device("cpu"), dtype))
+
+
+def random_tensors(config: Any, seed: int, dtype: torch.dtype = torch.bfloat16,
+                   **spec_kw: Any) -> Iterator[Tuple[str, torch.Tensor]]:
+    """(name, CPU tensor) for every tensor a file of this model holds; matrices in ``dtype``."""
+    model = _cpu_model(config, dtype, **spec_kw)
+    for name, spec in sorted(model.expected_weights().items()):
+        if not spec.write_when_random:
+            continue
+        t = draw(spec, seed, name, torch.device("cpu"))
+        yield name, t.to(dtype)
+
+
+def write_random_model(config: Any, out_dir: str, seed: int, dtype: torch.dtype = torch.bfloat16,
+                       **spec_kw: Any) -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``; returns out_dir."""
+    from .safetensors_io import write_safetensors
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(config.to_dict(), f, indent=2)
+    write_safetensors(os.path.join(out_dir, "model.safetensors"), random_tensors(config, seed, dtype, **spec_kw))
+    return out_dir
+
+
+def random_weights_on_device(model, seed: int) -> None:
+    """Fill a model with random weights made on its own device (nothing is written)."""
+    rt: Runtime = model.rt
+    expected = model.expected_weights()
+    tensors: Dict[str, torch.Tensor] = {}
+    for name, spec in sorted(expected.items()):
+        if not spec.write_when_random and spec.fallback is not None:
+            continue                              # shares its fallback's buffer, below
+        t = draw(spec, seed, name, rt.device)
+        target = rt.dtype if (spec.follows_compute_dtype or rt.dtype == torch.float32) else torch.float32
+        tensors[name] = t.to(target)
+    for name, spec in expected.items():          # a tied head whose fallback sorts after it
+        if name not in tensors:
+            tensors[name] = tensors[spec.fallback]
+    model.load_weights(tensors)
