@@ -272,3 +272,13 @@ def gemm_skinny_available() -> bool:
     if "skinny" not in _has:
         _has["skinny"] = hasattr(_core(), "ia_gemm_skinny")
     return _has["skinny"]
+
+
+def attention_mfma_available(d: int) -> bool:
+    """Whether the MFMA attention kernels exist for head size d (built on first use)."""
+    import os
+    key = f"attn{d}"
+    if key not in _has:
+        _has[key] = (d in _build.SUPPORTED_HEAD_DIMS
+                     and os.path.isfile(os.path.join(_build.CSRC_DIR, "attention_mfma.hip")))
+    return _has[key]

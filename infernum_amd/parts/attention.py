@@ -46,7 +46,8 @@ class Attention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         if kernels not in ("auto", "generic"):
             raise ValueError("kernels must be 'auto' or 'generic'")
-        self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and self.d % 16 == 0)
+        self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
+                         and K.attention_mfma_available(self.d))
 
     # ---- what it needs ---------------------------------------------------
     def cache_spec(self) -> CacheSpec:

@@ -1,0 +1,146 @@
+"""The engine against the plain implementation on the GPU: whole requests, the tail
+decoded one by one, portions of changing size, and mixed batches with so few pages
+that they are used again; in 32-bit and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+import tiny_models as TM
+import trace_tools as TT
+
+pytestmark = pytest.mark.gpu
+
+# Largest |difference| allowed, as a fraction of the RMS of the plain logits.
+# fp32: sums of a few hundred to a few thousand fp32 products per element, a dozen
+# such stages; measured ratios are 2e-6 to 4e-6, so 2e-5 holds a real fault out.
+# bf16: every stored activation is rounded to 8 bits of mantissa (2^-9 relative);
+# a dozen stages stacked, largest over ~10^5 elements.
+TOL = {"float32": 2e-5, "bfloat16": 6e-2}
+LENGTHS = {"A": (7, 40, 75, 33), "B": (5, 13, 29, 97, 64, 50), "C": (90, 41, 66, 120)}
+MIXED_LENGTHS = {"A": (70, 131, 64, 190, 33, 97, 150, 66, 81, 120), "B": (129, 65, 200, 90, 47, 160, 72, 111, 99, 140),
+                 "C": (90, 180, 66, 120, 75, 143, 35, 101, 170, 88)}
+PAGE = {"A": 4, "B": 8, "C": 16}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name in ("A", "B", "C"):
+        for dt, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+            d = str(tmp_path_factory.mktemp(f"tiny{name}_{dt}"))
+            TM.write_tiny(name, d, dtype=tdt)
+            cfg, w = P.read_model(d)
+            reqs = TT.make_requests(cfg["vocab_size"], LENGTHS[name], seed=11)
+            ref = {r: P.forward(cfg, w, toks) for r, toks in reqs.items()}
+            mreqs = TT.make_requests(cfg["vocab_size"], MIXED_LENGTHS[name], seed=23)
+            mref = {r: P.forward(cfg, w, toks) for r, toks in mreqs.items()}
+            out[(name, dt)] = (d, cfg, reqs, ref)
+            out[(name, dt, "mixed")] = (d, cfg, mreqs, mref)
+    return out
+
+
+def _engine(model_dir, dtype, page_size, num_pages, poison=True):
+    from infernum_amd import CacheConfig, Engine
+    return Engine.from_pretrained(model_dir, dtype=dtype,
+                                  cache_config=CacheConfig(page_size=page_size, num_pages=num_pages,
+                                                           num_state_slots=8, poison_freed_pages=poison))
+
+
+def _check(got, ref, dtype, what):
+    worst, rms, where = TT.error_against(got, ref)
+    print(f"{what}: max|diff| = {worst:.3e}, rms of logits = {rms:.3e}, ratio {worst / rms:.2e} at {where}")
+    assert worst == worst, f"{what}: NaN in the logits at {where}"
+    assert worst <= TOL[dtype] * rms, f"{what}: max|diff| {worst:.3e} > {TOL[dtype]} * rms {rms:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(models, name, dtype):
+    d, cfg, reqs, ref = models[(name, dtype)]
+    eng = _engine(d, dtype, PAGE[name], 64)
+    got = TT.run_steps(eng, TT.trace_whole(reqs))
+    assert len(got) == sum(len(t) for t in reqs.values())
+    _check(got, ref, dtype, f"{name} {dtype} whole")
+    eng.cache.check()
+    assert eng.cache.free_pages(0) == 64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_tail_one_by_one(models, name, dtype):
+    d, cfg, reqs, ref = models[(name, dtype)]
+    eng = _engine(d, dtype, PAGE[name], 64)
+    got = TT.run_steps(eng, TT.trace_tail_one_by_one(reqs, 32))
+    _check(got, ref, dtype, f"{name} {dtype} tail one by one")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions(models, name, dtype):
+    d, cfg, reqs, ref = models[(name, dtype)]
+    eng = _engine(d, dtype, PAGE[name], 64)
+    got = TT.run_steps(eng, TT.trace_portions(reqs))
+    _check(got, ref, dtype, f"{name} {dtype} portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_with_page_reuse(models, name, dtype):
+    d, cfg, reqs, ref = models[(name, dtype, "mixed")]
+    prompt_len = {r: max(2, len(t) - 20) for r, t in reqs.items()}
+    steps, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=5)
+    ps = PAGE[name]
+    num_pages = max_tokens // ps
+    total_pages = sum(-(-len(t) // ps) for t in reqs.values())
+    assert total_pages > num_pages, "the pool must be too small to hold all requests without reuse"
+    eng = _engine(d, dtype, ps, num_pages)
+    got = TT.run_steps(eng, steps)
+    _check(got, ref, dtype, f"{name} {dtype} mixed")
+    eng.cache.check()
+    assert eng.cache.free_pages(0) == num_pages
+
+
+def test_cutting_does_not_change_fp32_logits(models):
+    """In the 32-bit path a position's logits are the same bits however the tokens
+    are cut into steps: each output is one chain of operations in a fixed order."""
+    d, cfg, reqs, ref = models[("B", "float32")]
+    a = TT.run_steps(_engine(d, "float32", 8, 64), TT.trace_whole(reqs))
+    b = TT.run_steps(_engine(d, "float32", 8, 64), TT.trace_portions(reqs))
+    c = TT.run_steps(_engine(d, "float32", 4, 128), TT.trace_tail_one_by_one(reqs))
+    for k in a:
+        assert torch.equal(a[k], b[k]), k
+        assert torch.equal(a[k], c[k]), k
+
+
+def test_trace_run_program(models, tmp_path):
+    """bin/trace_run as a user starts it: steps on standard input, files out."""
+    d, cfg, reqs, ref = models[("A", "float32")]
+    prompt_len = {r: max(2, len(t) - 10) for r, t in reqs.items()}
+    steps, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=9)
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", str(max_tokens)],
+                          input="".join(json.dumps(s) + "\n" for s in steps), text=True, capture_output=True,
+                          timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    V = cfg["vocab_size"]
+    pos, got = {}, {}
+    for s in steps:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        arr = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(n_want, V)
+        row = 0
+        for e in s["entries"]:
+            base = pos.get(e["id"], 0)
+            for w in e["want"]:
+                got[(e["id"], base + w)] = torch.from_numpy(arr[row].copy())
+                row += 1
+            pos[e["id"]] = base + len(e["tokens"])
+    _check(got, ref, "float32", "trace_run A float32 mixed")
