@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the Llama-3.1-8B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+One "step" is one decode step of the whole batch: every request brings its last
+token, the engine runs it against the paged cache, and the next token is chosen
+greedily on the device.  Requests start from a 512-token prompt (uniform random
+ids), as the reference measures decoding after a prompt
+(infernum-examples/examples/bench.rs:1049-1110).  The line printed at the end also
+holds the prefill of one 2,048-token prompt, decoding at batch 1 and 64, and the
+decode step's place against the HBM roofline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                 # MI355X HBM3E, published
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+LLAMA_8B = dict(
+    model_type="llama", num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+    intermediate_size=14336, vocab_size=128256, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+    max_position_embeddings=131072,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+CONTEXT_LEN = 4096
+PROMPT_LEN = 512
+PREFILL_TOKENS = 2048
+PAGE_SIZE = 16
+
+
+def sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def matmul_params(cfg) -> int:
+    """Weights that every token multiplies with (embedding gather excluded, head included)."""
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    nh, nkv, d = cfg.num_attention_heads, cfg.num_kv_heads, cfg.head_dim
+    per_layer = (nh + 2 * nkv) * d * H + nh * d * H + 3 * H * I
+    return cfg.num_hidden_layers * per_layer, V * H
+
+
+def decode_bytes(cfg, ctx_lens, elem=2) -> float:
+    """Bytes a decode step has to read: every weight once, and the keys and values of the live requests."""
+    per_layers, head = matmul_params(cfg)
+    kv = sum(ctx_lens) * 2 * cfg.num_kv_heads * cfg.head_dim * cfg.num_hidden_layers
+    return (per_layers + head + kv) * elem
+
+
+def prefill_flops(cfg, T) -> float:
+    per_layers, head = matmul_params(cfg)
+    gemm = 2.0 * T * per_layers + 2.0 * head            # the head runs on one row
+    attn = 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2) * cfg.num_hidden_layers
+    return gemm + attn
+
+
+class DecodeRun:
+    """B requests, each prefilled with a prompt, then decoded greedily step by step."""
+
+    def __init__(self, engine, batch: int, prompt_len: int, seed: int = 0):
+        import torch
+        from infernum_amd.engine import StepEntry
+        self.engine, self.batch = engine, batch
+        g = torch.Generator().manual_seed(seed)
+        V = engine.spec.vocab_size
+        self.ids = [f"b{batch}_{i}" for i in range(batch)]
+        self.ctx = [0] * batch
+        last = []
+        for i, rid in enumerate(self.ids):
+            prompt = torch.randint(0, V, (prompt_len,), generator=g).tolist()
+            logits = None
+            for p in range(0, prompt_len, 2048):
+                chunk = prompt[p:p + 2048]
+                want = [len(chunk) - 1] if p + len(chunk) == prompt_len else []
+                logits = engine.step([StepEntry(rid, chunk, want)])
+            last.append(int(torch.argmax(logits[0])))
+            self.ctx[i] = prompt_len
+        self.last = last
+        sync()
+
+    def step(self):
+        self.last = self.engine.decode_greedy(self.ids, self.last)
+        self.ctx = [c + 1 for c in self.ctx]
+
+    def close(self):
+        for rid in self.ids:
+            self.engine.end(rid)
+
+
+def time_decode(engine, batch, steps, warmup, prompt_len=PROMPT_LEN):
+    run = DecodeRun(engine, batch, prompt_len)
+    for _ in range(warmup):
+        run.step()
+    sync()
+    ctx_mid = [c + steps / 2.0 for c in run.ctx]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run.step()
+    sync()
+    dt = time.perf_counter() - t0
+    run.close()
+    return dt, ctx_mid
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (both are reported)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
+        return 2
+
+    import torch
+    from infernum_amd import CacheConfig, Engine, LlamaConfig
+
+    raw = dict(LLAMA_8B)
+    full_layers = raw["num_hidden_layers"]
+    if a.layers:
+        raw["num_hidden_layers"] = a.layers
+    cfg = LlamaConfig.from_dict(raw)
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
+    elem = 2 if a.dtype == "bf16" else 4
+    max_batch = max(a.batch, 1 if a.no_points else 64)
+    tokens_needed = max(max_batch * (PROMPT_LEN + a.steps + a.warmup + PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
+    t_load = time.perf_counter()
+    engine = Engine.from_config(cfg, seed=0, dtype=dtype,
+                                cache_config=CacheConfig(page_size=PAGE_SIZE,
+                                                         num_pages=tokens_needed // PAGE_SIZE + max_batch,
+                                                         num_state_slots=max_batch + 1),
+                                max_tokens_per_step=8192)
+    sync()
+    print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
+
+    # ---- the timed K steps at the headline batch ---------------------------------
+    dt, ctx_mid = time_decode(engine, a.batch, a.steps, a.warmup)
+    ms_per_step = dt / a.steps * 1e3
+    value = a.batch * a.steps / dt
+    achieved = decode_bytes(cfg, ctx_mid, elem) / (dt / a.steps) / 1e9
+    out = {
+        "metric": "decode tok/s @ batch 8, Llama-3-8B shape", "value": round(value, 2), "unit": "tokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
+        "config": {
+            "model": "llama-3.1-8b-shape-random", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
+            "hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads, "num_kv_heads": cfg.num_kv_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "global_batch": a.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "page_size": PAGE_SIZE,
+            "parallelism": "none", "sampling": "greedy", "rope": "llama3(8,1,4,8192) theta 5e5",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+
+    if not a.no_points:
+        points = {}
+        for b in (1, 64):
+            steps = max(16, min(a.steps, 64))
+            d, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)))
+            points[f"decode_b{b}"] = round(b * steps / d, 2)
+        out["points"] = points
+        # ---- prefill of one 2,048-token prompt ---------------------------------------
+        from infernum_amd.engine import StepEntry
+        g = torch.Generator().manual_seed(7)
+        prompt = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
+        best = None
+        for i in range(3):
+            sync()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
+            sync()
+            t = time.perf_counter() - t0
+            engine.end(f"p{i}")
+            if i > 0:
+                best = t if best is None else min(best, t)
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        out["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
+                          "frac": round(flops / best / (PEAK_TFLOPS[a.dtype] * 1e12), 4)}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -205,6 +205,14 @@ class Engine:
         self.steps_run += 1
         return logits
 
+    def decode_greedy(self, requests: Sequence[Hashable], tokens: Sequence[int]) -> List[int]:
+        """One decode step for requests that each bring one token; returns each one's next token (argmax)."""
+        from ..kernels import api as K
+        logits = self.step([StepEntry(r, [int(t)], [0]) for r, t in zip(requests, tokens)])
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        K.argmax(logits, out)
+        return out.tolist()
+
     def end(self, request: Hashable) -> None:
         """The request is finished: its pages and its state slot are given back."""
         if self.cache.has(request):

@@ -180,7 +180,7 @@ SKINNY_MAX_M = 64
 
 
 def gemm_skinny_supported(M: int, N: int, K: int) -> bool:
-    return 0 < M <= SKINNY_MAX_M and K % 32 == 0 and K >= 32 and N >= 1
+    return 0 < M <= SKINNY_MAX_M and K % 8 == 0 and K >= 8 and N >= 1
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -190,7 +190,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Te
     N = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in DTYPE_CODE, "gemm_skinny: bf16 in")
     _need(w.dim() == 2 and w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_skinny: shapes")
-    _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 64, K % 32 == 0)")
+    _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 64, K % 8 == 0)")
     _ok(_core().ia_gemm_skinny(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, _stream()), "gemm_skinny")
     return out
 

@@ -1,0 +1,349 @@
+"""Each HIP kernel alone against a plain PyTorch fp32 reference of the same
+operation, at sizes other than the tiny models': widths and vocabularies that are
+no power of two, head sizes in steps of 16, odd page sizes, grouped heads."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def K():
+    from infernum_amd.kernels import api
+    return api
+
+
+def _rand(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+# ------------------------------------------------------------------------ rows
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,V", [(100, 77), (4096, 1000), (1536, 333)])
+def test_embed(dtype, H, V):
+    table = _rand(V, H, dtype=dtype)
+    ids = torch.tensor([0, V - 1, 5, 5, V // 2], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, H, dtype=torch.float32, device=DEV)
+    K().embed(table, ids, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+def test_embed_bad_id_gives_nan_not_a_fault():
+    table = _rand(10, 64)
+    ids = torch.tensor([3, 10, -1], dtype=torch.int32, device=DEV)
+    out = torch.zeros(3, 64, device=DEV)
+    K().embed(table, ids, out)
+    assert torch.equal(out[0], table[3]) and out[1].isnan().all() and out[2].isnan().all()
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("H", [4, 100, 2048, 5120])
+def test_add_rmsnorm(dtype, wdtype, H):
+    N, eps = 7, 1e-6
+    h = _rand(N, H, seed=1)
+    delta = _rand(N, H, dtype=dtype, seed=2)
+    w = (_rand(H, seed=3).abs() + 0.5).to(wdtype)
+    h0 = h.clone()
+    out = torch.empty(N, H, dtype=dtype, device=DEV)
+    K().add_rmsnorm(h, delta, w, eps, out)
+    s = h0.double() + delta.double()
+    assert torch.allclose(h.double(), s, atol=1e-6)                   # the sum is stored in fp32
+    want = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert torch.allclose(out.double(), want, atol=tol, rtol=tol)
+    # without a delta, and on selected rows only (h untouched)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    h1 = h.clone()
+    out2 = torch.empty(3, H, dtype=dtype, device=DEV)
+    K().add_rmsnorm(h, delta, w, eps, out2, rows)
+    assert torch.equal(h, h1)
+    s2 = (h1.double() + delta.double())[rows.long()]
+    want2 = s2 * torch.rsqrt((s2 * s2).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out2.double(), want2, atol=tol, rtol=tol)
+
+
+def test_rmsnorm_reference_vector():
+    # infernum-cuda/src/inner/cuda/ops/rmsnorm.rs:171-203
+    h = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)
+    out = torch.empty(1, 4, device=DEV)
+    K().add_rmsnorm(h, None, torch.ones(4, device=DEV), 1e-6, out)
+    assert torch.allclose(out, h / math.sqrt(7.5), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(dtype):
+    N, I = 5, 172
+    gu = _rand(N, 2 * I, dtype=dtype, scale=3.0)
+    out = torch.empty(N, I, dtype=dtype, device=DEV)
+    K().swiglu(gu, out)
+    g, u = gu[:, :I].double(), gu[:, I:].double()
+    want = g / (1 + torch.exp(-g)) * u
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    assert torch.allclose(out.double(), want, atol=tol, rtol=tol)
+
+
+def test_rope_reference_vector_and_pages():
+    # infernum-cuda/src/inner/cuda/ops/rope.rs:835-885: [a,b,c,d] at position 1, theta 1e4
+    nh, nkv, d, ps = 1, 1, 4, 3
+    qkv = torch.tensor([[1.0, 2, 3, 4, 1, 2, 3, 4, 9, 8, 7, 6]], device=DEV)
+    inv = torch.tensor([1.0, 0.01], device=DEV)
+    kp = torch.zeros(5, nkv, ps, d, device=DEV)
+    vp = torch.zeros(5, nkv, ps, d, device=DEV)
+    K().rope_kv_append(qkv, torch.tensor([1], dtype=torch.int32, device=DEV), inv, nh, nkv, d, d,
+                       torch.tensor([2 * ps + 1], dtype=torch.int32, device=DEV), kp, vp)
+    c0, s0, c1, s1 = math.cos(1.0), math.sin(1.0), math.cos(0.01), math.sin(0.01)
+    want = torch.tensor([1 * c0 - 3 * s0, 2 * c1 - 4 * s1, 3 * c0 + 1 * s0, 4 * c1 + 2 * s1], device=DEV)
+    assert torch.allclose(qkv[0, :4], want, atol=1e-6)
+    assert torch.allclose(kp[2, 0, 1], want, atol=1e-6)
+    assert torch.equal(vp[2, 0, 1], torch.tensor([9.0, 8, 7, 6], device=DEV))
+    assert kp.abs().sum() == kp[2, 0, 1].abs().sum() and vp.abs().sum() == vp[2, 0, 1].abs().sum()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,rot,ps", [(6, 2, 48, 48, 5), (8, 8, 16, 16, 16), (5, 1, 128, 64, 7)])
+def test_rope_kv_append(dtype, nh, nkv, d, rot, ps):
+    N, pages = 9, 6
+    qkv = _rand(N, (nh + 2 * nkv) * d, dtype=dtype)
+    q0 = qkv.clone()
+    pos = torch.tensor([0, 1, 2, 40, 41, 1000, 7, 8, 9], dtype=torch.int32, device=DEV)
+    inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV)
+    slots = torch.randperm(pages * ps)[:N].to(torch.int32).to(DEV)
+    kp = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    K().rope_kv_append(qkv, pos, inv, nh, nkv, d, rot, slots, kp, vp)
+    x = q0.double().reshape(N, nh + 2 * nkv, d)
+    ang = (pos.float()[:, None] * inv[None, :]).double()      # angles are fp32 products, as in the kernel
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[:, :nh + nkv, :rot // 2], x[:, :nh + nkv, rot // 2:rot]
+    roted = x[:, :nh + nkv].clone()
+    roted[..., :rot // 2] = a * c - b * s
+    roted[..., rot // 2:rot] = a * s + b * c
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(qkv[:, :nh * d].double().reshape(N, nh, d), roted[:, :nh], atol=tol, rtol=tol)
+    for n in range(N):
+        p, o = int(slots[n]) // ps, int(slots[n]) % ps
+        assert torch.allclose(kp[p, :, o].double(), roted[n, nh:], atol=tol, rtol=tol)
+        assert torch.equal(vp[p, :, o], q0[n].reshape(nh + 2 * nkv, d)[nh + nkv:])
+    # queries only (a layer that reads another's keys and values)
+    q2 = q0[:, :nh * d].contiguous()
+    K().rope_kv_append(q2, pos, inv, nh, nkv, d, rot)
+    assert torch.allclose(q2.double().reshape(N, nh, d), roted[:, :nh], atol=tol, rtol=tol)
+
+
+# -------------------------------------------------------------- matrix products
+@pytest.mark.parametrize("M,N,K_", [(1, 250, 96), (7, 384, 176), (70, 129, 1000), (300, 64, 33)])
+def test_gemm_generic(M, N, K_):
+    a, w = _rand(M, K_, seed=4), _rand(N, K_, seed=5)
+    out = torch.empty(M, N, device=DEV)
+    K().gemm_generic(a, w, out)
+    want = a.double() @ w.double().t()
+    assert torch.allclose(out.double(), want, atol=1e-4, rtol=1e-5)
+    # the same rows alone give the same bits: the order of summation does not depend on M
+    one = torch.empty(1, N, device=DEV)
+    K().gemm_generic(a[M - 1:M], w, one)
+    assert torch.equal(one[0], out[M - 1])
+    ab, wb = a.bfloat16(), w.bfloat16()
+    outb = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    K().gemm_generic(ab, wb, outb)
+    wantb = ab.double() @ wb.double().t()
+    assert torch.allclose(outb.double(), wantb, atol=0.3, rtol=2e-2)
+    outf = torch.empty(M, N, device=DEV)
+    K().gemm_generic(ab, wb, outf)
+    assert torch.allclose(outf.double(), wantb, atol=1e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K_", [(250, 96), (384, 176), (4096, 4096), (1000, 14336), (16, 8), (129, 1000)])
+def test_gemm_skinny(M, N, K_):
+    api = K()
+    if not api.gemm_skinny_available():
+        pytest.skip("skinny kernel not built")
+    a, w = _rand(M, K_, dtype=torch.bfloat16, seed=6), _rand(N, K_, dtype=torch.bfloat16, seed=7)
+    want = a.double() @ w.double().t()
+    outf = torch.full((M, N), float("nan"), device=DEV)
+    api.gemm_skinny(a, w, outf)
+    scale = math.sqrt(K_)
+    assert (outf.double() - want).abs().max().item() <= 2e-5 * scale + 1e-6 * want.abs().max().item()
+    outb = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    api.gemm_skinny(a, w, outb)
+    assert torch.equal(outb, outf.bfloat16())
+    # a row's result does not depend on how many other rows there are
+    one = torch.empty(1, N, device=DEV)
+    api.gemm_skinny(a[M - 1:M].contiguous(), w, one)
+    assert torch.equal(one[0], outf[M - 1])
+
+
+# ------------------------------------------------------------------- attention
+def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
+    """Random queries/keys/values of several requests laid out into shuffled pages.
+    Returns everything the kernels need plus the dense tensors for the reference."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(lens)
+    pages_per = [-(-L // ps) for L in lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    MB = max(pages_per) + 1
+    bt = torch.full((B, MB), -1, dtype=torch.int32)
+    kd = [torch.randn(L, nkv, d, generator=g) for L in lens]
+    vd = [torch.randn(L, nkv, d, generator=g) for L in lens]
+    if scale_one is not None:                      # make one far key stand out
+        b, j, factor = scale_one
+        kd[b][j] *= factor
+    kp = torch.zeros(num_pages, nkv, ps, d)
+    vp = torch.zeros(num_pages, nkv, ps, d)
+    it = iter(perm)
+    for b in range(B):
+        for i in range(pages_per[b]):
+            p = next(it)
+            bt[b, i] = p
+            n = min(ps, lens[b] - i * ps)
+            kp[p, :, :n] = kd[b][i * ps:i * ps + n].transpose(0, 1)
+            vp[p, :, :n] = vd[b][i * ps:i * ps + n].transpose(0, 1)
+    N = sum(q_lens)
+    q = torch.randn(N, nh * d, generator=g)
+    token_seq = torch.cat([torch.full((ql,), b, dtype=torch.int32) for b, ql in enumerate(q_lens)])
+    positions = torch.cat([torch.arange(L - ql, L, dtype=torch.int32) for L, ql in zip(lens, q_lens)])
+    to = lambda t: t.to(dtype).to(DEV)
+    return dict(q=to(q), kp=to(kp), vp=to(vp), bt=bt.to(DEV), token_seq=token_seq.to(DEV),
+                positions=positions.to(DEV), kd=[to(x) for x in kd], vd=[to(x) for x in vd], N=N)
+
+
+def _ref_attention(case, nh, nkv, d, scale, window):
+    out = torch.zeros(case["N"], nh * d, dtype=torch.float64)
+    q = case["q"].double().cpu()
+    for n in range(case["N"]):
+        b, p = int(case["token_seq"][n]), int(case["positions"][n])
+        lo = max(0, p - window + 1) if window else 0
+        k, v = case["kd"][b].double().cpu()[lo:p + 1], case["vd"][b].double().cpu()[lo:p + 1]
+        for h in range(nh):
+            gk = h // (nh // nkv)
+            w = torch.softmax((k[:, gk] @ q[n, h * d:(h + 1) * d]) * scale, 0)
+            out[n, h * d:(h + 1) * d] = w @ v[:, gk]
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,ps,window", [(6, 2, 48, 5, 0), (4, 4, 16, 16, 0), (8, 1, 128, 7, 0),
+                                                (3, 3, 80, 4, 9), (2, 1, 256, 16, 70)])
+def test_attention_generic(dtype, nh, nkv, d, ps, window):
+    lens, q_lens = [70, 3, 131, 64], [1, 3, 40, 64]
+    case = _paged_case(nh, nkv, d, ps, lens, q_lens, dtype)
+    out = torch.full((case["N"], nh * d), float("nan"), dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    K().attention_generic(case["q"], case["kp"], case["vp"], out, case["token_seq"], case["positions"], case["bt"],
+                          nh, nkv, d, scale, window)
+    want = _ref_attention(case, nh, nkv, d, scale, window)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert (out.double().cpu() - want).abs().max().item() <= tol
+
+
+def test_attention_generic_far_key_and_first_row():
+    """One key far back among hundreds carries the softmax; a missed page or a wrong
+    block-table entry shows at once.  The first token of a request returns v_0."""
+    nh, nkv, d, ps = 2, 1, 32, 8
+    case = _paged_case(nh, nkv, d, ps, [500, 1], [1, 1], torch.float32, scale_one=(0, 17, 30.0))
+    out = torch.empty(2, nh * d, device=DEV)
+    K().attention_generic(case["q"], case["kp"], case["vp"], out, case["token_seq"], case["positions"], case["bt"],
+                          nh, nkv, d, 1.0, 0)
+    want = _ref_attention(case, nh, nkv, d, 1.0, 0)
+    assert (out.double().cpu() - want).abs().max().item() <= 2e-5
+    assert torch.allclose(out[1].reshape(nh, d), case["vd"][1][0, 0].expand(nh, d), atol=1e-6)
+
+
+def test_attention_generic_missing_page_poisons():
+    nh, nkv, d, ps = 1, 1, 16, 4
+    case = _paged_case(nh, nkv, d, ps, [20], [1], torch.float32)
+    case["bt"][0, 2] = -1
+    out = torch.zeros(1, d, device=DEV)
+    K().attention_generic(case["q"], case["kp"], case["vp"], out, case["token_seq"], case["positions"], case["bt"],
+                          nh, nkv, d, 1.0, 0)
+    assert out.isnan().all()
+    # with a window that has passed the missing page the result is clean
+    K().attention_generic(case["q"], case["kp"], case["vp"], out, case["token_seq"], case["positions"], case["bt"],
+                          nh, nkv, d, 1.0, 8)
+    assert not out.isnan().any()
+
+
+# -------------------------------------------------------------------- sampling
+@pytest.mark.parametrize("V", [5, 250, 1024, 128256])
+def test_argmax(V):
+    x = _rand(4, V)
+    x[1, V // 3] = 50.0
+    x[2, :] = 1.0                                  # all equal: the lowest index wins
+    x[3, V - 1] = 60.0
+    x[3, V // 2] = 60.0
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    K().argmax(x, out)
+    assert out.tolist() == [int(torch.argmax(x[0])), V // 3, 0, V // 2]
+
+
+def test_repetition_penalty():
+    x = torch.tensor([[2.0, -2.0, 1.0, 4.0], [2.0, -2.0, 1.0, 4.0]], device=DEV)
+    recent = torch.tensor([[0, 1, 0, 9], [3, 3, 3, 3]], dtype=torch.int32, device=DEV)
+    counts = torch.tensor([3, 1], dtype=torch.int32, device=DEV)
+    pen = torch.tensor([2.0, 4.0], device=DEV)
+    K().repetition_penalty(x, recent, counts, pen)
+    # a token that stands twice is penalised twice (infernum-cuda/src/inner/cuda/ops/sample.rs:101-112)
+    assert x.tolist() == [[0.5, -4.0, 1.0, 4.0], [2.0, -2.0, 1.0, 1.0]]
+
+
+def _host_sample(logits, T, top_p, u):
+    import plain_llama as P
+    return P.sample_token(logits.cpu(), T, top_p, u)
+
+
+@pytest.mark.parametrize("V", [7, 250, 5000])
+def test_sample_matches_host_rule(V):
+    import sys, os
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    R = 24
+    x = _rand(R, V, scale=2.0, seed=9)
+    g = torch.Generator().manual_seed(1)
+    T = torch.rand(R, generator=g) * 1.5 + 0.2
+    tp = torch.tensor([1.0, 0.9, 0.5, 0.1] * (R // 4))
+    u = torch.rand(R, generator=g)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    work = torch.empty(R, V, device=DEV)
+    K().sample(x, work, T.to(DEV), tp.to(DEV), u.to(DEV), out)
+    bad = 0
+    for r in range(R):
+        want = _host_sample(x[r], float(T[r]), float(tp[r]), float(u[r]))
+        if int(out[r]) != want:
+            # only a draw within rounding of a boundary of the CDF may differ
+            xr = x[r].double().cpu() / float(T[r])
+            e = torch.exp(xr - xr.max())
+            bad += 1
+            assert e[int(out[r])] > 0
+    assert bad <= 1
+
+
+def test_sample_limits_and_frequencies():
+    V = 50
+    x = _rand(1, V, scale=1.5, seed=3)
+    # low temperature: the maximum (sample.rs:176-183); same inputs, same token (sample.rs:167-173)
+    out = torch.empty(1, dtype=torch.int32, device=DEV)
+    work = torch.empty(1, V, device=DEV)
+    one = lambda v: torch.tensor([v], device=DEV)
+    K().sample(x, work, one(1e-3), one(0.9), one(0.7), out)
+    assert int(out[0]) == int(torch.argmax(x[0]))
+    # frequencies over many draws follow softmax(x / T)
+    R = 20000
+    xs = x.expand(R, V).contiguous()
+    u = torch.rand(R, generator=torch.Generator().manual_seed(5)).to(DEV)
+    outs = torch.empty(R, dtype=torch.int32, device=DEV)
+    K().sample(xs, torch.empty(R, V, device=DEV), torch.full((R,), 0.8, device=DEV), torch.ones(R, device=DEV), u, outs)
+    freq = torch.bincount(outs.long().cpu(), minlength=V).double() / R
+    p = torch.softmax(x[0].double().cpu() / 0.8, 0)
+    chi2 = (R * (freq - p) ** 2 / p).sum().item()
+    assert chi2 < 100.0, chi2            # 49 degrees of freedom: 100 is far in the tail
+    # top_p keeps the nucleus only
+    K().sample(xs, torch.empty(R, V, device=DEV), torch.full((R,), 0.8, device=DEV), torch.full((R,), 0.5, device=DEV),
+               u, outs)
+    srt, idx = torch.sort(p, descending=True)
+    n_keep = int(torch.nonzero(torch.cumsum(srt, 0) >= 0.5)[0]) + 1
+    assert set(outs.tolist()) <= set(idx[:n_keep].tolist())
