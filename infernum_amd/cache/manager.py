@@ -151,9 +151,11 @@ class CacheManager:
         if device is not None:
             for i, (cs, ss) in enumerate(needs):
                 if cs is not None:
-                    shape = (config.num_pages, cs.num_kv_heads, self.page_size, cs.head_dim)
-                    self.k_pages[i] = torch.zeros(shape, dtype=dtype, device=device)
-                    self.v_pages[i] = torch.zeros(shape, dtype=dtype, device=device)
+                    # values are kept transposed within a page: what the PV product of the matrix cores reads
+                    self.k_pages[i] = torch.zeros((config.num_pages, cs.num_kv_heads, self.page_size, cs.head_dim),
+                                                  dtype=dtype, device=device)
+                    self.v_pages[i] = torch.zeros((config.num_pages, cs.num_kv_heads, cs.head_dim, self.page_size),
+                                                  dtype=dtype, device=device)
                 if ss is not None:
                     self.state[i] = torch.zeros((config.num_state_slots,) + tuple(ss.shape), dtype=ss.dtype,
                                                 device=device)

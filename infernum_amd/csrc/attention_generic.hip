@@ -5,8 +5,8 @@
 // window.  Keys are summed in the order of their positions, 64 at a time, so the
 // result at a position does not depend on what else the batch holds.
 //
-// Pages are [num_pages, nkv, page_size, d]; block_tables[s, j / page_size] is the
-// page of key j of sequence s.  The query of token n stands at positions[n] and
+// Key pages are [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d,
+// page_size]; block_tables[s, j / page_size] is the page of key j of sequence s.  The query of token n stands at positions[n] and
 // sees keys max(0, pos - window + 1) .. pos  (window <= 0: all keys from 0).
 #include "common.h"
 
@@ -68,12 +68,15 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const T* __restrict__ 
     __syncthreads();
     const int cnt = (j_hi - j0 + 1) < 64 ? (j_hi - j0 + 1) : 64;
     for (int jj = 0; jj < cnt; ++jj) {
-      const T* vr = v_pages + (size_t)rs[jj] * d;
+      // rs = (page * nkv + g) * page_size + offset  ->  value (dim) at ((page*nkv+g) * d + dim) * page_size + offset
+      const int r = rs[jj];
+      const int head_page = r / page_size, off = r - head_page * page_size;
+      const T* vr = v_pages + (size_t)head_page * d * page_size + off;
       const float pj = ps[jj];
 #pragma unroll
       for (int c = 0; c < AG_MAX_D / 64; ++c) {
         const int dim = lane + 64 * c;
-        if (dim < d) acc[c] = fmaf(pj, to_float(vr[dim]), acc[c]);
+        if (dim < d) acc[c] = fmaf(pj, to_float(vr[(size_t)dim * page_size]), acc[c]);
       }
     }
     __syncthreads();

@@ -1,0 +1,336 @@
+// bf16 attention over the paged cache on the matrix cores (v_mfma_f32_16x16x16_bf16),
+// compiled for one head size, IA_HEAD_DIM (a multiple of 16, at most 256).
+//
+// Both kernels work on the transposed problem, one wave per workgroup and no LDS:
+//   S^T[key, col] = K[key, :] . Q[col, :]      A operand = 16 keys of K, B operand = 16 columns of Q
+//   O^T[dim, col] += V^T[dim, key] P^T[key, col]
+// A column is one (token, query head).  The accumulator of S^T leaves lane l with
+// the keys 4*(l/16) .. +3 of column l%16, which is exactly what the B operand of
+// the second product wants, so the probabilities go from registers to registers;
+// and value pages are stored transposed, [num_pages, nkv, d, page_size], so that
+// its A operand is 8 contiguous bytes.  The statistics of a column (maximum, sum)
+// are fp32 and live in the lanes l%16 == column; scores are scaled by
+// scale * log2(e) and exponentiated with exp2.
+//
+// Decoding: the 16 columns are up to 16 query heads of ONE key/value head for one
+// token, so a page is read once for its whole group of heads; the keys of a
+// request are split over blockIdx.z, each part leaves (max, sum, unnormalised
+// output) and a second kernel joins the parts in a fixed order.
+// Prefill: a wave takes CT column tiles that share their keys: GH heads of one
+// key/value head times CT/GH blocks of 16 consecutive tokens; K and V^T registers
+// are loaded once per 16 keys and used for all CT tiles.
+//
+// Key pages are [num_pages, nkv, page_size, d]; page_size must be a multiple of 4.
+// Keys outside [first key any column may see, last key of the request] are
+// zeroed (values) or masked (scores): a stale or poisoned page never leaks in.
+// A key that is needed but has no page in the block table gives NaN, not a fault.
+#include "common.h"
+
+#ifndef IA_HEAD_DIM
+#error "compile with -DIA_HEAD_DIM=<head size>"
+#endif
+#define HD IA_HEAD_DIM
+#define NS (HD / 16)
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
+#define PREFILL_CT (HD <= 128 ? 4 : 2)
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ s16x4 as_s16x4(uint32_t a, uint32_t b) {
+  uint2 u = make_uint2(a, b);
+  return __builtin_bit_cast(s16x4, u);
+}
+
+// The 16 k-steps' worth of one row (a key of K or a column of Q) for lane group qd.
+// Step s of lane group qd covers the dims  (s/2)*32 + qd*8 + (s%2)*4 .. +3  (16-byte loads,
+// 64 contiguous bytes per row and instruction); an odd last step covers (HD/32)*32 + qd*4 .. +3.
+// K and Q use the same map, and a dot product does not care about the order of its terms.
+__device__ __forceinline__ void load_row_operand(const uint16_t* __restrict__ row, int qd, s16x4 (&reg)[NS]) {
+#pragma unroll
+  for (int t = 0; t < HD / 32; ++t) {
+    const uint4 v = *reinterpret_cast<const uint4*>(row + t * 32 + qd * 8);
+    reg[2 * t] = as_s16x4(v.x, v.y);
+    reg[2 * t + 1] = as_s16x4(v.z, v.w);
+  }
+  if (HD % 32) {
+    const uint2 v = *reinterpret_cast<const uint2*>(row + (HD / 32) * 32 + qd * 4);
+    reg[NS - 1] = as_s16x4(v.x, v.y);
+  }
+}
+
+__device__ __forceinline__ void zero_row_operand(s16x4 (&reg)[NS]) {
+#pragma unroll
+  for (int s = 0; s < NS; ++s) reg[s] = (s16x4){0, 0, 0, 0};
+}
+
+__device__ __forceinline__ float bf16_round(float x) { return bf16_bits_to_float(float_to_bf16_bits(x)); }
+
+// One tile of 16 keys, t0 .. t0+15, for CT column tiles.
+//   pos[c], lo[c]: this lane's column (lane % 16) of tile c sees keys lo .. pos; pos < 0: no such column
+//   key_lo, key_hi: keys outside are not data of this request (wave-uniform)
+template <int CT>
+__device__ __forceinline__ void attn_tile(int t0, int key_lo, int key_hi, const int* __restrict__ bt, int ps,
+                                          int num_pages, int nkv, int g, const uint16_t* __restrict__ k_pages,
+                                          const uint16_t* __restrict__ v_pages, const s16x4 (&q)[CT][NS],
+                                          const int (&pos)[CT], const int (&lo)[CT], float scale_log2,
+                                          f32x4 (&o)[CT][NS], float (&m)[CT], float (&l)[CT], int lane) {
+  const int j = lane & 15, qd = lane >> 4;
+  // ---- S^T = K Q^T
+  const int key = t0 + j;
+  const int keyc = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
+  const int page = bt[keyc / ps];
+  const bool page_ok = (unsigned)page < (unsigned)num_pages;
+  const bool needed = key >= key_lo && key <= key_hi;
+  const uint16_t* krow = k_pages + (((size_t)(page_ok ? page : 0) * nkv + g) * ps + (keyc % ps)) * HD;
+  s16x4 kreg[NS];
+  load_row_operand(krow, qd, kreg);
+  const bool poison = __any(needed && !page_ok);
+  f32x4 s[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    s[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; ++st) s[c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[st], q[c][st], s[c], 0, 0, 0);
+  }
+  // ---- softmax statistics of each column; probabilities as the B operand of the next product
+  const int kg = t0 + 4 * qd;   // this lane holds the keys kg .. kg+3 of its column
+  s16x4 pb[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    float sv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int kr = kg + r;
+      const bool ok = pos[c] >= 0 && kr <= pos[c] && kr >= lo[c];
+      sv[r] = ok ? s[c][r] * scale_log2 : -INFINITY;
+    }
+    float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, IA_WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE));
+    const float m_new = fmaxf(m[c], tmax);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    float p[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) p[r] = bf16_round(exp2f(sv[r] - m_safe));
+    const float corr = exp2f(m[c] - m_safe);
+    float psum = (p[0] + p[1]) + (p[2] + p[3]);
+    psum += __shfl_xor(psum, 16, IA_WAVE);
+    psum += __shfl_xor(psum, 32, IA_WAVE);
+    l[c] = l[c] * corr + psum;
+    if (poison) l[c] = __uint_as_float(0x7fc00000u);
+    m[c] = m_new;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) o[c][n] *= corr;
+    pb[c] = as_s16x4((uint32_t)float_to_bf16_bits(p[0]) | ((uint32_t)float_to_bf16_bits(p[1]) << 16),
+                     (uint32_t)float_to_bf16_bits(p[2]) | ((uint32_t)float_to_bf16_bits(p[3]) << 16));
+  }
+  // ---- O^T += V^T P^T
+  const int kgc = kg < key_lo ? (key_lo & ~3) : (kg > key_hi ? (key_hi & ~3) : kg);
+  const int pagev = bt[kgc / ps];
+  const bool pagev_ok = (unsigned)pagev < (unsigned)num_pages;
+  const uint16_t* vbase = v_pages + ((size_t)(pagev_ok ? pagev : 0) * nkv + g) * HD * ps + (kgc % ps);
+  // keep the values of keys key_lo .. key_hi, zero the others (16 bits each)
+  uint32_t mlo = 0u, mhi = 0u;
+  if (kg == kgc) {
+    mlo = ((kg >= key_lo && kg <= key_hi) ? 0x0000ffffu : 0u) | ((kg + 1 >= key_lo && kg + 1 <= key_hi) ? 0xffff0000u : 0u);
+    mhi = ((kg + 2 >= key_lo && kg + 2 <= key_hi) ? 0x0000ffffu : 0u) | ((kg + 3 >= key_lo && kg + 3 <= key_hi) ? 0xffff0000u : 0u);
+  }
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const uint2 v = *reinterpret_cast<const uint2*>(vbase + (size_t)(n * 16 + j) * ps);
+    const s16x4 vreg = as_s16x4(v.x & mlo, v.y & mhi);
+#pragma unroll
+    for (int c = 0; c < CT; ++c) o[c][n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg, pb[c], o[c][n], 0, 0, 0);
+  }
+}
+
+// ------------------------------------------------------------------------ decode
+// grid (B, nkv * ceil(G/16), num_splits), 64 threads.  Token b is row b of q and out.
+extern "C" __global__ __launch_bounds__(64) void attn_decode_kernel(
+    const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const int* __restrict__ positions, const int* __restrict__ block_tables,
+    int bt_stride, int nh, int nkv, int ps, int num_pages, float scale_log2, int window, int num_splits) {
+  const int b = blockIdx.x, lane = threadIdx.x, j = lane & 15, qd = lane >> 4;
+  const int G = nh / nkv, HT = (G + 15) / 16;
+  const int g = blockIdx.y / HT, ht = blockIdx.y - g * HT;
+  const int split = blockIdx.z;
+  const int p = positions[b];
+  const int lo0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int hj = ht * 16 + j;
+  const bool col_ok = hj < G;
+  const int h = g * G + hj;
+  s16x4 qreg[1][NS];
+  if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg[0]);
+  else zero_row_operand(qreg[0]);
+  const int pos[1] = {col_ok ? p : -1};
+  const int lo[1] = {lo0};
+  f32x4 o[1][NS];
+#pragma unroll
+  for (int n = 0; n < NS; ++n) o[0][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m[1] = {-INFINITY}, l[1] = {0.f};
+  const int t_first = lo0 / 16, t_last = p / 16;
+  const int per = (t_last - t_first + 1 + num_splits - 1) / num_splits;
+  const int ta = t_first + split * per;
+  const int tb = (ta + per < t_last + 1) ? ta + per : t_last + 1;
+  const int* bt = block_tables + (size_t)b * bt_stride;
+  for (int t = ta; t < tb; ++t)
+    attn_tile<1>(t * 16, lo0, p, bt, ps, num_pages, nkv, g, k_pages, v_pages, qreg, pos, lo, scale_log2, o, m, l, lane);
+  if (!col_ok) return;
+  if (num_splits == 1) {
+    const float inv = 1.0f / l[0];
+    uint16_t* orow = out + (size_t)b * out_row_stride + (size_t)h * HD + 4 * qd;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      uint2 w;
+      w.x = (uint32_t)float_to_bf16_bits(o[0][n][0] * inv) | ((uint32_t)float_to_bf16_bits(o[0][n][1] * inv) << 16);
+      w.y = (uint32_t)float_to_bf16_bits(o[0][n][2] * inv) | ((uint32_t)float_to_bf16_bits(o[0][n][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + n * 16) = w;
+    }
+  } else {
+    const size_t rec = ((size_t)b * nh + h) * num_splits + split;
+    float* po = part_o + rec * HD + 4 * qd;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) *reinterpret_cast<f32x4*>(po + n * 16) = o[0][n];
+    if (qd == 0) { part_ml[rec * 2] = m[0]; part_ml[rec * 2 + 1] = l[0]; }
+  }
+}
+
+// Joins the parts of a split: grid (B * nh), 64 threads; parts are taken in the order of their index.
+extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, uint16_t* __restrict__ out,
+    int out_row_stride, int nh, int num_splits) {
+  const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+  const size_t rec0 = (size_t)blockIdx.x * num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, part_ml[(rec0 + s) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < num_splits; ++s) {
+    const float ms = part_ml[(rec0 + s) * 2];
+    L += (ms == -INFINITY ? 0.f : exp2f(ms - M)) * part_ml[(rec0 + s) * 2 + 1];
+  }
+  const float inv = 1.0f / L;
+  for (int dim = threadIdx.x; dim < HD; dim += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+      const float ms = part_ml[(rec0 + s) * 2];
+      if (ms != -INFINITY) acc += exp2f(ms - M) * part_o[(rec0 + s) * HD + dim];
+    }
+    out[(size_t)b * out_row_stride + (size_t)h * HD + dim] = float_to_bf16_bits(acc * inv);
+  }
+}
+
+// ----------------------------------------------------------------------- prefill
+// grid (num_tiles, nkv * ceil(G / GH), 64 / (16 * CT / GH)), 64 threads.
+// tiles[i] = (request, first row of a block of 64 rows among the request's new tokens).
+extern "C" __global__ __launch_bounds__(64) void attn_prefill_kernel(
+    const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
+    const int* __restrict__ seq_starts, const int* __restrict__ seq_ctx, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, float scale_log2,
+    int window, int GH) {
+  constexpr int CT = PREFILL_CT;
+  const int lane = threadIdx.x, j = lane & 15, qd = lane >> 4;
+  const int sidx = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
+  const int G = nh / nkv, HC = (G + GH - 1) / GH, TT = CT / GH;
+  const int g = blockIdx.y / HC, hc = blockIdx.y - g * HC;
+  const int rb = row0 + blockIdx.z * TT * 16;
+  const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
+  if (rb >= qlen) return;
+  s16x4 qreg[CT][NS];
+  int pos[CT], lo[CT];
+  f32x4 o[CT][NS];
+  float m[CT], l[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int hh = c % GH, tt = c / GH;
+    const int hj = hc * GH + hh, row = rb + tt * 16 + j;
+    const bool ok = hj < G && row < qlen;
+    pos[c] = ok ? ctx + row : -1;
+    lo[c] = (window > 0 && pos[c] - window + 1 > 0) ? pos[c] - window + 1 : 0;
+    if (ok) load_row_operand(q + (size_t)(qstart + row) * q_row_stride + (size_t)(g * G + hj) * HD, qd, qreg[c]);
+    else zero_row_operand(qreg[c]);
+    m[c] = -INFINITY;
+    l[c] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) o[c][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  const int last_row = (rb + TT * 16 < qlen ? rb + TT * 16 : qlen) - 1;
+  const int key_hi = ctx + last_row;
+  const int key_lo = (window > 0 && ctx + rb - window + 1 > 0) ? ctx + rb - window + 1 : 0;
+  const int* bt = block_tables + (size_t)sidx * bt_stride;
+  for (int t = key_lo / 16; t <= key_hi / 16; ++t)
+    attn_tile<CT>(t * 16, key_lo, key_hi, bt, ps, num_pages, nkv, g, k_pages, v_pages, qreg, pos, lo, scale_log2, o, m,
+                  l, lane);
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    if (pos[c] < 0) continue;
+    const int hh = c % GH, tt = c / GH;
+    const int row = rb + tt * 16 + j;
+    const float inv = 1.0f / l[c];
+    uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride + (size_t)(g * G + hc * GH + hh) * HD + 4 * qd;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      uint2 w;
+      w.x = (uint32_t)float_to_bf16_bits(o[c][n][0] * inv) | ((uint32_t)float_to_bf16_bits(o[c][n][1] * inv) << 16);
+      w.y = (uint32_t)float_to_bf16_bits(o[c][n][2] * inv) | ((uint32_t)float_to_bf16_bits(o[c][n][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + n * 16) = w;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ C interface
+extern "C" int ia_attn_head_dim() { return HD; }
+
+extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
+                              int out_row_stride, float* part_o, float* part_ml, const int* positions,
+                              const int* block_tables, int bt_stride, int B, int nh, int nkv, int ps, int num_pages,
+                              float scale, int window, int num_splits, hipStream_t stream) {
+  if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 || bt_stride <= 0 ||
+      num_splits < 1 || num_splits > 65535)
+    return IA_ERR_BAD_ARG;
+  if (num_splits > 1 && (!part_o || !part_ml)) return IA_ERR_BAD_ARG;
+  if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
+  if (B == 0) return IA_OK;
+  const int G = nh / nkv, HT = (G + 15) / 16;
+  if (nkv * HT > 65535) return IA_ERR_UNSUPPORTED;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  dim3 grid(B, nkv * HT, num_splits);
+  attn_decode_kernel<<<grid, 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
+                                              (const uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o,
+                                              part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages,
+                                              scale_log2, window, num_splits);
+  IA_LAUNCH_CHECK();
+  if (num_splits > 1) {
+    attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,
+                                                         num_splits);
+    IA_LAUNCH_CHECK();
+  }
+  return IA_OK;
+}
+
+extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
+                               int out_row_stride, const int* seq_starts, const int* seq_ctx, const int* block_tables,
+                               int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
+                               float scale, int window, hipStream_t stream) {
+  if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
+      bt_stride <= 0)
+    return IA_ERR_BAD_ARG;
+  if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
+  if (num_tiles == 0) return IA_OK;
+  constexpr int CT = PREFILL_CT;
+  const int G = nh / nkv;
+  int GH = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+  if (GH > CT) GH = CT;
+  const int HC = (G + GH - 1) / GH, TT = CT / GH;
+  if (nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  dim3 grid(num_tiles, nkv * HC, 64 / (16 * TT));
+  attn_prefill_kernel<<<grid, 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
+                                               (const uint16_t*)v_pages, (uint16_t*)out, out_row_stride, seq_starts,
+                                               seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages,
+                                               scale_log2, window, GH);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}

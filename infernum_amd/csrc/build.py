@@ -42,7 +42,7 @@ CORE_SOURCES = [
     "attention_generic.hip",
     "sampling.hip",
 ]
-HEADERS = ["common.h", "attention_mfma.h"]
+HEADERS = ["common.h"]
 
 # Head sizes whose attention library `build_all` compiles ahead of time.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)

@@ -110,7 +110,9 @@ extern "C" int ia_residual_add(float* h, const void* delta, int act_dtype, int N
 // The first `rot` values of every q and k head are rotated in half-split pairs
 // (x[i], x[i + rot/2]) by the angle pos * inv_freq[i], computed in fp32.
 // q is rotated in place; rotated k and raw v go to the page slot of the token:
-// pages are [num_pages, nkv, page_size, d]; slot = page * page_size + offset.
+// key pages are [num_pages, nkv, page_size, d]; value pages are stored transposed,
+// [num_pages, nkv, d, page_size], which is the layout the matrix cores want for
+// the product of probabilities and values; slot = page * page_size + offset.
 // inv_freq == nullptr: no rotation.  slot < 0 or write_kv == 0: nothing is written.
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_append_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(T* __restrict__ qkv
   }
   for (int idx = threadIdx.x; idx < nkv * d; idx += 256) {
     const int g = idx / d, i = idx - g * d;
-    v_pages[(((size_t)page * nkv + g) * page_size + off) * d + i] = row[(size_t)(nh + nkv + g) * d + i];
+    v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] = row[(size_t)(nh + nkv + g) * d + i];
   }
 }
 

@@ -124,8 +124,8 @@ def rope_kv_append(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optiona
                    v_pages: Optional[torch.Tensor] = None) -> None:
     """Rotate q (in place) and k, and write k and v to their page slots.
 
-    qkv is [N, (nh + 2 nkv) d] (or [N, nh d] when no pages are given).  Pages are
-    [num_pages, nkv, page_size, d].
+    qkv is [N, (nh + 2 nkv) d] (or [N, nh d] when no pages are given).  Key pages are
+    [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size].
     """
     _dev(qkv, positions, inv_freq, slots, k_pages, v_pages)
     write = k_pages is not None
@@ -140,9 +140,10 @@ def rope_kv_append(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optiona
     if write:
         _need(v_pages is not None and slots is not None, "rope: k_pages, v_pages and slots go together")
         _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "rope: pages must have qkv's dtype")
-        _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
-              and tuple(v_pages.shape) == tuple(k_pages.shape), "rope: pages must be [num_pages, nkv, page_size, d]")
         num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+        _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
+              and tuple(v_pages.shape) == (num_pages, nkv, d, page_size),
+              "rope: key pages must be [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size]")
         _i32(slots, N, "rope slots")
     _ok(_core().ia_rope_kv_append(_p(qkv), DTYPE_CODE[qkv.dtype], _p(positions), _p(slots), _p(inv_freq),
                                   _p(k_pages), _p(v_pages), N, row, nh, nkv, d, rot if inv_freq is not None else 0,
@@ -204,7 +205,8 @@ def _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, what):
     _need(out.dim() == 2 and out.shape[1] == nh * d and out.shape[0] == qkv.shape[0],
           f"{what}: out must be [N, nh*d]")
     _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
-          and tuple(v_pages.shape) == tuple(k_pages.shape), f"{what}: pages must be [num_pages, nkv, page_size, d]")
+          and tuple(v_pages.shape) == (k_pages.shape[0], nkv, d, k_pages.shape[2]),
+          f"{what}: key pages must be [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size]")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, f"{what}: block_tables int32 [B, MB]")
     _need(nh % nkv == 0, f"{what}: nh must be a multiple of nkv")
 
@@ -226,6 +228,68 @@ def attention_generic(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
                                      DTYPE_CODE[out.dtype], _p(token_seq), _p(positions), _p(block_tables),
                                      block_tables.shape[1], N, nh, nkv, d, k_pages.shape[2], k_pages.shape[0],
                                      ctypes.c_float(scale), int(window), _stream()), "attention_generic")
+
+
+def _attn(d: int) -> ctypes.CDLL:
+    lib = load_library(f"attn_d{d}")
+    return lib
+
+
+def decode_splits(batch: int, nh: int, nkv: int, max_len: int) -> int:
+    """Parts the keys of a request are cut into, so that a small batch still fills the GPU."""
+    groups = batch * nkv * ((nh // nkv + 15) // 16)
+    tiles = max(1, (max_len + 15) // 16)
+    return max(1, min((1024 + groups - 1) // groups, (tiles + 1) // 2, 64))
+
+
+def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                     positions: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                     window: int, max_len: int, num_splits: Optional[int] = None) -> None:
+    """bf16 attention of B single tokens (row b of qkv: token b at positions[b]) over their pages, on MFMA.
+
+    ``max_len`` bounds the positions (host side), and sets how many parts the keys are split into.
+    """
+    _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, "attention_decode")
+    B = out.shape[0]
+    _need(qkv.dtype == torch.bfloat16, "attention_decode: bf16 only")
+    _i32(positions, B, "attention_decode positions")
+    _need(block_tables.shape[0] >= B, "attention_decode: one row of block_tables per token")
+    ps = k_pages.shape[2]
+    _need(ps % 4 == 0, f"attention_decode: page size {ps} is not a multiple of 4")
+    _need(block_tables.shape[1] * ps >= max_len, "attention_decode: block_tables are narrower than max_len")
+    splits = num_splits or decode_splits(B, nh, nkv, max_len)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)
+        part_ml = torch.empty(B * nh * splits * 2, dtype=torch.float32, device=out.device)
+    _ok(_attn(d).ia_attn_decode(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d, _p(part_o),
+                                _p(part_ml), _p(positions), _p(block_tables), block_tables.shape[1], B, nh, nkv, ps,
+                                k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _stream()),
+        "attention_decode")
+
+
+def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                      seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
+                      tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, d: int, scale: float,
+                      window: int) -> None:
+    """bf16 causal attention of portions of prompts over their pages, on MFMA.
+
+    Request s brings rows seq_starts[s] .. seq_starts[s+1]-1 of qkv and had seq_ctx[s] tokens cached
+    before; tiles[i] = (s, first row of a block of 64 among the request's rows).
+    """
+    _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, "attention_prefill")
+    _need(qkv.dtype == torch.bfloat16, "attention_prefill: bf16 only")
+    B = block_tables.shape[0]
+    _i32(seq_starts, B + 1, "attention_prefill seq_starts")
+    _i32(seq_ctx, B, "attention_prefill seq_ctx")
+    _need(tiles.dtype == torch.int32 and tiles.is_cuda and tiles.is_contiguous() and tiles.numel() >= 2 * num_tiles,
+          "attention_prefill: tiles int32 [num_tiles, 2]")
+    ps = k_pages.shape[2]
+    _need(ps % 4 == 0, f"attention_prefill: page size {ps} is not a multiple of 4")
+    _ok(_attn(d).ia_attn_prefill(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d, _p(seq_starts),
+                                 _p(seq_ctx), _p(block_tables), block_tables.shape[1], _p(tiles), num_tiles, nh, nkv,
+                                 ps, k_pages.shape[0], ctypes.c_float(scale), int(window), _stream()),
+        "attention_prefill")
 
 
 # ------------------------------------------------------------------------- sampling

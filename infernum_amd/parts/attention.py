@@ -89,14 +89,14 @@ class Attention(Mixer):
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d
         bt = ctx.block_tables[cache.group]
-        if not self.use_mfma:
+        if not self.use_mfma or cache.k_pages.shape[2] % 4:
             K.attention_generic(qkv, cache.k_pages, cache.v_pages, out, ctx.token_seq, ctx.positions, bt, nh, nkv, d,
                                 self.scale, self.window)
             return
         nd = ctx.num_decode
         if nd > 0:
             K.attention_decode(qkv[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.positions[:nd], bt[:nd], nh, nkv,
-                               d, self.scale, self.window, ctx.max_total_len, ctx.extras.get("decode_workspace"))
+                               d, self.scale, self.window, ctx.max_total_len)
         if ctx.num_seqs > nd:
             K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
                                 ctx.prefill_tiles, ctx.num_prefill_tiles, nh, nkv, d, self.scale, self.window)

@@ -93,15 +93,15 @@ def test_rope_reference_vector_and_pages():
     qkv = torch.tensor([[1.0, 2, 3, 4, 1, 2, 3, 4, 9, 8, 7, 6]], device=DEV)
     inv = torch.tensor([1.0, 0.01], device=DEV)
     kp = torch.zeros(5, nkv, ps, d, device=DEV)
-    vp = torch.zeros(5, nkv, ps, d, device=DEV)
+    vp = torch.zeros(5, nkv, d, ps, device=DEV)
     K().rope_kv_append(qkv, torch.tensor([1], dtype=torch.int32, device=DEV), inv, nh, nkv, d, d,
                        torch.tensor([2 * ps + 1], dtype=torch.int32, device=DEV), kp, vp)
     c0, s0, c1, s1 = math.cos(1.0), math.sin(1.0), math.cos(0.01), math.sin(0.01)
     want = torch.tensor([1 * c0 - 3 * s0, 2 * c1 - 4 * s1, 3 * c0 + 1 * s0, 4 * c1 + 2 * s1], device=DEV)
     assert torch.allclose(qkv[0, :4], want, atol=1e-6)
     assert torch.allclose(kp[2, 0, 1], want, atol=1e-6)
-    assert torch.equal(vp[2, 0, 1], torch.tensor([9.0, 8, 7, 6], device=DEV))
-    assert kp.abs().sum() == kp[2, 0, 1].abs().sum() and vp.abs().sum() == vp[2, 0, 1].abs().sum()
+    assert torch.equal(vp[2, 0, :, 1], torch.tensor([9.0, 8, 7, 6], device=DEV))     # values lie transposed
+    assert kp.abs().sum() == kp[2, 0, 1].abs().sum() and vp.abs().sum() == vp[2, 0, :, 1].abs().sum()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -114,7 +114,7 @@ def test_rope_kv_append(dtype, nh, nkv, d, rot, ps):
     inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV)
     slots = torch.randperm(pages * ps)[:N].to(torch.int32).to(DEV)
     kp = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV)
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros(pages, nkv, d, ps, dtype=dtype, device=DEV)
     K().rope_kv_append(qkv, pos, inv, nh, nkv, d, rot, slots, kp, vp)
     x = q0.double().reshape(N, nh + 2 * nkv, d)
     ang = (pos.float()[:, None] * inv[None, :]).double()      # angles are fp32 products, as in the kernel
@@ -128,7 +128,7 @@ def test_rope_kv_append(dtype, nh, nkv, d, rot, ps):
     for n in range(N):
         p, o = int(slots[n]) // ps, int(slots[n]) % ps
         assert torch.allclose(kp[p, :, o].double(), roted[n, nh:], atol=tol, rtol=tol)
-        assert torch.equal(vp[p, :, o], q0[n].reshape(nh + 2 * nkv, d)[nh + nkv:])
+        assert torch.equal(vp[p, :, :, o], q0[n].reshape(nh + 2 * nkv, d)[nh + nkv:])
     # queries only (a layer that reads another's keys and values)
     q2 = q0[:, :nh * d].contiguous()
     K().rope_kv_append(q2, pos, inv, nh, nkv, d, rot)
@@ -195,7 +195,7 @@ def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
         b, j, factor = scale_one
         kd[b][j] *= factor
     kp = torch.zeros(num_pages, nkv, ps, d)
-    vp = torch.zeros(num_pages, nkv, ps, d)
+    vp = torch.zeros(num_pages, nkv, d, ps)
     it = iter(perm)
     for b in range(B):
         for i in range(pages_per[b]):
@@ -203,7 +203,7 @@ def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
             bt[b, i] = p
             n = min(ps, lens[b] - i * ps)
             kp[p, :, :n] = kd[b][i * ps:i * ps + n].transpose(0, 1)
-            vp[p, :, :n] = vd[b][i * ps:i * ps + n].transpose(0, 1)
+            vp[p, :, :, :n] = vd[b][i * ps:i * ps + n].permute(1, 2, 0)
     N = sum(q_lens)
     q = torch.randn(N, nh * d, generator=g)
     token_seq = torch.cat([torch.full((ql,), b, dtype=torch.int32) for b, ql in enumerate(q_lens)])
@@ -267,6 +267,87 @@ def test_attention_generic_missing_page_poisons():
     K().attention_generic(case["q"], case["kp"], case["vp"], out, case["token_seq"], case["positions"], case["bt"],
                           nh, nkv, d, 1.0, 8)
     assert not out.isnan().any()
+
+
+def _prefill_tiles(q_lens, first_prefill=0):
+    tiles = [(s, r) for s in range(first_prefill, len(q_lens)) for r in range(0, q_lens[s], 64)]
+    return torch.tensor(tiles, dtype=torch.int32, device=DEV).reshape(-1, 2), len(tiles)
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,window", [(8, 2, 128, 16, 0), (6, 3, 48, 4, 0), (4, 4, 16, 8, 0), (32, 8, 128, 16, 0),
+                                                (20, 1, 64, 64, 0), (3, 1, 80, 12, 0), (2, 1, 256, 16, 0),
+                                                (8, 2, 128, 16, 100), (6, 3, 48, 4, 9), (7, 7, 32, 8, 33)])
+def test_attention_mfma_prefill(nh, nkv, d, ps, window):
+    """Portions of prompts with earlier context, rows that do not fill a tile, several requests."""
+    lens, q_lens = [70, 3, 331, 64, 150], [70, 3, 140, 17, 1]
+    case = _paged_case(nh, nkv, d, ps, lens, q_lens, torch.bfloat16, seed=d + nh)
+    N = case["N"]
+    out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    starts = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    ctx = torch.tensor([L - q for L, q in zip(lens, q_lens)], dtype=torch.int32, device=DEV)
+    tiles, nt = _prefill_tiles(q_lens)
+    K().attention_prefill(case["q"], case["kp"], case["vp"], out, starts, ctx, case["bt"], tiles, nt, nh, nkv, d, scale,
+                          window)
+    want = _ref_attention(case, nh, nkv, d, scale, window)
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err <= 2e-2, err
+    gen = torch.empty_like(out)
+    K().attention_generic(case["q"], case["kp"], case["vp"], gen, case["token_seq"], case["positions"], case["bt"], nh,
+                          nkv, d, scale, window)
+    assert (out.double() - gen.double()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("splits", [None, 1, 3, 7])
+@pytest.mark.parametrize("nh,nkv,d,ps,window", [(8, 2, 128, 16, 0), (6, 3, 48, 4, 0), (32, 8, 128, 16, 0), (40, 2, 64, 8, 0),
+                                                (5, 5, 16, 16, 0), (2, 1, 256, 64, 0), (8, 2, 128, 16, 100), (4, 1, 96, 4, 17)])
+def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
+    lens = [70, 1, 331, 64, 150, 16, 17]
+    q_lens = [1] * len(lens)
+    case = _paged_case(nh, nkv, d, ps, lens, q_lens, torch.bfloat16, seed=d + nh + 1)
+    B = len(lens)
+    out = torch.full((B, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    K().attention_decode(case["q"], case["kp"], case["vp"], out, case["positions"], case["bt"], nh, nkv, d, scale,
+                         window, max(lens), num_splits=splits)
+    want = _ref_attention(case, nh, nkv, d, scale, window)
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err <= 2e-2, err
+
+
+def test_attention_mfma_far_key_stale_pages_and_missing_page():
+    """A far key carries the softmax; pages hold NaN wherever this request has no data;
+    a needed key without a page gives NaN instead of a fault."""
+    nh, nkv, d, ps = 4, 1, 64, 16
+    lens, q_lens = [500, 40, 77], [1, 40, 30]
+    case = _paged_case(nh, nkv, d, ps, lens, q_lens, torch.bfloat16, seed=3, scale_one=(0, 17, 6.0))
+    # poison every slot that holds no key of these requests
+    used_k = torch.zeros_like(case["kp"], dtype=torch.bool)
+    used_v = torch.zeros_like(case["vp"], dtype=torch.bool)
+    for b, L in enumerate(lens):
+        for i in range(-(-L // ps)):
+            n = min(ps, L - i * ps)
+            pg = int(case["bt"][b, i])
+            used_k[pg, :, :n] = True
+            used_v[pg, :, :, :n] = True
+    case["kp"][~used_k] = float("nan")
+    case["vp"][~used_v] = float("nan")
+    scale = 1.0 / math.sqrt(d)
+    want = _ref_attention(case, nh, nkv, d, scale, 0)
+    out = torch.full((case["N"], nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    starts = torch.tensor([0, 1, 41, 71], dtype=torch.int32, device=DEV)
+    ctx = torch.tensor([499, 0, 47], dtype=torch.int32, device=DEV)
+    tiles, nt = _prefill_tiles(q_lens, first_prefill=1)
+    K().attention_prefill(case["q"], case["kp"], case["vp"], out, starts, ctx, case["bt"], tiles, nt, nh, nkv, d, scale, 0)
+    K().attention_decode(case["q"][:1], case["kp"], case["vp"], out[:1], case["positions"][:1], case["bt"][:1], nh, nkv,
+                         d, scale, 0, 500)
+    assert not out.isnan().any()
+    assert (out.double().cpu() - want).abs().max().item() <= 2e-2
+    bt = case["bt"].clone()
+    bt[0, 3] = -1
+    K().attention_decode(case["q"][:1], case["kp"], case["vp"], out[:1], case["positions"][:1], bt[:1], nh, nkv, d,
+                         scale, 0, 500)
+    assert out[:1].isnan().all()
 
 
 # -------------------------------------------------------------------- sampling
