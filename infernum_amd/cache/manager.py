@@ -189,6 +189,27 @@ class CacheManager:
     def num_tokens(self, req: Hashable) -> int:
         return self._tokens[req]
 
+    def pages_needed(self, req: Optional[Hashable], n_new: int) -> List[int]:
+        """Per group, the pages that n_new more tokens of the request would take from the pool
+        (a request that is not admitted yet holds nothing)."""
+        if req is not None and req in self._slot_of:
+            return [g.pages_missing(req, n_new) for g in self.groups]
+        return [pages_for(n_new, g.page_size) for g in self.groups]
+
+    def tokens_that_fit(self, req: Optional[Hashable], promised: Optional[Sequence[int]] = None) -> int:
+        """How many more tokens of the request the pool can hold, with ``promised[g]`` pages of
+        every group already spoken for."""
+        best = 1 << 60
+        for i, g in enumerate(self.groups):
+            avail = g.allocator.num_free - (promised[i] if promised is not None else 0)
+            if req is not None and req in self._slot_of:
+                t = g.tables[req]
+                room = (len(t.pages) + max(avail, 0)) * g.page_size - t.num_tokens
+            else:
+                room = max(avail, 0) * g.page_size
+            best = min(best, room)
+        return max(best, 0)
+
     def can_reserve(self, req: Hashable, n_new: int) -> bool:
         return all(g.allocator.can_allocate(g.pages_missing(req, n_new)) for g in self.groups)
 

@@ -64,20 +64,26 @@ def find_hipcc() -> Optional[str]:
     return None
 
 
+_lib_dir: Optional[str] = None
+_lib_dir_lock = threading.Lock()
+
+
 def lib_dir() -> str:
     """Folder for built libraries: in the package if writable, else a temporary one."""
-    d = os.path.join(PKG_DIR, "_lib")
-    try:
-        os.makedirs(d, exist_ok=True)
-        probe = os.path.join(d, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
-        os.unlink(probe)
-        return d
-    except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"infernum_amd_lib_{os.getuid()}")
-        os.makedirs(d, exist_ok=True)
-        return d
+    global _lib_dir
+    with _lib_dir_lock:
+        if _lib_dir is None:
+            d = os.path.join(PKG_DIR, "_lib")
+            try:
+                os.makedirs(d, exist_ok=True)
+                fd, probe = tempfile.mkstemp(prefix=".w", dir=d)
+                os.close(fd)
+                os.unlink(probe)
+            except OSError:
+                d = os.path.join(tempfile.gettempdir(), f"infernum_amd_lib_{os.getuid()}")
+                os.makedirs(d, exist_ok=True)
+            _lib_dir = d
+        return _lib_dir
 
 
 def _existing(files: Sequence[str]) -> List[str]:

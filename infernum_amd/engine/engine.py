@@ -105,15 +105,12 @@ class Engine:
     # ---- the step ------------------------------------------------------------------
     def pages_short(self, entries: Sequence[StepEntry]) -> bool:
         """True when the pool cannot hold this step's new tokens."""
-        for g in self.cache.groups:
-            need = 0
-            for e in entries:
-                if self.cache.has(e.request):
-                    need += g.pages_missing(e.request, len(e.tokens))
-                else:
-                    need += (len(e.tokens) + g.page_size - 1) // g.page_size
-            if need > g.allocator.num_free:
-                return True
+        need = [0] * len(self.cache.groups)
+        for e in entries:
+            for i, n in enumerate(self.cache.pages_needed(e.request, len(e.tokens))):
+                need[i] += n
+        if any(n > g.allocator.num_free for n, g in zip(need, self.cache.groups)):
+            return True
         new = sum(1 for e in entries if not self.cache.has(e.request))
         return new > self.cache.slots.num_free
 

@@ -1,0 +1,229 @@
+"""The generation loop: scheduler, step function and sampler put together.
+
+``Runtime`` is what a user of the package talks to.  It takes requests
+(``submit``), and every ``step`` asks the scheduler for a batch, runs it through
+:meth:`Engine.step` as one mixed batch, chooses the next token of every request
+whose last token was in the batch, and tells the scheduler.  ``generate`` and
+``generate_stream`` drive the loop until their request is done; any other
+requests that are waiting or running move along in the same steps.
+
+The reference splits this over ``Engine`` (a worker thread fed through a
+channel, infernum-runtime/src/engine.rs:39-238) and ``Runtime`` (tokenizer on
+top, infernum-runtime/src/runtime.rs:17-135).  Here one object runs on the
+caller's thread: the model, the cache and the scheduler have one owner, and
+nothing needs a lock.
+"""
+from __future__ import annotations
+
+import os
+from typing import Any, Callable, Iterator, List, Optional, Sequence, Union
+
+from ..cache import CacheConfig
+from ..sampling.params import GenerateOptions, SamplingParams
+from ..sampling.sampler import RowRequest
+from .engine import Engine, StepEntry
+from .scheduler import (BatchConfig, FinishReason, GenerationEvent, Scheduler, SchedulerOutput, SequencePhase,
+                        SequenceState, TokenSender)
+
+Prompt = Union[str, Sequence[int]]
+
+
+class GenerationError(RuntimeError):
+    pass
+
+
+class Runtime:
+    def __init__(self, engine: Any, tokenizer: Any = None, batch_config: Optional[BatchConfig] = None,
+                 max_seq_len: Optional[int] = None, sampler: Any = None):
+        """``engine`` has ``step(entries)``, ``end(request)`` and ``cache``; ``sampler`` has
+        ``select(logits, rows)``; ``tokenizer`` (optional) has ``encode`` and ``decode``."""
+        self.engine = engine
+        self.tokenizer = tokenizer
+        cc = engine.cache.config
+        if batch_config is None:
+            batch_config = BatchConfig(block_size=cc.page_size, num_blocks=cc.num_pages,
+                                       max_batch_size=min(32, cc.num_state_slots))
+        if batch_config.block_size != cc.page_size or batch_config.num_blocks != cc.num_pages:
+            raise ValueError("batch_config's block_size and num_blocks must be those the engine's cache was made with")
+        if batch_config.max_batch_size > cc.num_state_slots:
+            raise ValueError("max_batch_size is larger than the number of state slots of the cache")
+        limit = getattr(getattr(engine, "rt", None), "max_tokens_per_step", None)
+        if limit is not None and batch_config.max_tokens_per_step > limit:
+            raise ValueError(f"max_tokens_per_step {batch_config.max_tokens_per_step} is above the engine's {limit}")
+        self.batch_config = batch_config
+        self.scheduler = Scheduler(batch_config, max_seq_len=max_seq_len)
+        if sampler is None:
+            from ..sampling.sampler import Sampler
+            sampler = Sampler(engine.rt.device)
+        self.sampler = sampler
+        self.steps = 0
+        self.tokens_run = 0
+
+    # ---- building ---------------------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", batch_config: Optional[BatchConfig] = None,
+                        max_seq_len: Optional[int] = None, device: Any = "cuda:0") -> "Runtime":
+        bc = batch_config or BatchConfig()
+        engine = Engine.from_pretrained(
+            model_dir, dtype=dtype, device=device, max_tokens_per_step=bc.max_tokens_per_step,
+            cache_config=CacheConfig(page_size=bc.block_size, num_pages=bc.num_blocks,
+                                     num_state_slots=bc.max_batch_size))
+        return cls(engine, load_tokenizer(model_dir), bc, max_seq_len)
+
+    # ---- requests ----------------------------------------------------------------------
+    def submit(self, input_ids: Sequence[int], options: GenerateOptions,
+               token_tx: Optional[TokenSender] = None) -> SequenceState:
+        """Queue a request; its tokens arrive through ``token_tx`` as the loop runs (engine.rs:112-126)."""
+        V = getattr(getattr(self.engine, "spec", None), "vocab_size", None)
+        if V is not None and any(not 0 <= int(t) < V for t in input_ids):
+            raise ValueError(f"prompt holds a token id outside the vocabulary [0, {V})")
+        return self.scheduler.add_request(input_ids, options, token_tx)
+
+    def step(self) -> SchedulerOutput:
+        """One iteration: schedule, run the batch, choose tokens, update (engine.rs:191-237)."""
+        plan = self.scheduler.step(self.engine.cache)
+        if plan.is_empty():
+            return plan
+        entries: List[StepEntry] = []
+        rows: List[RowRequest] = []
+        for t in plan.decode:
+            s = t.seq
+            entries.append(StepEntry(s.id, [s.generated_ids[-1]], [0]))
+            rows.append(self._row(s))
+        for t in plan.prefill:
+            entries.append(StepEntry(t.seq.id, t.token_ids, [len(t.token_ids) - 1] if t.completes else []))
+            if t.completes:
+                rows.append(self._row(t.seq))
+        try:
+            logits = self.engine.step(entries)
+            tokens = self.sampler.select(logits, rows)
+        except Exception as e:                    # the requests of this batch end with an error event
+            for t in list(plan.decode) + list(plan.prefill):
+                self.scheduler._fail(t.seq, f"{type(e).__name__}: {e}")
+            raise
+        self.steps += 1
+        self.tokens_run += plan.num_tokens
+        k = 0
+        for t in plan.decode:
+            self.scheduler.on_decode_done(t, tokens[k])
+            k += 1
+        for t in plan.prefill:
+            if t.completes:
+                self.scheduler.on_prefill_done(t, tokens[k])
+                k += 1
+            else:
+                self.scheduler.on_prefill_done(t, None)
+        return plan
+
+    @staticmethod
+    def _row(s: SequenceState) -> RowRequest:
+        sp = s.options.sampling
+        if sp is None:
+            return RowRequest(None)
+        hist = s.all_tokens() if abs(sp.repetition_penalty - 1.0) > 1.1920929e-07 else ()
+        return RowRequest(sp, len(s.generated_ids), hist)
+
+    def run(self, until: Optional[Callable[[], bool]] = None) -> None:
+        """Step until nothing waits or runs (or until ``until()`` is true)."""
+        while not self.scheduler.is_idle():
+            if until is not None and until():
+                return
+            self.step()
+        self.scheduler.reap(self.engine.cache)
+
+    # ---- whole generations ---------------------------------------------------------------
+    def generate(self, prompt: Prompt, options: Optional[GenerateOptions] = None) -> Union[str, List[int]]:
+        """Blocks until done.  A list of token ids gives a list of new token ids (engine.rs:132-145);
+        a string is encoded with the tokenizer, the end-of-sequence id is filled in from the model's
+        configuration when the options name none, and the new text comes back (runtime.rs:81-97)."""
+        ids, options, is_text = self._prepare(prompt, options)
+        out = self.generate_batch([ids], options)[0]
+        return self.tokenizer.decode(out) if is_text else out
+
+    def generate_batch(self, prompts: Sequence[Sequence[int]],
+                       options: Union[None, GenerateOptions, Sequence[GenerateOptions]] = None) -> List[List[int]]:
+        """Several requests at once through continuous batching; new token ids of each, in order."""
+        if options is None or isinstance(options, GenerateOptions):
+            options = [options or GenerateOptions()] * len(prompts)
+        if len(options) != len(prompts):
+            raise ValueError("one GenerateOptions per prompt, or one for all")
+        if any(not o.use_kv_cache for o in options):
+            return [self._generate_without_cache(p, o) for p, o in zip(prompts, options)]
+        seqs = [self.submit(p, o) for p, o in zip(prompts, options)]
+        self.run(until=lambda: all(s.phase == SequencePhase.FINISHED for s in seqs))
+        self.scheduler.reap(self.engine.cache)
+        for s in seqs:
+            if s.error is not None:
+                raise GenerationError(s.error)
+        return [list(s.generated_ids) for s in seqs]
+
+    def generate_stream(self, prompt: Prompt, options: Optional[GenerateOptions] = None) -> Iterator[Union[int, str]]:
+        """Yields each new token (its text for a string prompt) as soon as it is chosen (engine.rs:148-170)."""
+        ids, options, is_text = self._prepare(prompt, options)
+        fresh: List[int] = []
+        seq = self.submit(ids, options, lambda ev: (fresh.append(ev.token) if ev.kind == "token" else None, True)[1])
+        try:
+            while seq.phase != SequencePhase.FINISHED or fresh:
+                if not fresh:
+                    self.step()
+                while fresh:
+                    t = fresh.pop(0)
+                    yield self.tokenizer.decode([t]) if is_text else t
+        finally:
+            self.scheduler.cancel(seq)            # a consumer that stops early cancels the request
+            self.scheduler.reap(self.engine.cache)
+        if seq.error is not None:
+            raise GenerationError(seq.error)
+
+    def _prepare(self, prompt: Prompt, options: Optional[GenerateOptions]):
+        options = options or GenerateOptions()
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise GenerationError("a text prompt needs a tokenizer (tokenizer.json in the model folder); "
+                                      "pass token ids instead")
+            ids = self.tokenizer.encode(prompt, add_bos=True)
+            if options.eos_token_id is None:
+                eos = getattr(getattr(self.engine, "spec", None), "eos_token_id", None)
+                options = GenerateOptions(options.max_new_tokens, eos, options.sampling, options.use_kv_cache)
+            return ids, options, True
+        return [int(t) for t in prompt], options, False
+
+    def _generate_without_cache(self, prompt: Sequence[int], options: GenerateOptions) -> List[int]:
+        """Every new token from the whole sequence, computed afresh (GenerateOptions.use_kv_cache = false)."""
+        toks, out = [int(t) for t in prompt], []
+        probe = SequenceState("nocache", toks, options)
+        for _ in range(options.max_new_tokens):
+            logits = self.engine.step([StepEntry("__no_kv_cache__", toks + out, [len(toks) + len(out) - 1])])
+            self.engine.end("__no_kv_cache__")
+            probe.generated_ids = out
+            tok = self.sampler.select(logits, [self._row(probe)])[0]
+            if options.eos_token_id is not None and tok == options.eos_token_id:
+                break
+            out = out + [tok]
+        return out
+
+
+class TextTokenizer:
+    """tokenizer.json of a model folder through the ``tokenizers`` library."""
+
+    def __init__(self, path: str, bos_token_id: Optional[int] = None):
+        from tokenizers import Tokenizer
+        self._tok = Tokenizer.from_file(path)
+        self.bos_token_id = bos_token_id
+
+    def encode(self, text: str, add_bos: bool = True) -> List[int]:
+        ids = list(self._tok.encode(text, add_special_tokens=False).ids)
+        if add_bos and self.bos_token_id is not None and (not ids or ids[0] != self.bos_token_id):
+            ids = [self.bos_token_id] + ids
+        return ids
+
+    def decode(self, ids: Sequence[int]) -> str:
+        return self._tok.decode(list(ids), skip_special_tokens=True)
+
+
+def load_tokenizer(model_dir: str) -> Optional[TextTokenizer]:
+    path = os.path.join(model_dir, "tokenizer.json")
+    if not os.path.isfile(path):
+        return None
+    from ..config.registry import load_config
+    return TextTokenizer(path, getattr(load_config(model_dir), "bos_token_id", None))

@@ -1,0 +1,3 @@
+from .params import GenerateOptions, SamplingParams
+from .rng import token_uniform
+from .sampler import RowRequest, Sampler

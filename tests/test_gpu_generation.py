@@ -1,0 +1,116 @@
+"""Generation through the entry points on the GPU: greedy tokens against the plain
+implementation, sampled tokens against the plain sampler fed with the engine's logits,
+continuous batching with portions and with too few pages, the command line."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_llama as P
+import tiny_models as TM
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name in ("A", "B"):
+        d = str(tmp_path_factory.mktemp(f"gen{name}"))
+        TM.write_tiny(name, d, dtype=torch.float32)
+        out[name] = (d,) + P.read_model(d)
+    return out
+
+
+def _runtime(d, dtype, **kw):
+    from infernum_amd import BatchConfig, Runtime
+    return Runtime.from_pretrained(d, dtype=dtype, batch_config=BatchConfig(**kw))
+
+
+def test_greedy_A_through_the_entry_point(folders):
+    """Configuration A's workload: one prompt of 7 tokens, 16 greedy tokens, pages of 4."""
+    from infernum_amd import GenerateOptions
+    d, cfg, w = folders["A"]
+    prompt = [3, 141, 59, 26, 53, 58, 97]
+    want = P.greedy(cfg, w, prompt, 16)
+    rt = _runtime(d, "float32", block_size=4, num_blocks=16, max_batch_size=2)
+    assert rt.generate(prompt, GenerateOptions(max_new_tokens=16)) == want
+    assert list(rt.generate_stream(prompt, GenerateOptions(max_new_tokens=16))) == want
+    assert rt.generate(prompt, GenerateOptions(max_new_tokens=5, use_kv_cache=False)) == want[:5]
+    # the end-of-sequence token stops and is not emitted
+    assert rt.generate(prompt, GenerateOptions(max_new_tokens=16, eos_token_id=want[6])) == want[:want.index(want[6])]
+    assert rt.engine.cache.free_pages() == 16
+
+
+def test_sampled_B_portions_mixed_with_decoding(folders):
+    """Configuration B's workload: prompts of 5, 13 and 29 tokens, portions of 8 beside decoded tokens,
+    temperature 0.7 with a fixed seed, 12 new tokens each, pages of 8.  The engine's tokens must be the
+    plain sampler's tokens on the plain model's logits of the same history."""
+    from infernum_amd import GenerateOptions, SamplingParams
+    d, cfg, w = folders["B"]
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (5, 13, 29)]
+    sp = [SamplingParams(temperature=0.7, top_p=0.9, seed=100 + i, repetition_penalty=1.1,
+                         repetition_penalty_window=8) for i in range(3)]
+    rt = _runtime(d, "float32", block_size=8, num_blocks=24, max_batch_size=3, max_prefill_tokens=8,
+                  max_tokens_per_step=16)
+    sizes, real_step = [], rt.engine.step
+    rt.engine.step = lambda entries: (sizes.append(sorted(len(e.tokens) for e in entries)), real_step(entries))[1]
+    got = rt.generate_batch(prompts, [GenerateOptions(max_new_tokens=12, sampling=s) for s in sp])
+    assert any(e[0] == 1 and e[-1] > 1 for e in sizes), f"no step mixed decoded tokens with a portion: {sizes}"
+    assert max(sum(e) for e in sizes) <= 16 and max(max(e) for e in sizes) <= 8
+    for p, s, out in zip(prompts, sp, got):
+        assert len(out) == 12
+        toks = list(p)
+        for i, t in enumerate(out):
+            logits = P.forward(cfg, w, toks)[-1]
+            u = P.uniform_for_token(s.seed, i)
+            want = P.sample_token(logits, s.temperature, s.top_p, u, s.repetition_penalty, toks[-8:])
+            assert want == t, f"request with seed {s.seed}: token {i} is {t}, the plain sampler gives {want}"
+            toks.append(t)
+
+
+def test_too_few_pages_changes_no_greedy_token(folders):
+    from infernum_amd import GenerateOptions
+    d, cfg, w = folders["A"]
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, 256, (n,), generator=g).tolist() for n in (9, 17, 6, 12)]
+    want = [P.greedy(cfg, w, p, 20) for p in prompts]
+    roomy = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=4, max_prefill_tokens=8)
+    assert roomy.generate_batch(prompts, GenerateOptions(max_new_tokens=20)) == want
+    tight = _runtime(d, "float32", block_size=4, num_blocks=18, max_batch_size=4, max_prefill_tokens=8)
+    seqs = [tight.submit(p, GenerateOptions(max_new_tokens=20)) for p in prompts]
+    n_back = 0
+    while not tight.scheduler.is_idle():
+        n_back += len(tight.step().set_back)
+    assert [s.generated_ids for s in seqs] == want
+    assert n_back > 0, "the pool was meant to run out"
+    tight.scheduler.reap(tight.engine.cache)
+    tight.engine.cache.check()
+    assert tight.engine.cache.free_pages() == 18
+
+
+def test_bfloat16_generation_runs_and_mostly_agrees(folders):
+    from infernum_amd import GenerateOptions
+    d, cfg, w = folders["B"]
+    prompt = list(range(40, 60))
+    want = P.greedy(cfg, w, prompt, 8)
+    got = _runtime(d, "bfloat16", block_size=8, num_blocks=16, max_batch_size=2).generate(
+        prompt, GenerateOptions(max_new_tokens=8))
+    assert len(got) == 8 and got[0] == want[0]
+
+
+def test_command_line(folders):
+    d, cfg, w = folders["A"]
+    prompt = [3, 141, 59, 26, 53, 58, 97]
+    want = P.greedy(cfg, w, prompt, 6)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), "-m", d, "--greedy", "-n", "6",
+                           "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)), "--max-seq-len", "64"],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert "Decoding: greedy (argmax)" in proc.stdout and "KV cache: enabled" in proc.stdout
+    assert " ".join(map(str, want)) in proc.stdout
+    assert "Generated 6 tokens in" in proc.stdout
