@@ -13,7 +13,6 @@ int32 buffer, copies it to the device once, and runs the model's forward pass.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
@@ -23,26 +22,11 @@ from ..cache import CacheConfig, CacheManager
 from ..models.model import DecoderModel
 from ..parts.base import Runtime, StepContext
 
-PREFILL_TILE_ROWS = 64      # query rows per workgroup of the tiled prefill attention
+from .batch import PackedStep, StepEntry, StepError, check_entries, pack_step
 
 
 class OutOfPages(RuntimeError):
     """The pool has too few free pages (or state slots) for this step; nothing was changed."""
-
-
-class StepError(ValueError):
-    """A step's entries are malformed (unknown place wanted, token outside the vocabulary, ...)."""
-
-
-@dataclass
-class StepEntry:
-    request: Hashable
-    tokens: Sequence[int]
-    want: Sequence[int] = field(default_factory=list)     # places among ``tokens`` whose logits are wanted
-
-
-def _align4(n: int) -> int:
-    return (n + 3) & ~3
 
 
 class Engine:
@@ -120,20 +104,9 @@ class Engine:
         V = self.spec.vocab_size
         if not entries:
             return torch.empty((0, V), dtype=torch.float32, device=self.rt.device)
-        seen = set()
-        for e in entries:
-            if e.request in seen:
-                raise StepError(f"request {e.request!r} stands twice in one step")
-            seen.add(e.request)
-            if len(e.tokens) == 0:
-                raise StepError(f"request {e.request!r} brings no tokens")
-            for w in e.want:
-                if not 0 <= w < len(e.tokens):
-                    raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
-        total = sum(len(e.tokens) for e in entries)
-        if total > self.rt.max_tokens_per_step:
-            raise StepError(f"a step of {total} tokens is above max_tokens_per_step {self.rt.max_tokens_per_step}")
+        check_entries(entries, V, self.rt.max_tokens_per_step)
         if self.pages_short(entries):
+            total = sum(len(e.tokens) for e in entries)
             raise OutOfPages(f"not enough free pages or state slots for a step of {total} tokens")
         cache = self.cache
         for e in entries:
@@ -141,63 +114,10 @@ class Engine:
                 cache.admit(e.request)
             ok = cache.reserve(e.request, len(e.tokens))
             assert ok
-
-        # single tokens first, portions of prompts after them
-        order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
-        batch = [entries[i] for i in order]
-        B = len(batch)
-        num_decode = sum(1 for e in batch if len(e.tokens) == 1)
-        q_lens = [len(e.tokens) for e in batch]
-        ctx_lens = [cache.num_tokens(e.request) for e in batch]
-        starts = np.zeros(B + 1, dtype=np.int32)
-        starts[1:] = np.cumsum(q_lens)
-        N = int(starts[-1])
-        start_of = {e.request: int(starts[i]) for i, e in enumerate(batch)}
-
-        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in batch])
-        if token_ids.min() < 0 or token_ids.max() >= V:
-            raise StepError(f"token id outside the vocabulary [0, {V})")
-        positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(ctx_lens, q_lens)])
-        token_seq = np.repeat(np.arange(B, dtype=np.int32), q_lens)
-        logit_rows = np.asarray([start_of[e.request] + w for e in entries for w in e.want], dtype=np.int32)
-        state_slots = np.asarray([cache.state_slot(e.request) for e in batch], dtype=np.int32)
-        reqs = [e.request for e in batch]
-        tiles = [(s, r) for s in range(num_decode, B) for r in range(0, q_lens[s], PREFILL_TILE_ROWS)]
-        tiles_np = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
-
-        segs: List[np.ndarray] = [token_ids.astype(np.int32), positions, token_seq, starts,
-                                  np.asarray(ctx_lens, dtype=np.int32), state_slots, logit_rows, tiles_np.reshape(-1)]
-        bt_shapes = []
-        for g in cache.groups:
-            bt = cache.block_table_rows(g.index, reqs)
-            bt_shapes.append(bt.shape)
-            segs.append(np.concatenate([cache.token_slots(g.index, r, c, q)
-                                        for r, c, q in zip(reqs, ctx_lens, q_lens)]))
-            segs.append(bt.reshape(-1))
-        offs, total_ints = [], 0
-        for s in segs:
-            offs.append(total_ints)
-            total_ints += _align4(max(s.size, 1))
-        host = np.zeros(total_ints, dtype=np.int32)
-        for o, s in zip(offs, segs):
-            host[o:o + s.size] = s
-        dev = torch.from_numpy(host).to(self.rt.device)
-
-        def seg(i: int) -> torch.Tensor:
-            return dev[offs[i]:offs[i] + segs[i].size]
-
-        ctx = StepContext(
-            num_tokens=N, num_seqs=B, num_decode=num_decode,
-            token_ids=seg(0), positions=seg(1), token_seq=seg(2), seq_starts=seg(3), seq_ctx=seg(4),
-            state_slots=seg(5), logit_rows=seg(6),
-            block_tables=[seg(9 + 2 * gi).view(bt_shapes[gi]) for gi in range(len(cache.groups))],
-            slots=[seg(8 + 2 * gi) for gi in range(len(cache.groups))],
-            q_lens=q_lens, ctx_lens=ctx_lens, max_q_len=max(q_lens),
-            max_total_len=max(c + q for c, q in zip(ctx_lens, q_lens)),
-            prefill_tiles=seg(7).view(-1, 2), num_prefill_tiles=len(tiles),
-        )
+        packed = pack_step(cache, entries)
+        ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
         logits = self.model.forward(ctx, self.views)
-        for e in batch:
+        for e in packed.batch:
             cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
         return logits

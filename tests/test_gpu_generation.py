@@ -45,6 +45,19 @@ def test_greedy_A_through_the_entry_point(folders):
     assert rt.engine.cache.free_pages() == 16
 
 
+@pytest.mark.parametrize("dtype", ["float32"])
+def test_greedy_B_varied_tokens(folders, dtype):
+    """A's tied head mostly repeats the last token; B's separate head gives a varied continuation,
+    which a fault in the cache or the positions would change."""
+    from infernum_amd import GenerateOptions
+    d, cfg, w = folders["B"]
+    prompt = [3, 141, 59, 26, 53, 58, 97]
+    want = P.greedy(cfg, w, prompt, 24)
+    assert len(set(want)) >= 5
+    rt = _runtime(d, dtype, block_size=8, num_blocks=8, max_batch_size=2, max_prefill_tokens=4)
+    assert rt.generate(prompt, GenerateOptions(max_new_tokens=24)) == want
+
+
 def test_sampled_B_portions_mixed_with_decoding(folders):
     """Configuration B's workload: prompts of 5, 13 and 29 tokens, portions of 8 beside decoded tokens,
     temperature 0.7 with a fixed seed, 12 new tokens each, pages of 8.  The engine's tokens must be the

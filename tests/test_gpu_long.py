@@ -1,0 +1,70 @@
+"""Long decoding and the first tokens of a sequence, against the plain implementation."""
+import pytest
+import torch
+
+import plain_llama as P
+import tiny_models as TM
+import trace_tools as TT
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": 2e-5, "bfloat16": 6e-2}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name in ("B", "C"):
+        for dt, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+            d = str(tmp_path_factory.mktemp(f"long{name}_{dt}"))
+            TM.write_tiny(name, d, dtype=tdt)
+            out[(name, dt)] = (d,) + P.read_model(d)
+    return out
+
+
+def _engine(d, dtype, ps, pages):
+    from infernum_amd import CacheConfig, Engine
+    return Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=ps, num_pages=pages,
+                                                                           num_state_slots=4, poison_freed_pages=True))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,ps", [("B", 8), ("C", 16)])
+def test_long_decoding(models, name, ps, dtype):
+    """A prompt of 20 tokens, then 400 tokens one by one: many pages, many splits of the keys, and (C)
+    a window that has long passed the first pages."""
+    d, cfg, w = models[(name, dtype)]
+    reqs = TT.make_requests(cfg["vocab_size"], (420,), seed=31)
+    ref = {r: P.forward(cfg, w, t) for r, t in reqs.items()}
+    steps = TT.trace_tail_one_by_one(reqs, tail=400)
+    assert len(steps) == 401
+    eng = _engine(d, dtype, ps, 64)
+    got = TT.run_steps(eng, steps)
+    worst, rms, where = TT.error_against(got, ref)
+    print(f"{name} {dtype} long decoding: {worst / rms:.2e} at {where}")
+    assert worst == worst and worst <= TOL[dtype] * rms, (worst / rms, where)
+    eng.cache.check()
+    assert all(g.allocator.num_free == 64 for g in eng.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_first_tokens(models, name, dtype):
+    """Position 0 sees itself only; prompts of one and of two tokens; the second token decoded."""
+    d, cfg, w = models[(name, dtype)]
+    from infernum_amd import StepEntry
+    eng = _engine(d, dtype, 8, 8)
+    toks = [17, 201, 5, 99]
+    ref = P.forward(cfg, w, toks)
+    rms = ref.pow(2).mean().sqrt().item()
+
+    def close(row, p):
+        return (row.double().cpu() - ref[p]).abs().max().item() <= TOL[dtype] * rms
+    one = eng.step([StepEntry("a", toks[:1], [0])])
+    assert close(one[0], 0)
+    nxt = eng.step([StepEntry("a", toks[1:2], [0])])
+    assert close(nxt[0], 1)
+    two = eng.step([StepEntry("b", toks[:2], [0, 1]), StepEntry("a", toks[2:3], [0])])
+    assert close(two[0], 0) and close(two[1], 1) and close(two[2], 2)
+    # a token's logits at position 0 are those of a sequence of that token alone
+    alone = P.forward(cfg, w, toks[:1])[0]
+    assert (one[0].double().cpu() - alone).abs().max().item() <= TOL[dtype] * rms

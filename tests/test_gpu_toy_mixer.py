@@ -1,0 +1,189 @@
+"""A mixer that the framework does not know, with per-request state of its own, defined here,
+registered, built into a model beside attention layers, loaded from a model folder and stepped:
+without a change to the framework's files.  The schedule names layers twice and lets one run read
+another run's cache."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import plain_llama as P
+import trace_tools as TT
+from infernum_amd import CacheConfig, Engine, register_architecture, register_part
+from infernum_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleEntry, StateSpec, WeightSpec)
+from infernum_amd.weights import write_random_model
+
+pytestmark = pytest.mark.gpu
+
+
+class EmaMixer(Mixer):
+    """s_t = decay * s_{t-1} + W_in x_t (per request, s_{-1} = 0);  y_t = W_out s_t.
+    The state s has a fixed size; it lives in the cache manager's state slots."""
+
+    def __init__(self, rt, hidden_size, state_size):
+        super().__init__(rt)
+        self.H, self.S = hidden_size, state_size
+
+    def state_spec(self):
+        return StateSpec((self.S,))
+
+    def weights(self):
+        return {"in_proj.weight": WeightSpec((self.S, self.H), ("normal", 0.2)),
+                "out_proj.weight": WeightSpec((self.H, self.S), ("normal", 0.2)),
+                "decay": WeightSpec((self.S,), ("uniform", 0.5, 0.95), follows_compute_dtype=False)}
+
+    def load(self, tensors):
+        self.w_in, self.w_out, self.decay = tensors["in_proj.weight"], tensors["out_proj.weight"], tensors["decay"]
+
+    def forward(self, x, ctx, cache):
+        assert cache.state is not None and cache.k_pages is None
+        u = (x.float() @ self.w_in.float().t())
+        s_all = torch.empty_like(u)
+        slots = ctx.state_slots.tolist()
+        row = 0
+        for b, n in enumerate(ctx.q_lens):
+            s = cache.state[slots[b]]
+            for _ in range(n):
+                s = self.decay.float() * s + u[row]
+                s_all[row] = s
+                row += 1
+            cache.state[slots[b]] = s
+        return (s_all @ self.w_out.float().t()).to(x.dtype)
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    vocab_size: int = 90
+    hidden_size: int = 48
+    state_size: int = 20
+    num_heads: int = 3
+    num_kv_heads: int = 1
+    intermediate_size: int = 72
+    eps: float = 1e-5
+    theta: float = 1000.0
+    model_type: str = "toy-ema"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return ToyConfig(**{k: v for k, v in raw.items() if k in ToyConfig.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+SCHEDULE = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_of=0), ScheduleEntry(1), ScheduleEntry(2)]
+
+
+def toy_spec(cfg: ToyConfig) -> ModelSpec:
+    H, d = cfg.hidden_size, cfg.hidden_size // cfg.num_heads
+    norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": cfg.eps, "init": ("uniform", 0.5, 1.5)}, prefix)
+    ff = lambda prefix: PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size,
+                                            "init_std": 0.1}, prefix)
+    att = lambda prefix, window: PartSpec("attention", {
+        "hidden_size": H, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads, "head_dim": d,
+        "window": window, "init_std": 0.1,
+        "position": {"kind": "rope", "params": {"head_dim": d, "theta": cfg.theta, "scaling": None}}}, prefix)
+    ema = lambda prefix: PartSpec("ema", {"hidden_size": H, "state_size": cfg.state_size}, prefix)
+    layers = []
+    for i, mixer in enumerate([att("layers.0.attn.", None), ema("layers.1.ema."), att("layers.2.attn.", 9)]):
+        layers.append(LayerSpec("prenorm", mixer, ff(f"layers.{i}.ff."), norm(f"layers.{i}.norm1."),
+                                norm(f"layers.{i}.norm2.")))
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.5},
+                                        "embed."),
+                     layers=layers, schedule=SCHEDULE, final_norm=norm("final_norm."),
+                     head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.1}, "head."))
+
+
+def plain_forward(cfg: ToyConfig, w, ids):
+    """The toy model on a whole sequence, from the plain functions."""
+    W = {k: v.double() for k, v in w.items()}
+    H, nh, nkv = cfg.hidden_size, cfg.num_heads, cfg.num_kv_heads
+    d = H // nh
+    T = len(ids)
+    freqs, pos = P.rope_frequencies(d, cfg.theta, None), torch.arange(T)
+    h = P.embedding(W["embed.weight"], ids)
+    kept = {}
+    for e_idx, e in enumerate(SCHEDULE):
+        i = e.layer
+        n = P.rms_norm(h, W[f"layers.{i}.norm1.weight"], cfg.eps)
+        if i == 1:
+            p = "layers.1.ema."
+            u = P.linear(n, W[p + "in_proj.weight"])
+            s, rows = torch.zeros(cfg.state_size, dtype=torch.float64), []
+            for t in range(T):
+                s = W[p + "decay"] * s + u[t]
+                rows.append(s)
+            a = P.linear(torch.stack(rows), W[p + "out_proj.weight"])
+        else:
+            p = f"layers.{i}.attn."
+            q = P.rope(P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d), pos, freqs)
+            if e.cache_of is None:
+                k = P.rope(P.linear(n, W[p + "k_proj.weight"]).reshape(T, nkv, d), pos, freqs)
+                v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, nkv, d)
+                kept[e_idx] = (k, v)
+            else:
+                k, v = kept[e.cache_of]
+            a = P.linear(P.causal_attention(q, k, v, 1.0 / math.sqrt(d), 9 if i == 2 else None).reshape(T, H),
+                         W[p + "o_proj.weight"])
+        h = h + a
+        m = P.rms_norm(h, W[f"layers.{i}.norm2.weight"], cfg.eps)
+        h = h + P.linear(P.swiglu(P.linear(m, W[f"layers.{i}.ff.gate_proj.weight"]),
+                                  P.linear(m, W[f"layers.{i}.ff.up_proj.weight"])),
+                         W[f"layers.{i}.ff.down_proj.weight"])
+    return P.linear(P.rms_norm(h, W["final_norm.weight"], cfg.eps), W["head.weight"])
+
+
+@pytest.fixture(scope="module")
+def toy(tmp_path_factory):
+    register_part("mixer", "ema", EmaMixer, replace=True)
+    register_architecture("toy-ema", ToyConfig, toy_spec, replace=True)
+    out = {}
+    for dt, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        d = str(tmp_path_factory.mktemp(f"toy_{dt}"))
+        write_random_model(ToyConfig(), d, seed=4, dtype=tdt)
+        out[dt] = d
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_model_is_registered_built_loaded_and_stepped(toy, dtype):
+    d = toy[dtype]
+    cfg = ToyConfig()
+    _, w = P.read_model(d)
+    assert "layers.1.ema.decay" in w
+    eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=4, num_pages=48,
+                                                                          num_state_slots=4, poison_freed_pages=True))
+    assert eng.config == cfg
+    kinds = [type(b.mixer).__name__ for b in eng.model.blocks]
+    assert kinds == ["Attention", "EmaMixer", "Attention"]
+    # groups: all keys (layer 0), a window of 9 (layer 2); the ema runs have state and no pages
+    assert len(eng.cache.groups) == 2
+    assert [v.state is not None for v in eng.views] == [False, True, False, True, False]
+    assert eng.views[2].writable is False and eng.views[2].k_pages is eng.views[0].k_pages
+    reqs = TT.make_requests(cfg.vocab_size, (37, 5, 60, 23), seed=2)
+    ref = {r: plain_forward(cfg, w, t) for r, t in reqs.items()}
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 16)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=1)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+        eng.cache.check()
+        assert eng.cache.slots.num_free == 4 and all(g.allocator.num_free == 48 for g in eng.cache.groups)
+
+
+def test_state_slot_is_zeroed_when_taken_again(toy):
+    """A request that takes the slot of a finished one must not see its state."""
+    eng = Engine.from_pretrained(toy["float32"], dtype="float32",
+                                 cache_config=CacheConfig(page_size=4, num_pages=16, num_state_slots=1))
+    from infernum_amd import StepEntry
+    a = eng.step([StepEntry("a", [1, 2, 3, 4, 5], [4])]).cpu()
+    eng.end("a")
+    eng.step([StepEntry("b", [9, 8, 7, 6, 5, 4, 3], [])])
+    eng.end("b")
+    again = eng.step([StepEntry("c", [1, 2, 3, 4, 5], [4])]).cpu()
+    assert torch.equal(a, again)
