@@ -87,3 +87,31 @@ def random_weights_on_device(model, seed: int) -> None:
         if name not in tensors:
             tensors[name] = tensors[spec.fallback]
     model.load_weights(tensors)
+
+
+def main(argv: Optional[list] = None) -> int:
+    """python -m infernum_amd.weights.random_init --config CONFIG.json --seed S --out DIR [--dtype bfloat16|float32]"""
+    import argparse
+    from ..config.registry import config_from_dict
+    from ..config.base import read_config_json
+    from .. import models  # noqa: F401  (registers the architectures)
+    ap = argparse.ArgumentParser(prog="random_init", description="write a model folder (config.json, "
+                                 "model.safetensors) with random weights from a configuration and a seed")
+    ap.add_argument("--config", required=True, help="a config.json (or a folder that holds one)")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--out", required=True)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--norm-init", default="ones", choices=["ones", "uniform"],
+                    help="norm weights: 1.0, or uniform in [0.5, 1.5]")
+    a = ap.parse_args(argv)
+    config = config_from_dict(read_config_json(a.config), where=a.config)
+    kw = {"norm_init": ("uniform", 0.5, 1.5)} if a.norm_init == "uniform" else {}
+    out = write_random_model(config, a.out, a.seed, {"bfloat16": torch.bfloat16, "float32": torch.float32}[a.dtype],
+                             **kw)
+    print(f"wrote {out}")
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(main())
