@@ -197,27 +197,45 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_kernel(
   }
 }
 
-// Joins the parts of a split: grid (B * nh), 64 threads; parts are taken in the order of their index.
+// Joins the parts of a split: grid (B * nh), 64 threads; parts are added in the order of their index.
+// Lane s holds the weight of part s (of parts s, s + 64, ... in turn), so the statistics are read once and
+// the loads of the partial outputs do not wait for each other.
 extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, uint16_t* __restrict__ out,
     int out_row_stride, int nh, int num_splits) {
-  const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+  const int b = blockIdx.x / nh, h = blockIdx.x - b * nh, lane = threadIdx.x;
   const size_t rec0 = (size_t)blockIdx.x * num_splits;
   float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, part_ml[(rec0 + s) * 2]);
+  for (int s = lane; s < num_splits; s += 64) M = fmaxf(M, part_ml[(rec0 + s) * 2]);
+  M = wave_max(M);
+  float acc[(HD + 63) / 64];
+#pragma unroll
+  for (int c = 0; c < (HD + 63) / 64; ++c) acc[c] = 0.f;
   float L = 0.f;
-  for (int s = 0; s < num_splits; ++s) {
-    const float ms = part_ml[(rec0 + s) * 2];
-    L += (ms == -INFINITY ? 0.f : exp2f(ms - M)) * part_ml[(rec0 + s) * 2 + 1];
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {
+    const int s = s0 + lane;
+    float wgt = 0.f, wl = 0.f;
+    if (s < num_splits) {
+      const float ms = part_ml[(rec0 + s) * 2];
+      wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - M);
+      wl = wgt * part_ml[(rec0 + s) * 2 + 1];
+    }
+    const int cnt = (num_splits - s0) < 64 ? (num_splits - s0) : 64;
+    for (int j = 0; j < cnt; ++j) {
+      L += __shfl(wl, j, IA_WAVE);
+      const float wj = __shfl(wgt, j, IA_WAVE);
+#pragma unroll
+      for (int c = 0; c < (HD + 63) / 64; ++c) {
+        const int dim = lane + 64 * c;
+        if (dim < HD && wj != 0.f) acc[c] += wj * part_o[(rec0 + s0 + j) * HD + dim];
+      }
+    }
   }
   const float inv = 1.0f / L;
-  for (int dim = threadIdx.x; dim < HD; dim += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-      const float ms = part_ml[(rec0 + s) * 2];
-      if (ms != -INFINITY) acc += exp2f(ms - M) * part_o[(rec0 + s) * HD + dim];
-    }
-    out[(size_t)b * out_row_stride + (size_t)h * HD + dim] = float_to_bf16_bits(acc * inv);
+#pragma unroll
+  for (int c = 0; c < (HD + 63) / 64; ++c) {
+    const int dim = lane + 64 * c;
+    if (dim < HD) out[(size_t)b * out_row_stride + (size_t)h * HD + dim] = float_to_bf16_bits(acc[c] * inv);
   }
 }
 

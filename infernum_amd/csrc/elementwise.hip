@@ -35,50 +35,167 @@ extern "C" int ia_embed(const void* table, int table_dtype, const int* ids, floa
 }
 
 // ------------------------------------------------------- add + RMSNorm
-// s = h[src] + delta[src]   (fp32; stored back into h unless `rows` selects rows)
+// s = h[src] + sum_k delta[k][src]   (fp32; stored back into h unless `rows` selects rows)
 // out[row] = s * (1 / sqrt(mean(s^2) + eps)) * w
 // `rows` (nullable) picks the source rows; then h is left unchanged.
-template <typename T>
-__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+// delta (nullable) is [splits, n_rows, H]: one tensor in the activations' dtype, or a stack of fp32
+// partial sums that a split matrix product left; the splits are added in the order of their index.
+//
+// Scalar kernel: any H.
+template <typename TD, typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                          int splits, size_t split_stride,
                                                           const void* __restrict__ w, int w_dtype,
-                                                          T* __restrict__ out, const int* __restrict__ rows, int H,
+                                                          TO* __restrict__ out, const int* __restrict__ rows, int H,
                                                           float eps) {
   __shared__ float red[4];
   const int row = blockIdx.x;
   const int src = rows ? rows[row] : row;
   float* hr = h + (size_t)src * H;
-  const T* dr = delta ? delta + (size_t)src * H : nullptr;
+  const TD* dr = delta ? delta + (size_t)src * H : nullptr;
   const bool store = (rows == nullptr) && (delta != nullptr);
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += 256) {
     float s = hr[i];
-    if (dr) s += to_float(dr[i]);
+    if (dr) {
+      float d = 0.f;
+      for (int k = 0; k < splits; ++k) d += to_float(dr[k * split_stride + i]);
+      s += d;
+    }
     if (store) hr[i] = s;
     ss += s * s;
   }
   ss = block_sum<256>(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-  T* o = out + (size_t)row * H;
+  TO* o = out + (size_t)row * H;
   for (int i = threadIdx.x; i < H; i += 256) {
     float s = hr[i];
-    if (dr && !store) s += to_float(dr[i]);
-    o[i] = from_float<T>(s * inv * load_as_float(w, w_dtype, i));
+    if (dr && !store) {
+      float d = 0.f;
+      for (int k = 0; k < splits; ++k) d += to_float(dr[k * split_stride + i]);
+      s += d;
+    }
+    o[i] = from_float<TO>(s * inv * load_as_float(w, w_dtype, i));
   }
 }
 
-extern "C" int ia_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* w, int w_dtype, void* out,
-                              const int* rows, int N, int H, float eps, hipStream_t stream) {
-  if (N < 0 || H <= 0 || !(eps > 0.f)) return IA_ERR_BAD_ARG;
-  if (N == 0) return IA_OK;
-  if (act_dtype == IA_F32)
-    add_rmsnorm_kernel<float><<<N, 256, 0, stream>>>(h, (const float*)delta, w, w_dtype, (float*)out, rows, H, eps);
-  else if (act_dtype == IA_BF16)
-    add_rmsnorm_kernel<bf16_t><<<N, 256, 0, stream>>>(h, (const bf16_t*)delta, w, w_dtype, (bf16_t*)out, rows, H,
-                                                       eps);
-  else
-    return IA_ERR_BAD_ARG;
+// Four consecutive values of a row as floats.
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ float4 load4_any(const void* p, int dtype, int i) {
+  return dtype == IA_F32 ? load4((const float*)p + i) : load4((const bf16_t*)p + i);
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16);
+  u.y = (uint32_t)float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+// Vector kernel: H a multiple of 4 and at most NT * 4 * RN_MAXV.  Every thread keeps its part of the row in
+// registers (16-byte loads, all issued before the first use), so the row is read once and no load waits for
+// another.  Sums are taken in the same order whatever the batch: a row's result depends on the row alone.
+#define RN_MAXV 4
+template <typename TD, typename TO, int NT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                             int splits, size_t split_stride,
+                                                             const void* __restrict__ w, int w_dtype,
+                                                             TO* __restrict__ out, const int* __restrict__ rows,
+                                                             int H, float eps) {
+  __shared__ float red[NT / 64];
+  const int row = blockIdx.x;
+  const int src = rows ? rows[row] : row;
+  float* hr = h + (size_t)src * H;
+  const TD* dr = delta ? delta + (size_t)src * H : nullptr;
+  const bool store = (rows == nullptr) && (delta != nullptr);
+  float4 v[RN_MAXV];
+#pragma unroll
+  for (int c = 0; c < RN_MAXV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    v[c] = (i < H) ? load4(hr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  if (dr) {
+    float4 ds[RN_MAXV];
+#pragma unroll
+    for (int c = 0; c < RN_MAXV; ++c) ds[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < splits; ++k) {
+#pragma unroll
+      for (int c = 0; c < RN_MAXV; ++c) {
+        const int i = (threadIdx.x + c * NT) * 4;
+        if (i < H) {
+          const float4 d = load4(dr + k * split_stride + i);
+          ds[c].x += d.x; ds[c].y += d.y; ds[c].z += d.z; ds[c].w += d.w;
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < RN_MAXV; ++c) { v[c].x += ds[c].x; v[c].y += ds[c].y; v[c].z += ds[c].z; v[c].w += ds[c].w; }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < RN_MAXV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    if (i < H) {
+      if (store) store4(hr + i, v[c]);
+      ss += (v[c].x * v[c].x + v[c].y * v[c].y) + (v[c].z * v[c].z + v[c].w * v[c].w);
+    }
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)row * H;
+#pragma unroll
+  for (int c = 0; c < RN_MAXV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    if (i < H) {
+      const float4 g = load4_any(w, w_dtype, i);
+      store4(o + i, make_float4(v[c].x * inv * g.x, v[c].y * inv * g.y, v[c].z * inv * g.z, v[c].w * inv * g.w));
+    }
+  }
+}
+
+template <typename TD, typename TO>
+static int launch_add_rmsnorm(float* h, const void* delta, int splits, size_t split_stride, const void* w, int w_dtype,
+                              void* out, const int* rows, int N, int H, float eps, hipStream_t stream) {
+  const TD* d = (const TD*)delta;
+  TO* o = (TO*)out;
+  if ((H & 3) == 0 && H <= 1024 * 4 * RN_MAXV) {
+    // wide rows: 1024 threads, one to four 16-byte pieces each.  The choice depends on H alone, so a row's
+    // sums are taken in the same order whatever the batch holds.
+    if (H >= 2048)
+      add_rmsnorm_vec_kernel<TD, TO, 1024><<<N, 1024, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o, rows,
+                                                                    H, eps);
+    else
+      add_rmsnorm_vec_kernel<TD, TO, 256><<<N, 256, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o, rows, H,
+                                                                  eps);
+  } else {
+    add_rmsnorm_kernel<TD, TO><<<N, 256, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o, rows, H, eps);
+  }
   IA_LAUNCH_CHECK();
   return IA_OK;
+}
+
+// delta_dtype: dtype of delta (IA_F32 for a stack of partial sums in the bf16 path); act_dtype: dtype of out.
+// delta is [splits, delta_rows, H].
+extern "C" int ia_add_rmsnorm(float* h, const void* delta, int delta_dtype, int splits, int delta_rows,
+                              int act_dtype, const void* w, int w_dtype, void* out, const int* rows, int N, int H,
+                              float eps, hipStream_t stream) {
+  if (N < 0 || H <= 0 || !(eps > 0.f)) return IA_ERR_BAD_ARG;
+  if (delta && (splits < 1 || delta_rows < 0)) return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  const size_t stride = (size_t)delta_rows * H;
+  if (!delta) delta_dtype = act_dtype;
+  if (act_dtype == IA_F32 && delta_dtype == IA_F32)
+    return launch_add_rmsnorm<float, float>(h, delta, splits, stride, w, w_dtype, out, rows, N, H, eps, stream);
+  if (act_dtype == IA_BF16 && delta_dtype == IA_BF16)
+    return launch_add_rmsnorm<bf16_t, bf16_t>(h, delta, splits, stride, w, w_dtype, out, rows, N, H, eps, stream);
+  if (act_dtype == IA_BF16 && delta_dtype == IA_F32)
+    return launch_add_rmsnorm<float, bf16_t>(h, delta, splits, stride, w, w_dtype, out, rows, N, H, eps, stream);
+  return IA_ERR_BAD_ARG;
 }
 
 // h[n, :] += delta[n, :] without a norm (used when a model ends without one).
@@ -105,83 +222,107 @@ extern "C" int ia_residual_add(float* h, const void* delta, int act_dtype, int N
 }
 
 // ------------------------------------------- rotary + write of K/V pages
-// Row n of qkv (row_stride elements apart) holds [nh q heads | nkv k heads |
-// nkv v heads], each of d values; with write_kv == 0 only the q heads are read.
-// The first `rot` values of every q and k head are rotated in half-split pairs
-// (x[i], x[i + rot/2]) by the angle pos * inv_freq[i], computed in fp32.
-// q is rotated in place; rotated k and raw v go to the page slot of the token:
-// key pages are [num_pages, nkv, page_size, d]; value pages are stored transposed,
-// [num_pages, nkv, d, page_size], which is the layout the matrix cores want for
-// the product of probabilities and values; slot = page * page_size + offset.
-// inv_freq == nullptr: no rotation.  slot < 0 or write_kv == 0: nothing is written.
-template <typename T>
-__global__ __launch_bounds__(256) void rope_kv_append_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+// Row n of src holds [nh q heads | nkv k heads | nkv v heads], each of d values; with write_kv == 0 only
+// the q heads are read.  src is [splits, N, row_stride]: one tensor in the activations' dtype, or a stack
+// of fp32 partial sums of a split matrix product (added in the order of their index).
+// The first `rot` values of every q and k head are rotated in half-split pairs (x[i], x[i + rot/2]) by the
+// angle pos * inv_freq[i], computed in fp32 (one sincos per thread, used for all its heads).
+// Rotated q goes to q_out (row stride q_stride; it may be src itself: rotation in place); rotated k and raw
+// v go to the page slot of the token: key pages are [num_pages, nkv, page_size, d]; value pages are stored
+// transposed, [num_pages, nkv, d, page_size], the layout the matrix cores want for the product of
+// probabilities and values; slot = page * page_size + offset.
+// inv_freq == nullptr: no rotation.  slot < 0 or write_kv == 0: nothing is written to pages.
+template <typename TS>
+__device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t split_stride) {
+  float v = to_float(p[0]);
+  for (int k = 1; k < splits; ++k) v += to_float(p[k * split_stride]);
+  return v;
+}
+
+template <typename TS, typename T>
+__global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restrict__ src, int splits,
+                                                             size_t split_stride, T* __restrict__ q_out,
+                                                             int q_stride, const int* __restrict__ positions,
                                                              const int* __restrict__ slots,
                                                              const float* __restrict__ inv_freq,
                                                              T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                              int row_stride, int nh, int nkv, int d, int rot,
-                                                             int page_size, int num_pages, int write_kv) {
+                                                             int page_size, int num_pages, int write_kv,
+                                                             int copy_q_tail, int lanes_per_head) {
   const int n = blockIdx.x;
   const float pos = (float)positions[n];
-  T* row = qkv + (size_t)n * row_stride;
+  const TS* row = src + (size_t)n * row_stride;
+  T* qrow = q_out + (size_t)n * q_stride;
   const int slot = (write_kv && slots) ? slots[n] : -1;
   const bool do_write = slot >= 0 && slot < num_pages * page_size;
   const int page = do_write ? slot / page_size : 0;
   const int off = do_write ? slot % page_size : 0;
   const int half = rot >> 1;
   const int rot_heads = nh + (do_write ? nkv : 0);
-  const int pairs = rot_heads * half;
-  for (int idx = threadIdx.x; idx < pairs; idx += 256) {
-    const int head = idx / half, i = idx - head * half;
-    T* x = row + (size_t)head * d;
-    const float a = to_float(x[i]), b = to_float(x[i + half]);
-    float o1 = a, o2 = b;
-    if (inv_freq) {
-      float s, c;
-      sincosf(pos * inv_freq[i], &s, &c);
-      o1 = a * c - b * s;
-      o2 = a * s + b * c;
-    }
-    if (head < nh) {
-      x[i] = from_float<T>(o1);
-      x[i + half] = from_float<T>(o2);
-    } else {
-      T* dst = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
-      dst[i] = from_float<T>(o1);
-      dst[i + half] = from_float<T>(o2);
+  // thread = (head group hg, pair i): lanes_per_head is a power of two that covers `half` (at most 256)
+  const int i0 = threadIdx.x % lanes_per_head, hg = threadIdx.x / lanes_per_head, HG = 256 / lanes_per_head;
+  for (int i = i0; i < half; i += lanes_per_head) {
+    float sn = 0.f, cs = 1.f;
+    if (inv_freq) sincosf(pos * inv_freq[i], &sn, &cs);
+    for (int head = hg; head < rot_heads; head += HG) {
+      const TS* x = row + (size_t)head * d;
+      const float a = load_split_sum(x + i, splits, split_stride);
+      const float b = load_split_sum(x + i + half, splits, split_stride);
+      const float o1 = a * cs - b * sn, o2 = a * sn + b * cs;
+      if (head < nh) {
+        qrow[(size_t)head * d + i] = from_float<T>(o1);
+        qrow[(size_t)head * d + i + half] = from_float<T>(o2);
+      } else {
+        T* dst = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
+        dst[i] = from_float<T>(o1);
+        dst[i + half] = from_float<T>(o2);
+      }
     }
   }
-  if (!do_write) return;
-  // values of k beyond the rotated part, and all of v: plain copies
+  // values beyond the rotated part are plain copies
   const int tail = d - rot;
+  if (copy_q_tail)
+    for (int idx = threadIdx.x; idx < nh * tail; idx += 256) {
+      const int hd = idx / tail, i = rot + (idx - hd * tail);
+      qrow[(size_t)hd * d + i] = from_float<T>(load_split_sum(row + (size_t)hd * d + i, splits, split_stride));
+    }
+  if (!do_write) return;
   for (int idx = threadIdx.x; idx < nkv * tail; idx += 256) {
     const int g = idx / tail, i = rot + (idx - g * tail);
-    k_pages[(((size_t)page * nkv + g) * page_size + off) * d + i] = row[(size_t)(nh + g) * d + i];
+    k_pages[(((size_t)page * nkv + g) * page_size + off) * d + i] =
+        from_float<T>(load_split_sum(row + (size_t)(nh + g) * d + i, splits, split_stride));
   }
   for (int idx = threadIdx.x; idx < nkv * d; idx += 256) {
     const int g = idx / d, i = idx - g * d;
-    v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] = row[(size_t)(nh + nkv + g) * d + i];
+    v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] =
+        from_float<T>(load_split_sum(row + (size_t)(nh + nkv + g) * d + i, splits, split_stride));
   }
 }
 
-extern "C" int ia_rope_kv_append(void* qkv, int act_dtype, const int* positions, const int* slots,
-                                 const float* inv_freq, void* k_pages, void* v_pages, int N, int row_stride, int nh,
-                                 int nkv, int d, int rot, int page_size, int num_pages, int write_kv,
-                                 hipStream_t stream) {
+// src: [splits, src_rows, row_stride] of src_dtype; q_out, pages: act_dtype.
+extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int src_rows, void* q_out, int q_stride,
+                                 int act_dtype, const int* positions, const int* slots, const float* inv_freq,
+                                 void* k_pages, void* v_pages, int N, int row_stride, int nh, int nkv, int d, int rot,
+                                 int page_size, int num_pages, int write_kv, hipStream_t stream) {
   if (N < 0 || nh <= 0 || nkv <= 0 || d <= 0 || rot < 0 || rot > d || (rot & 1)) return IA_ERR_BAD_ARG;
-  if (row_stride < (nh + (write_kv ? 2 * nkv : 0)) * d) return IA_ERR_BAD_ARG;
+  if (row_stride < (nh + (write_kv ? 2 * nkv : 0)) * d || q_stride < nh * d || splits < 1 || src_rows < N)
+    return IA_ERR_BAD_ARG;
   if (write_kv && (page_size <= 0 || num_pages <= 0 || !k_pages || !v_pages || !slots)) return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
-  if (act_dtype == IA_F32)
-    rope_kv_append_kernel<float><<<N, 256, 0, stream>>>((float*)qkv, positions, slots, inv_freq, (float*)k_pages,
-                                                        (float*)v_pages, row_stride, nh, nkv, d, rot, page_size,
-                                                        num_pages, write_kv);
-  else if (act_dtype == IA_BF16)
-    rope_kv_append_kernel<bf16_t><<<N, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, inv_freq, (bf16_t*)k_pages,
-                                                         (bf16_t*)v_pages, row_stride, nh, nkv, d, rot, page_size,
-                                                         num_pages, write_kv);
-  else
-    return IA_ERR_BAD_ARG;
+  if (!inv_freq) rot = 0;
+  const size_t stride = (size_t)src_rows * row_stride;
+  const int copy_q_tail = (src != q_out || splits > 1) ? 1 : 0;
+  int lph = 1;
+  while (lph < (rot >> 1) && lph < 256) lph <<= 1;
+#define ROPE_LAUNCH(TS, T)                                                                                        \
+  rope_kv_append_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, splits, stride, (T*)q_out, q_stride, positions, \
+                                                      slots, inv_freq, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
+                                                      d, rot, page_size, num_pages, write_kv, copy_q_tail, lph)
+  if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_LAUNCH(float, float);
+  else if (act_dtype == IA_BF16 && src_dtype == IA_BF16) ROPE_LAUNCH(bf16_t, bf16_t);
+  else if (act_dtype == IA_BF16 && src_dtype == IA_F32) ROPE_LAUNCH(float, bf16_t);
+  else return IA_ERR_BAD_ARG;
+#undef ROPE_LAUNCH
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
@@ -200,10 +341,35 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T
   out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
 }
 
+// Four values per thread (I a multiple of 4).
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I,
+                                                         size_t total4) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total4) return;
+  const int per_row = I >> 2;
+  const size_t n = idx / per_row;
+  const int i = (int)(idx - n * per_row) << 2;
+  const float4 g = load4(gu + n * 2 * I + i), u = load4(gu + n * 2 * I + I + i);
+  store4(out + n * I + i, make_float4(g.x / (1.0f + expf(-g.x)) * u.x, g.y / (1.0f + expf(-g.y)) * u.y,
+                                      g.z / (1.0f + expf(-g.z)) * u.z, g.w / (1.0f + expf(-g.w)) * u.w));
+}
+
 extern "C" int ia_swiglu(const void* gu, void* out, int act_dtype, int N, int I, hipStream_t stream) {
   if (N < 0 || I <= 0) return IA_ERR_BAD_ARG;
   size_t total = (size_t)N * I;
   if (total == 0) return IA_OK;
+  if (act_dtype != IA_F32 && act_dtype != IA_BF16) return IA_ERR_BAD_ARG;
+  if ((I & 3) == 0) {
+    const size_t total4 = total >> 2;
+    const unsigned grid4 = (unsigned)((total4 + 255) / 256);
+    if (act_dtype == IA_F32)
+      swiglu_vec_kernel<float><<<grid4, 256, 0, stream>>>((const float*)gu, (float*)out, I, total4);
+    else
+      swiglu_vec_kernel<bf16_t><<<grid4, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total4);
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
   unsigned grid = (unsigned)((total + 255) / 256);
   if (act_dtype == IA_F32)
     swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);

@@ -1,15 +1,25 @@
 // C[M, N] = X[M, K] * W[N, K]^T in bf16 with fp32 accumulation, for M <= 64: the
 // matrix product of a decode step.  The weight is read once from HBM, which is
-// what bounds the step; the few rows of X come from L2.
+// what bounds the step.
 //
-// One workgroup of 8 waves owns 16 rows of W (16 output features).  The waves
-// split K into chunks of 128 and take every eighth chunk; each wave multiplies
-// its chunks with v_mfma_f32_16x16x32_bf16 (W as the A operand, X^T as the B
-// operand), and the eight partial tiles are summed through LDS in a fixed order,
-// so a result does not depend on timing.  In a chunk, lane (r, q) = (lane % 16,
-// lane / 16) reads 64 contiguous bytes of row r: k = chunk*128 + q*32 .. +31;
-// the operand of X uses the same k for the same lane, and a sum over k does not
-// care in which order the matrix core takes them.
+// A workgroup of 4 waves owns 64 rows of W (16 per wave) and a range of K.  K is
+// walked in chunks of 256.  The chunk of X (all M rows) is staged in LDS once per
+// workgroup and shared by its waves; every wave reads its own 16 rows of W
+// straight from global memory into registers (each byte of W is used by one wave
+// only, so LDS would gain nothing), one chunk ahead of the matrix cores, with
+// non-temporal loads.  Products run on v_mfma_f32_16x16x32_bf16 with W as the A
+// operand and X^T as the B operand.  Lane (r, q) = (lane % 16, lane / 16) holds,
+// for load i of a chunk, the 8 values k = chunk*256 + (4 i + q) * 8 .. +7 of row
+// r: the four lanes of a row read 64 contiguous bytes.  X uses the same k for the
+// same lane, and a sum over k does not care in which order the matrix core takes
+// them.
+//
+// To fill the GPU when N is small, K is split over blockIdx.y; every split
+// writes its fp32 partial tile to a workspace [splits, M, N], and a second kernel
+// adds the splits in the order of their index (no atomics: the result does not
+// depend on timing), optionally applies SwiGLU to [gate | up] halves, and stores.
+// The number of splits depends on N and K only, never on M, so a row's result
+// does not depend on what else is in the batch.
 //
 // K must be a multiple of 8 (16-byte loads); N and M are arbitrary (rows beyond
 // them are read from the last valid row and not stored).
@@ -17,102 +27,217 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-#define SK_WAVES 8
-#define SK_CHUNK 128
+#define SK_WAVES 4
+#define SK_KC 256               // k per chunk
+#define SK_NLD (SK_KC / 32)     // 16-byte loads per lane and chunk
+#define SK_XPAD 8               // bf16 elements of padding per LDS row (spreads the banks)
+#define SK_BN (SK_WAVES * 16)   // rows of W per workgroup
+#define SK_TARGET_BLOCKS 512    // K is split until the grid has about this many workgroups
 
-__device__ __forceinline__ bf16x8 load_bf16x8(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+enum { SK_EPI_NONE = 0, SK_EPI_SWIGLU = 1 };
+
+__device__ __forceinline__ uint4 load_stream_16(const uint16_t* p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
 }
 
 template <typename TO> __device__ __forceinline__ void store_out(TO* p, float v);
 template <> __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_out<uint16_t>(uint16_t* p, float v) { *p = float_to_bf16_bits(v); }
 
+// part != nullptr: fp32 partial tiles go to part[split, m, n]; else the result goes to C (one split only).
 template <int MT, typename TO>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ X,
                                                                     const uint16_t* __restrict__ W,
-                                                                    TO* __restrict__ C, int M, int N, int K) {
-  __shared__ f32x4 red[SK_WAVES][MT][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                                                                    TO* __restrict__ C, float* __restrict__ part,
+                                                                    int M, int N, int K, int chunks_per_split) {
+  constexpr int XROW = SK_KC + SK_XPAD;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][XROW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int n = (n0 + r < N) ? n0 + r : N - 1;
-  const uint16_t* wrow = W + (size_t)n * K;
-  const uint16_t* xrow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = (mt * 16 + r < M) ? mt * 16 + r : M - 1;
-    xrow[mt] = X + (size_t)m * K;
-  }
+  const int n_base = blockIdx.x * SK_BN + wave * 16;
+  const int split = blockIdx.y;
+  const int nchunks = (K + SK_KC - 1) / SK_KC;
+  const int c0 = split * chunks_per_split;
+  const int c1 = min(nchunks, c0 + chunks_per_split);
+
+  const int n_row = (n_base + r < N) ? n_base + r : N - 1;
+  const uint16_t* wrow = W + (size_t)n_row * K;
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 
-  const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
-#pragma unroll 2
-  for (int c = wave; c < nchunks; c += SK_WAVES) {
-    const int kbase = c * SK_CHUNK + q * 32;
-    bf16x8 wv[4];
+  // the chunk of X is MT*16 rows of 256 values = MT*512 pieces of 16 bytes, spread over the 256 threads
+  constexpr int XPIECES = MT * 16 * (SK_KC / 8);
+  constexpr int XPT = XPIECES / (SK_WAVES * 64);
+  static_assert(XPIECES % (SK_WAVES * 64) == 0, "pieces of X must divide over the threads");
+  uint4 xreg[XPT];
+  auto load_x = [&](int c) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int k = kbase + s * 8;
-      wv[s] = (k < K) ? load_bf16x8(wrow + k) : zero;
+    for (int i = 0; i < XPT; ++i) {
+      const int pc = tid + i * SK_WAVES * 64;
+      const int row = pc / (SK_KC / 8), kk = (pc % (SK_KC / 8)) * 8;
+      const int k = c * SK_KC + kk;
+      const int m = row < M ? row : M - 1;
+      xreg[i] = (k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      const int pc = tid + i * SK_WAVES * 64;
+      const int row = pc / (SK_KC / 8), kk = (pc % (SK_KC / 8)) * 8;
+      *reinterpret_cast<uint4*>(&xs[buf][row][kk]) = xreg[i];
+    }
+  };
+  uint4 wcur[SK_NLD], wnext[SK_NLD];
+  auto load_w = [&](int c, uint4 (&dst)[SK_NLD]) {
+#pragma unroll
+    for (int i = 0; i < SK_NLD; ++i) {
+      const int k = c * SK_KC + (i * 4 + q) * 8;
+      dst[i] = (k < K) ? load_stream_16(wrow + k) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+
+  if (c0 < c1) {
+    load_x(c0);
+    load_w(c0, wcur);
+    store_x(0);
+  }
+  __syncthreads();
+  for (int c = c0; c < c1; ++c) {
+    const int buf = (c - c0) & 1;
+    const bool more = c + 1 < c1;
+    if (more) {
+      // X first, W after it: the wait for X at the end of the round then leaves the loads of W in flight
+      load_x(c + 1);
+      load_w(c + 1, wnext);
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int i = 0; i < SK_NLD; ++i) {
+      const bf16x8 wv = __builtin_bit_cast(bf16x8, wcur[i]);
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int k = kbase + s * 8;
-        const bf16x8 xv = (k < K) ? load_bf16x8(xrow[mt] + k) : zero;
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[s], xv, acc[mt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint4 xv = *reinterpret_cast<const uint4*>(&xs[buf][mt * 16 + r][(i * 4 + q) * 8]);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, __builtin_bit_cast(bf16x8, xv), acc[mt], 0, 0, 0);
       }
     }
+    if (more) {
+      store_x(buf ^ 1);
+#pragma unroll
+      for (int i = 0; i < SK_NLD; ++i) wcur[i] = wnext[i];
+    }
+    __syncthreads();
   }
+  // lane holds D[i = 4 q + e][j = r]: i counts rows of W in the tile, j rows of X
+  const int n = n_base + 4 * q;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) red[wave][mt][lane] = acc[mt];
-  __syncthreads();
-  if (threadIdx.x < MT * 64) {
-    const int mt = threadIdx.x >> 6, ln = threadIdx.x & 63;
-    f32x4 s = red[0][mt][ln];
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r;
+    if (m >= M) continue;
+    if (part) {
+      float* o = part + ((size_t)split * M + m) * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<f32x4*>(o) = acc[mt];
+      } else {
 #pragma unroll
-    for (int w = 1; w < SK_WAVES; ++w) s += red[w][mt][ln];
-    // lane ln holds D[i = 4*(ln/16) + e][j = ln%16]: i counts rows of W, j rows of X
-    const int m = mt * 16 + (ln & 15);
-    const int nn = n0 + (ln >> 4) * 4;
-    if (m < M) {
-      TO* o = C + (size_t)m * N + nn;
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) o[e] = acc[mt][e];
+      }
+    } else {
+      TO* o = C + (size_t)m * N + n;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (nn + e < N) store_out<TO>(o + e, s[e]);
+        if (n + e < N) store_out<TO>(o + e, acc[mt][e]);
     }
   }
 }
 
+// C[m, n] = sum_s part[s, m, n]                                       (SK_EPI_NONE,   n < N)
+// C[m, n] = silu(sum_s part[s, m, n]) * sum_s part[s, m, N/2 + n]      (SK_EPI_SWIGLU, n < N/2)
+template <typename TO, int EPI>
+__global__ __launch_bounds__(256) void gemm_skinny_join_kernel(const float* __restrict__ part, TO* __restrict__ C,
+                                                               int M, int N, int splits) {
+  const int NO = EPI == SK_EPI_SWIGLU ? N / 2 : N;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)M * NO) return;
+  const int m = (int)(idx / NO), n = (int)(idx - (size_t)m * NO);
+  const size_t MN = (size_t)M * N;
+  const float* p = part + (size_t)m * N + n;
+  float a = 0.f, b = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    a += p[s * MN];
+    if (EPI == SK_EPI_SWIGLU) b += p[s * MN + NO];
+  }
+  store_out<TO>(C + idx, EPI == SK_EPI_SWIGLU ? a / (1.0f + expf(-a)) * b : a);
+}
+
+static int skinny_splits(int N, int K) {
+  const int nb = (N + SK_BN - 1) / SK_BN;
+  const int nchunks = (K + SK_KC - 1) / SK_KC;
+  int ks = (SK_TARGET_BLOCKS + nb - 1) / nb;
+  if (ks > nchunks) ks = nchunks;
+  if (ks < 1) ks = 1;
+  const int cps = (nchunks + ks - 1) / ks;
+  return (nchunks + cps - 1) / cps;
+}
+
+// Number of K splits the kernel uses for a weight [N, K] (a function of N and K only).
+extern "C" int ia_gemm_skinny_splits(int N, int K) { return (N > 0 && K > 0) ? skinny_splits(N, K) : 0; }
+
 template <typename TO>
-static int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
-  const unsigned grid = (unsigned)((N + 15) / 16);
-  const int mt = (M + 15) / 16;
-  const uint16_t* x = (const uint16_t*)X;
-  const uint16_t* w = (const uint16_t*)W;
-  TO* c = (TO*)C;
-  switch (mt) {
-    case 1: gemm_skinny_kernel<1, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, M, N, K); break;
-    case 2: gemm_skinny_kernel<2, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, M, N, K); break;
-    case 3: gemm_skinny_kernel<3, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, M, N, K); break;
-    case 4: gemm_skinny_kernel<4, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, M, N, K); break;
+static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K, int splits,
+                         hipStream_t stream) {
+  const int nchunks = (K + SK_KC - 1) / SK_KC;
+  const int cps = (nchunks + splits - 1) / splits;
+  dim3 grid((N + SK_BN - 1) / SK_BN, splits);
+  switch ((M + 15) / 16) {
+    case 1: gemm_skinny_kernel<1, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 2: gemm_skinny_kernel<2, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 3: gemm_skinny_kernel<3, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 4: gemm_skinny_kernel<4, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
     default: return IA_ERR_UNSUPPORTED;
   }
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
 
-// X, W bf16; C bf16 (out_dtype 1) or fp32 (out_dtype 0); all contiguous.
+template <typename TO>
+static int launch_join(const float* part, TO* c, int M, int N, int splits, int epilogue, hipStream_t stream) {
+  const int NO = epilogue == SK_EPI_SWIGLU ? N / 2 : N;
+  const unsigned grid = (unsigned)(((size_t)M * NO + 255) / 256);
+  if (epilogue == SK_EPI_SWIGLU)
+    gemm_skinny_join_kernel<TO, SK_EPI_SWIGLU><<<grid, 256, 0, stream>>>(part, c, M, N, splits);
+  else
+    gemm_skinny_join_kernel<TO, SK_EPI_NONE><<<grid, 256, 0, stream>>>(part, c, M, N, splits);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// X [M, K], W [N, K] bf16, contiguous.  C: bf16 (out_dtype 1) or fp32 (0); [M, N], or [M, N/2] with the SwiGLU
+// epilogue.  workspace: fp32, at least ia_gemm_skinny_splits(N, K) * M * N values when that count is above one
+// or an epilogue is asked for; may be null otherwise.  C == null: the partial sums are left in the workspace
+// as [splits, M, N] for a later kernel to join.
 extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
-                              hipStream_t stream) {
+                              int epilogue, float* workspace, size_t workspace_floats, hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
-  if (out_dtype == IA_F32) return launch_skinny<float>(X, W, C, M, N, K, stream);
-  if (out_dtype == IA_BF16) return launch_skinny<uint16_t>(X, W, C, M, N, K, stream);
-  return IA_ERR_BAD_ARG;
+  if (epilogue != SK_EPI_NONE && epilogue != SK_EPI_SWIGLU) return IA_ERR_BAD_ARG;
+  if (epilogue == SK_EPI_SWIGLU && (N & 1)) return IA_ERR_BAD_ARG;
+  if (out_dtype != IA_F32 && out_dtype != IA_BF16) return IA_ERR_BAD_ARG;
+  const int splits = skinny_splits(N, K);
+  if (splits > 65535) return IA_ERR_UNSUPPORTED;
+  const bool via_workspace = splits > 1 || epilogue != SK_EPI_NONE || C == nullptr;
+  if (via_workspace && (!workspace || workspace_floats < (size_t)splits * M * N)) return IA_ERR_BAD_ARG;
+  const uint16_t* x = (const uint16_t*)X;
+  const uint16_t* w = (const uint16_t*)W;
+  if (!via_workspace) {
+    if (out_dtype == IA_F32) return launch_skinny<float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
+    return launch_skinny<uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
+  }
+  const int rc = launch_skinny<float>(x, w, nullptr, workspace, M, N, K, splits, stream);
+  if (rc != IA_OK || C == nullptr) return rc;
+  if (out_dtype == IA_F32) return launch_join<float>(workspace, (float*)C, M, N, splits, epilogue, stream);
+  return launch_join<uint16_t>(workspace, (uint16_t*)C, M, N, splits, epilogue, stream);
 }

@@ -88,25 +88,54 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Te
     return out
 
 
-def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+class SplitSum:
+    """A matrix [M, N] given as a stack of fp32 partial sums ``parts`` [S, M, N]: what a matrix product
+    whose inner dimension was split over workgroups leaves.  The kernels that take the product next
+    (residual add + norm, rotary + cache write) add the parts themselves, in the order of their index."""
+
+    __slots__ = ("parts",)
+
+    def __init__(self, parts: torch.Tensor):
+        if parts.dim() != 3 or parts.dtype != torch.float32 or not parts.is_contiguous():
+            raise KernelError("SplitSum: parts must be a contiguous fp32 [S, M, N] tensor")
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    def joined(self, dtype: torch.dtype) -> torch.Tensor:
+        """The sum as one tensor (a library reduction; for paths that are not hot)."""
+        return self.parts.sum(dim=0).to(dtype)
+
+
+def add_rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """h += delta (fp32, in place); out = h * rsqrt(mean(h^2) + eps) * weight.
 
+    ``delta`` is None, a tensor of h's shape in out's dtype, or a :class:`SplitSum`.
     With ``rows`` the norm is taken of the selected rows only and h stays as it is.
     """
-    _dev(h, delta, weight, out, rows)
+    split = isinstance(delta, SplitSum)
+    d = delta.parts if split else delta
+    _dev(h, d, weight, out, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2, "add_rmsnorm: h must be fp32 [N, H]")
     H = h.shape[1]
     n_out = rows.numel() if rows is not None else h.shape[0]
     _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (n_out, H), f"add_rmsnorm: out must be [{n_out}, {H}]")
-    if delta is not None:
-        _need(delta.dtype == out.dtype and tuple(delta.shape) == tuple(h.shape),
+    splits, d_rows, d_code = 1, h.shape[0], DTYPE_CODE[out.dtype]
+    if split:
+        _need(tuple(d.shape[1:]) == tuple(h.shape), "add_rmsnorm: partial sums must be [S, N, H]")
+        splits, d_code = d.shape[0], DTYPE_CODE[torch.float32]
+    elif d is not None:
+        _need(d.dtype == out.dtype and tuple(d.shape) == tuple(h.shape),
               "add_rmsnorm: delta must have h's shape and out's dtype")
     _need(weight.dtype in DTYPE_CODE and weight.numel() == H, f"add_rmsnorm: weight must hold {H} values")
     if rows is not None:
         _i32(rows, n_out, "add_rmsnorm rows")
-    _ok(_core().ia_add_rmsnorm(_p(h), _p(delta), DTYPE_CODE[out.dtype], _p(weight), DTYPE_CODE[weight.dtype],
-                               _p(out), _p(rows), n_out, H, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+    _ok(_core().ia_add_rmsnorm(_p(h), _p(d), d_code, splits, d_rows, DTYPE_CODE[out.dtype], _p(weight),
+                               DTYPE_CODE[weight.dtype], _p(out), _p(rows), n_out, H, ctypes.c_float(eps),
+                               _stream()), "add_rmsnorm")
     return out
 
 
@@ -119,18 +148,27 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return h
 
 
-def rope_kv_append(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], nh: int, nkv: int,
+def rope_kv_append(qkv, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], nh: int, nkv: int,
                    d: int, rot: int, slots: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
-                   v_pages: Optional[torch.Tensor] = None) -> None:
-    """Rotate q (in place) and k, and write k and v to their page slots.
+                   v_pages: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotate q and k, and write k and v to their page slots.  Returns the rotated q, [N, >= nh d].
 
-    qkv is [N, (nh + 2 nkv) d] (or [N, nh d] when no pages are given).  Key pages are
-    [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size].
+    qkv is [N, (nh + 2 nkv) d] (or [N, nh d] when no pages are given), a tensor or a :class:`SplitSum`.
+    A tensor is rotated in place unless ``q_out`` is given; a SplitSum needs ``q_out`` [N, nh d] (made here
+    when absent).  Key pages are [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size].
     """
-    _dev(qkv, positions, inv_freq, slots, k_pages, v_pages)
+    split = isinstance(qkv, SplitSum)
+    src = qkv.parts if split else qkv
     write = k_pages is not None
-    N, row = qkv.shape
-    _need(qkv.dtype in DTYPE_CODE, "rope: dtype")
+    N, row = (src.shape[1], src.shape[2]) if split else tuple(src.shape)
+    act = (k_pages.dtype if write else (q_out.dtype if q_out is not None else None)) if split else src.dtype
+    _need(act is not None, "rope: partial sums need pages or q_out to tell the activations' dtype")
+    if q_out is None:
+        q_out = torch.empty((N, nh * d), dtype=act, device=src.device) if split else src
+    _dev(src, positions, inv_freq, slots, k_pages, v_pages)
+    _need(q_out.is_cuda and q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == N
+          and q_out.shape[1] >= nh * d and q_out.dtype == act, "rope: q_out must be [N, >= nh*d] in the activations' dtype")
+    _need(act in DTYPE_CODE and src.dtype in DTYPE_CODE, "rope: dtype")
     _need(row >= (nh + (2 * nkv if write else 0)) * d, "rope: row of qkv is too short for its heads")
     _i32(positions, N, "rope positions")
     if inv_freq is not None:
@@ -139,15 +177,17 @@ def rope_kv_append(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optiona
     page_size = num_pages = 0
     if write:
         _need(v_pages is not None and slots is not None, "rope: k_pages, v_pages and slots go together")
-        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "rope: pages must have qkv's dtype")
+        _need(k_pages.dtype == act and v_pages.dtype == act, "rope: pages must have the activations' dtype")
         num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
         _need(k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d
               and tuple(v_pages.shape) == (num_pages, nkv, d, page_size),
               "rope: key pages must be [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size]")
         _i32(slots, N, "rope slots")
-    _ok(_core().ia_rope_kv_append(_p(qkv), DTYPE_CODE[qkv.dtype], _p(positions), _p(slots), _p(inv_freq),
+    _ok(_core().ia_rope_kv_append(_p(src), DTYPE_CODE[src.dtype], src.shape[0] if split else 1, N, _p(q_out),
+                                  q_out.stride(0), DTYPE_CODE[act], _p(positions), _p(slots), _p(inv_freq),
                                   _p(k_pages), _p(v_pages), N, row, nh, nkv, d, rot if inv_freq is not None else 0,
                                   page_size, num_pages, 1 if write else 0, _stream()), "rope_kv_append")
+    return q_out
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -178,21 +218,49 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.T
 
 
 SKINNY_MAX_M = 64
+EPILOGUE = {None: 0, "swiglu": 1}
 
 
 def gemm_skinny_supported(M: int, N: int, K: int) -> bool:
     return 0 < M <= SKINNY_MAX_M and K % 8 == 0 and K >= 8 and N >= 1
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """bf16 out[M, N] (or fp32) = a[M, K] @ w[N, K]^T for M <= 64 on MFMA, weights streamed once."""
+def gemm_skinny_splits(N: int, K: int) -> int:
+    """Parts the inner dimension is split into for a weight [N, K] (depends on N and K only)."""
+    return int(_core().ia_gemm_skinny_splits(N, K))
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+                epilogue: Optional[str] = None, keep_split: bool = False,
+                out_dtype: torch.dtype = torch.bfloat16):
+    """a[M, K] @ w[N, K]^T for M <= 64 on MFMA, weights streamed once; bf16 operands, fp32 sums.
+
+    Returns ``out`` ([M, N] bf16 or fp32; [M, N/2] with the "swiglu" epilogue, silu(left half) * right half),
+    or, with ``keep_split`` and a product that is split, a :class:`SplitSum` for the next kernel to join.
+    """
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
-    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in DTYPE_CODE, "gemm_skinny: bf16 in")
-    _need(w.dim() == 2 and w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_skinny: shapes")
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bf16 operands")
+    _need(w.dim() == 2 and w.shape[1] == K, "gemm_skinny: shapes")
     _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 64, K % 8 == 0)")
-    _ok(_core().ia_gemm_skinny(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, _stream()), "gemm_skinny")
+    _need(epilogue in EPILOGUE, f"gemm_skinny: unknown epilogue {epilogue!r}")
+    _need(epilogue is None or N % 2 == 0, "gemm_skinny: the swiglu epilogue needs an even N")
+    splits = gemm_skinny_splits(N, K)
+    ws = None
+    if splits > 1 or epilogue is not None:
+        ws = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+    if keep_split and epilogue is None and splits > 1:
+        _ok(_core().ia_gemm_skinny(_p(a), _p(w), None, 0, M, N, K, 0, _p(ws), ctypes.c_size_t(ws.numel()),
+                                   _stream()), "gemm_skinny")
+        return SplitSum(ws)
+    n_out = N // 2 if epilogue == "swiglu" else N
+    if out is None:
+        out = torch.empty((M, n_out), dtype=out_dtype, device=a.device)
+    _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (M, n_out) and out.is_contiguous(),
+          f"gemm_skinny: out must be contiguous [{M}, {n_out}]")
+    _ok(_core().ia_gemm_skinny(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, EPILOGUE[epilogue], _p(ws),
+                               ctypes.c_size_t(ws.numel() if ws is not None else 0), _stream()), "gemm_skinny")
     return out
 
 

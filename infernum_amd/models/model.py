@@ -101,6 +101,6 @@ class DecoderModel:
         else:
             from ..kernels import api as K
             if pending is not None:
-                K.residual_add(h, pending)
+                K.residual_add(h, pending.joined(self.rt.dtype) if isinstance(pending, K.SplitSum) else pending)
             f = h.index_select(0, rows.long()).to(self.rt.dtype)
         return self.head.forward(f)

@@ -69,22 +69,28 @@ class Attention(Mixer):
         self.w_o = tensors["o_proj.weight"].contiguous()
 
     # ---- one step --------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView):
         nh, nkv, d = self.nh, self.nkv, self.d
         if cache.k_pages is None:
             raise K.KernelError("attention needs pages of the cache")
         g = cache.group
+        q_out = None
         if cache.writable:
-            qkv = linear(x, self.w_qkv)
-            K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
-                             ctx.slots[g], cache.k_pages, cache.v_pages)
+            qkv = linear(x, self.w_qkv, keep_split=True)
+            if isinstance(qkv, K.SplitSum):
+                q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+            q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
+                                 ctx.slots[g], cache.k_pages, cache.v_pages, q_out=q_out)
         else:
             # keys and values of another run of a layer: only queries are made here
-            qkv = linear(x, self.w_qkv[: nh * d])
-            K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim)
+            qkv = linear(x, self.w_qkv[: nh * d], keep_split=True)
+            if isinstance(qkv, K.SplitSum):
+                q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+            q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
+                                 q_out=q_out)
         out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
-        self.attend(qkv, out, ctx, cache)
-        return linear(out, self.w_o)
+        self.attend(q, out, ctx, cache)
+        return linear(out, self.w_o, keep_split=True)
 
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d

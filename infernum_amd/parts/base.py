@@ -190,9 +190,11 @@ class Part:
 class Norm(Part):
     category = "norm"
 
-    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: Optional[torch.Tensor] = None,
+    def forward(self, h: torch.Tensor, delta: Any, out: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """h [N, H] fp32 += delta (in place, when given); returns norm(h) in the compute dtype."""
+        """h [N, H] fp32 += delta (in place, when given); returns norm(h) in the compute dtype.
+        ``delta`` is what a mixer or a feed-forward returned: a tensor [N, H] in the compute dtype, or
+        a ``kernels.api.SplitSum`` (fp32 partial sums [S, N, H] that are added here)."""
         raise NotImplementedError
 
 
@@ -209,15 +211,17 @@ class Mixer(Part):
     def state_spec(self) -> Optional[StateSpec]:
         return None
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView) -> torch.Tensor:
-        """x [N, H] in the compute dtype -> [N, H]; reads and writes its cache view."""
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView) -> Any:
+        """x [N, H] in the compute dtype -> [N, H] (a tensor in the compute dtype, or a SplitSum that the
+        next norm joins); reads and writes its cache view."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     category = "feed_forward"
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> Any:
+        """x [N, H] in the compute dtype -> [N, H] (a tensor, or a SplitSum that the next norm joins)."""
         raise NotImplementedError
 
 

@@ -8,38 +8,50 @@ and calls cuBLAS (infernum-cuda/src/inner/cuda/ops/matmul.rs:68-117).
 fp32: the hand-written fp32 kernel, always (no reduced-precision matrix mode).
 bf16: up to 64 rows the hand-written MFMA kernel that streams the weight once;
 above that the library product (hipBLASLt through torch), as the reference uses
-its library there; an fp32 result of many rows comes from the generic kernel.
+its library there; an fp32 result of many rows comes 64 rows at a time from the
+hand-written kernel.
+
+``epilogue="swiglu"`` returns silu(y[:, :N/2]) * y[:, N/2:]; the decode kernel
+does it while it joins its partial sums, the other paths in a kernel of its own.
+``keep_split`` lets the decode kernel hand its partial sums on as a
+:class:`SplitSum`, for a norm or the rotary kernel to join.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Union
 
 import torch
 
 from ..kernels import api as K
+from ..kernels.api import SplitSum
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+           epilogue: Optional[str] = None, keep_split: bool = False) -> Union[torch.Tensor, SplitSum]:
     M, Kdim = x.shape
     N = w.shape[0]
     out_dtype = out_dtype or x.dtype
-    if out is None:
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    n_out = N // 2 if epilogue == "swiglu" else N
     if M == 0:
-        return out
+        return torch.empty((0, n_out), dtype=out_dtype, device=x.device)
+    if x.dtype == torch.bfloat16 and K.gemm_skinny_supported(M, N, Kdim) and x.is_contiguous():
+        return K.gemm_skinny(x, w, epilogue=epilogue, keep_split=keep_split, out_dtype=out_dtype)
     if x.dtype == torch.float32:
-        return K.gemm_generic(x, w, out)
-    if x.dtype != torch.bfloat16:
+        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
+    elif x.dtype != torch.bfloat16:
         raise K.KernelError(f"linear: dtype {x.dtype} is not supported")
-    if K.gemm_skinny_available() and K.gemm_skinny_supported(M, N, Kdim) and x.is_contiguous():
-        return K.gemm_skinny(x, w, out)
-    if out_dtype == torch.bfloat16:
-        return torch.mm(x, w.t(), out=out)          # library product, fp32 accumulation
-    # fp32 result from bf16 operands, many rows: 64 rows at a time through the skinny kernel
-    if K.gemm_skinny_available() and K.gemm_skinny_supported(1, N, Kdim) and x.is_contiguous():
+    elif out_dtype == torch.bfloat16:
+        y = torch.mm(x, w.t())                      # library product, fp32 accumulation
+    elif K.gemm_skinny_supported(1, N, Kdim) and x.is_contiguous():
+        # fp32 result from bf16 operands, many rows: 64 rows at a time through the skinny kernel
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         for m0 in range(0, M, K.SKINNY_MAX_M):
             m1 = min(M, m0 + K.SKINNY_MAX_M)
-            K.gemm_skinny(x[m0:m1], w, out[m0:m1])
-        return out
-    return K.gemm_generic(x, w, out)
+            K.gemm_skinny(x[m0:m1], w, out=y[m0:m1])
+    else:
+        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
+    if epilogue == "swiglu":
+        return K.swiglu(y, torch.empty((M, n_out), dtype=y.dtype, device=y.device))
+    if epilogue is not None:
+        raise K.KernelError(f"linear: unknown epilogue {epilogue!r}")
+    return y

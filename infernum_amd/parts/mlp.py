@@ -35,11 +35,9 @@ class SwiGLUFeedForward(FeedForward):
         self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"].contiguous()
 
-    def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None) -> torch.Tensor:
-        gate_up = linear(x, self.w_gate_up)
-        act = torch.empty((x.shape[0], self.intermediate_size), dtype=x.dtype, device=x.device)
-        K.swiglu(gate_up, act)
-        return linear(act, self.w_down)
+    def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):
+        act = linear(x, self.w_gate_up, epilogue="swiglu")
+        return linear(act, self.w_down, keep_split=True)
 
 
 register_part("feed_forward", "swiglu", SwiGLUFeedForward)

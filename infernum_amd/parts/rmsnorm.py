@@ -30,7 +30,7 @@ class RMSNorm(Norm):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors["weight"].contiguous()
 
-    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: Optional[torch.Tensor] = None,
+    def forward(self, h: torch.Tensor, delta, out: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = rows.numel() if rows is not None else h.shape[0]
         if out is None:

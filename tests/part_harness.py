@@ -69,3 +69,9 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     if got.dtype == torch.bfloat16:
         d = (d - want.abs() * 2.0 ** -8).clamp_min(0.0)
     return d.max().item() / max(want.pow(2).mean().sqrt().item(), 1e-30)
+
+
+def dense(y, rt):
+    """What a mixer or a feed-forward returned, as one tensor in the compute dtype."""
+    from infernum_amd.kernels.api import SplitSum
+    return y.joined(rt.dtype) if isinstance(y, SplitSum) else y

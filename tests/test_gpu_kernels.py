@@ -67,6 +67,28 @@ def test_add_rmsnorm(dtype, wdtype, H):
     assert torch.allclose(out2.double(), want2, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("H", [100, 1024, 4096, 6000])
+@pytest.mark.parametrize("S", [1, 3, 8])
+def test_add_rmsnorm_joins_partial_sums(H, S):
+    """delta as a stack of fp32 partial sums [S, N, H] (what a split matrix product leaves)."""
+    api = K()
+    N, eps = 5, 1e-5
+    h = _rand(N, H, seed=1)
+    parts = _rand(S, N, H, seed=2)
+    w = (_rand(H, seed=3).abs() + 0.5).to(torch.bfloat16)
+    h0 = h.clone()
+    out = torch.empty(N, H, dtype=torch.bfloat16, device=DEV)
+    api.add_rmsnorm(h, api.SplitSum(parts), w, eps, out)
+    s = h0.double() + parts.double().sum(0)
+    assert torch.allclose(h.double(), s, atol=1e-5)
+    want = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out.double(), want, atol=1e-2, rtol=1e-2)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, H, dtype=torch.bfloat16, device=DEV)
+    api.add_rmsnorm(h0.clone(), api.SplitSum(parts), w, eps, out2, rows)
+    assert torch.equal(out2, out[rows.long()])
+
+
 def test_rmsnorm_reference_vector():
     # infernum-cuda/src/inner/cuda/ops/rmsnorm.rs:171-203
     h = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)
@@ -176,6 +198,69 @@ def test_gemm_skinny(M, N, K_):
     one = torch.empty(1, N, device=DEV)
     api.gemm_skinny(a[M - 1:M].contiguous(), w, one)
     assert torch.equal(one[0], outf[M - 1])
+
+
+@pytest.mark.parametrize("M", [1, 8, 40, 64])
+@pytest.mark.parametrize("N,K_", [(352, 128), (4096, 4096), (1000, 14336), (28672, 4096), (130, 1000)])
+def test_gemm_skinny_partial_sums_and_swiglu(M, N, K_):
+    api = K()
+    a, w = _rand(M, K_, dtype=torch.bfloat16, seed=6), _rand(N, K_, dtype=torch.bfloat16, scale=0.05, seed=7)
+    plain = api.gemm_skinny(a, w, out_dtype=torch.float32)
+    want = a.double() @ w.double().t()
+    assert (plain.double() - want).abs().max().item() <= 2e-5 * math.sqrt(K_) * 0.05 + 1e-6 * want.abs().max().item()
+    kept = api.gemm_skinny(a, w, keep_split=True)
+    S = api.gemm_skinny_splits(N, K_)
+    if S > 1:
+        assert isinstance(kept, api.SplitSum) and tuple(kept.parts.shape) == (S, M, N)
+        total = kept.parts[0].clone()
+        for s_ in range(1, S):
+            total += kept.parts[s_]                      # the join adds the parts in the order of their index
+        assert torch.equal(total, plain)
+    else:
+        assert torch.equal(kept, plain.bfloat16())
+    act = api.gemm_skinny(a, w, epilogue="swiglu", out_dtype=torch.float32)
+    g, u = plain[:, :N // 2].double(), plain[:, N // 2:].double()
+    assert tuple(act.shape) == (M, N // 2)
+    assert torch.allclose(act.double(), g / (1 + torch.exp(-g)) * u, atol=1e-6, rtol=1e-5)
+    actb = api.gemm_skinny(a, w, epilogue="swiglu")
+    assert torch.equal(actb, act.bfloat16())
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    api = K()
+    a, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
+    with pytest.raises(api.KernelError):
+        api.gemm_skinny(a, w)
+    with pytest.raises(api.KernelError):
+        api.gemm_skinny(_rand(4, 60, dtype=torch.bfloat16), _rand(32, 60, dtype=torch.bfloat16))
+    with pytest.raises(api.KernelError):
+        api.gemm_skinny(_rand(4, 64, dtype=torch.bfloat16), _rand(33, 64, dtype=torch.bfloat16), epilogue="swiglu")
+
+
+def test_rope_from_partial_sums():
+    """The rotary kernel joins a split product itself: same pages and queries as from the joined tensor."""
+    api = K()
+    nh, nkv, d, ps, N, S = 6, 2, 48, 4, 9, 3
+    row = (nh + 2 * nkv) * d
+    parts = _rand(S, N, row, seed=4)
+    joined = parts.sum(0).bfloat16()
+    pos = torch.arange(3, 3 + N, dtype=torch.int32, device=DEV)
+    slots = torch.randperm(40)[:N].to(torch.int32).to(DEV)
+    inv = (1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    kp1, vp1 = torch.zeros(10, nkv, ps, d, dtype=torch.bfloat16, device=DEV), torch.zeros(10, nkv, d, ps, dtype=torch.bfloat16, device=DEV)
+    kp2, vp2 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    q1 = api.rope_kv_append(api.SplitSum(parts), pos, inv, nh, nkv, d, d, slots, kp1, vp1)
+    # reference: the fp32 sum through the same kernel as one fp32 "part"
+    q2 = api.rope_kv_append(api.SplitSum(parts.sum(0, keepdim=True).contiguous()), pos, inv, nh, nkv, d, d, slots, kp2, vp2)
+    assert tuple(q1.shape) == (N, nh * d) and q1.dtype == torch.bfloat16
+    assert torch.allclose(q1.float(), q2.float(), atol=2e-2) and torch.allclose(kp1.float(), kp2.float(), atol=2e-2)
+    assert torch.allclose(vp1.float(), vp2.float(), atol=2e-2)
+    # and against the bf16 tensor rotated in place (rounded once more before the rotation)
+    q3 = joined.clone()
+    kp3, vp3 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    api.rope_kv_append(q3, pos, inv, nh, nkv, d, d, slots, kp3, vp3)
+    assert torch.allclose(q1.float(), q3[:, :nh * d].float(), atol=6e-2)
+    assert torch.allclose(kp1.float(), kp3.float(), atol=6e-2)
 
 
 # ------------------------------------------------------------------- attention

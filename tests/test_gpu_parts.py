@@ -7,7 +7,7 @@ import torch
 
 import plain_llama as P
 import tiny_models as TM
-from part_harness import DEV, DTYPES, TOL, Steps, build, rel_err, runtime
+from part_harness import DEV, DTYPES, TOL, Steps, build, dense, rel_err, runtime
 
 pytestmark = pytest.mark.gpu
 BOTH = pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -77,7 +77,7 @@ def test_feed_forward_alone(dtype, H, I, N):
     rt = runtime(dtype)
     ff, w = build("feed_forward", "swiglu", {"hidden_size": H, "intermediate_size": I}, rt)
     x = _x(N, H, dtype, 3)
-    out = ff.forward(x.to(DEV).to(rt.dtype))
+    out = dense(ff.forward(x.to(DEV).to(rt.dtype)), rt)
     xd = x.double()
     want = P.linear(P.swiglu(P.linear(xd, w["gate_proj.weight"]), P.linear(xd, w["up_proj.weight"])),
                     w["down_proj.weight"])
@@ -123,7 +123,7 @@ def _run_attention(att, rt, x, cuts, page_size, window_pages=64):
     outs, p = [], 0
     for n in cuts:
         ctx, packed = steps.begin([("r", n)])
-        outs.append(att.forward(x[p:p + n].to(DEV).to(rt.dtype).contiguous(), ctx, steps.views[0]).cpu())
+        outs.append(dense(att.forward(x[p:p + n].to(DEV).to(rt.dtype).contiguous(), ctx, steps.views[0]), rt).cpu())
         steps.end(packed)
         p += n
     assert p == x.shape[0]
@@ -237,7 +237,7 @@ def test_attention_key_at_a_pages_edge_with_shuffled_pages(dtype):
         outs, p = [], 0
         for n in (30, 19, 1):
             ctx, packed = steps.begin([("r", n)])
-            outs.append(att.forward(x[p:p + n].to(DEV).to(rt.dtype).contiguous(), ctx, steps.views[0]).cpu())
+            outs.append(dense(att.forward(x[p:p + n].to(DEV).to(rt.dtype).contiguous(), ctx, steps.views[0]), rt).cpu())
             steps.end(packed)
             p += n
         pages = steps.cache.block_table(0, "r").pages
@@ -266,7 +266,7 @@ def test_block_alone(dtype):
     steps = Steps([(att.cache_spec(), None)], rt, page_size=4)
     ctx, packed = steps.begin([("r", T)])
     hd = h0.to(DEV).clone()
-    out = block.forward(hd, pending.to(DEV).to(rt.dtype), ctx, steps.views[0])
+    out = dense(block.forward(hd, pending.to(DEV).to(rt.dtype), ctx, steps.views[0]), rt)
     s = h0.double() + pending.double()
     a = _plain_attention(P.rms_norm(s, w1["weight"], eps), wa, nh, nkv, d, P.rope_frequencies(d, 1e4, None), None)
     h1 = s + a
