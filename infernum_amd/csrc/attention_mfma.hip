@@ -146,13 +146,19 @@ __device__ __forceinline__ void attn_tile(int t0, int key_lo, int key_hi, const 
 }
 
 // ------------------------------------------------------------------------ decode
-// grid (B, nkv * ceil(G/16), num_splits), 64 threads.  Token b is row b of q and out.
-extern "C" __global__ __launch_bounds__(64) void attn_decode_kernel(
+// grid (B, nkv * ceil(G/16), num_splits), 256 threads.  Token b is row b of q and out.  The four waves of a
+// workgroup take every fourth tile of 16 keys of the workgroup's part of the keys and join what they found
+// through LDS (in the order of the waves), so that few requests still put many waves to work without more
+// partial results in memory.
+#define DEC_WAVES 4
+extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ positions, const int* __restrict__ block_tables,
     int bt_stride, int nh, int nkv, int ps, int num_pages, float scale_log2, int window, int num_splits) {
-  const int b = blockIdx.x, lane = threadIdx.x, j = lane & 15, qd = lane >> 4;
+  __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
+  __shared__ f32x4 s_o[DEC_WAVES][NS][64];
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, qd = lane >> 4;
   const int G = nh / nkv, HT = (G + 15) / 16;
   const int g = blockIdx.y / HT, ht = blockIdx.y - g * HT;
   const int split = blockIdx.z;
@@ -175,25 +181,45 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_kernel(
   const int ta = t_first + split * per;
   const int tb = (ta + per < t_last + 1) ? ta + per : t_last + 1;
   const int* bt = block_tables + (size_t)b * bt_stride;
-  for (int t = ta; t < tb; ++t)
+  for (int t = ta + wave; t < tb; t += DEC_WAVES)
     attn_tile<1>(t * 16, lo0, p, bt, ps, num_pages, nkv, g, k_pages, v_pages, qreg, pos, lo, scale_log2, o, m, l, lane);
+  // ---- join the waves: common maximum, rescale, add in the order of the waves
+  if (qd == 0) { s_m[wave][j] = m[0]; s_l[wave][j] = l[0]; }
+  __syncthreads();
+  float M = s_m[0][j];
+#pragma unroll
+  for (int w = 1; w < DEC_WAVES; ++w) M = fmaxf(M, s_m[w][j]);
+  float L = 0.f;
+#pragma unroll
+  for (int w = 0; w < DEC_WAVES; ++w) {
+    const float mw = s_m[w][j];
+    L += (mw == -INFINITY ? 0.f : exp2f(mw - M)) * s_l[w][j];
+  }
+  const float f = (m[0] == -INFINITY) ? 0.f : exp2f(m[0] - M);
+#pragma unroll
+  for (int n = 0; n < NS; ++n) s_o[wave][n][lane] = o[0][n] * f;
+  __syncthreads();
   if (!col_ok) return;
-  if (num_splits == 1) {
-    const float inv = 1.0f / l[0];
-    uint16_t* orow = out + (size_t)b * out_row_stride + (size_t)h * HD + 4 * qd;
+  // wave w finishes the slices n = w, w + 4, ... of the head
+  for (int n = wave; n < NS; n += DEC_WAVES) {
+    f32x4 acc = s_o[0][n][lane];
 #pragma unroll
-    for (int n = 0; n < NS; ++n) {
-      uint2 w;
-      w.x = (uint32_t)float_to_bf16_bits(o[0][n][0] * inv) | ((uint32_t)float_to_bf16_bits(o[0][n][1] * inv) << 16);
-      w.y = (uint32_t)float_to_bf16_bits(o[0][n][2] * inv) | ((uint32_t)float_to_bf16_bits(o[0][n][3] * inv) << 16);
-      *reinterpret_cast<uint2*>(orow + n * 16) = w;
+    for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w][n][lane];
+    if (num_splits == 1) {
+      const float inv = 1.0f / L;
+      uint2 wv;
+      wv.x = (uint32_t)float_to_bf16_bits(acc[0] * inv) | ((uint32_t)float_to_bf16_bits(acc[1] * inv) << 16);
+      wv.y = (uint32_t)float_to_bf16_bits(acc[2] * inv) | ((uint32_t)float_to_bf16_bits(acc[3] * inv) << 16);
+      *reinterpret_cast<uint2*>(out + (size_t)b * out_row_stride + (size_t)h * HD + 4 * qd + n * 16) = wv;
+    } else {
+      const size_t rec = ((size_t)b * nh + h) * num_splits + split;
+      *reinterpret_cast<f32x4*>(part_o + rec * HD + 4 * qd + n * 16) = acc;
     }
-  } else {
+  }
+  if (num_splits > 1 && wave == 0 && qd == 0) {
     const size_t rec = ((size_t)b * nh + h) * num_splits + split;
-    float* po = part_o + rec * HD + 4 * qd;
-#pragma unroll
-    for (int n = 0; n < NS; ++n) *reinterpret_cast<f32x4*>(po + n * 16) = o[0][n];
-    if (qd == 0) { part_ml[rec * 2] = m[0]; part_ml[rec * 2 + 1] = l[0]; }
+    part_ml[rec * 2] = M;
+    part_ml[rec * 2 + 1] = L;
   }
 }
 
@@ -227,7 +253,9 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 #pragma unroll
       for (int c = 0; c < (HD + 63) / 64; ++c) {
         const int dim = lane + 64 * c;
-        if (dim < HD && wj != 0.f) acc[c] += wj * part_o[(rec0 + s0 + j) * HD + dim];
+        // every part was written (an empty one holds zeros), so the load needs no guard and does not wait
+        const float v = dim < HD ? part_o[(rec0 + s0 + j) * HD + dim] : 0.f;
+        acc[c] += (wj != 0.f) ? wj * v : 0.f;
       }
     }
   }
@@ -315,7 +343,7 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
   if (nkv * HT > 65535) return IA_ERR_UNSUPPORTED;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(B, nkv * HT, num_splits);
-  attn_decode_kernel<<<grid, 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
+  attn_decode_kernel<<<grid, DEC_WAVES * 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
                                               (const uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o,
                                               part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages,
                                               scale_log2, window, num_splits);

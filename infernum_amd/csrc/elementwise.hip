@@ -239,6 +239,8 @@ __device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t 
   return v;
 }
 
+// grid (N, ceil(heads / 4)), 256 threads: one wave per (token, head), so that a handful of decoded tokens
+// still spread over the GPU; heads are nh queries, then nkv keys, then nkv values.
 template <typename TS, typename T>
 __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restrict__ src, int splits,
                                                              size_t split_stride, T* __restrict__ q_out,
@@ -248,55 +250,37 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restric
                                                              T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                              int row_stride, int nh, int nkv, int d, int rot,
                                                              int page_size, int num_pages, int write_kv,
-                                                             int copy_q_tail, int lanes_per_head) {
+                                                             int copy_q_tail) {
   const int n = blockIdx.x;
-  const float pos = (float)positions[n];
-  const TS* row = src + (size_t)n * row_stride;
-  T* qrow = q_out + (size_t)n * q_stride;
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int slot = (write_kv && slots) ? slots[n] : -1;
   const bool do_write = slot >= 0 && slot < num_pages * page_size;
+  if (head >= nh + (do_write ? 2 * nkv : 0)) return;
+  const TS* x = src + (size_t)n * row_stride + (size_t)head * d;
   const int page = do_write ? slot / page_size : 0;
   const int off = do_write ? slot % page_size : 0;
+  if (head >= nh + nkv) {             // a value head: a plain copy into the transposed page
+    const int g = head - nh - nkv;
+    T* dst = v_pages + ((size_t)page * nkv + g) * d * page_size + off;
+    for (int i = lane; i < d; i += 64) dst[(size_t)i * page_size] = from_float<T>(load_split_sum(x + i, splits, split_stride));
+    return;
+  }
+  const bool is_q = head < nh;
+  T* dst = is_q ? q_out + (size_t)n * q_stride + (size_t)head * d
+                : k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
   const int half = rot >> 1;
-  const int rot_heads = nh + (do_write ? nkv : 0);
-  // thread = (head group hg, pair i): lanes_per_head is a power of two that covers `half` (at most 256)
-  const int i0 = threadIdx.x % lanes_per_head, hg = threadIdx.x / lanes_per_head, HG = 256 / lanes_per_head;
-  for (int i = i0; i < half; i += lanes_per_head) {
-    float sn = 0.f, cs = 1.f;
-    if (inv_freq) sincosf(pos * inv_freq[i], &sn, &cs);
-    for (int head = hg; head < rot_heads; head += HG) {
-      const TS* x = row + (size_t)head * d;
-      const float a = load_split_sum(x + i, splits, split_stride);
-      const float b = load_split_sum(x + i + half, splits, split_stride);
-      const float o1 = a * cs - b * sn, o2 = a * sn + b * cs;
-      if (head < nh) {
-        qrow[(size_t)head * d + i] = from_float<T>(o1);
-        qrow[(size_t)head * d + i + half] = from_float<T>(o2);
-      } else {
-        T* dst = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
-        dst[i] = from_float<T>(o1);
-        dst[i + half] = from_float<T>(o2);
-      }
-    }
+  const float pos = (float)positions[n];
+  for (int i = lane; i < half; i += 64) {
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    const float a = load_split_sum(x + i, splits, split_stride);
+    const float b = load_split_sum(x + i + half, splits, split_stride);
+    dst[i] = from_float<T>(a * cs - b * sn);
+    dst[i + half] = from_float<T>(a * sn + b * cs);
   }
-  // values beyond the rotated part are plain copies
-  const int tail = d - rot;
-  if (copy_q_tail)
-    for (int idx = threadIdx.x; idx < nh * tail; idx += 256) {
-      const int hd = idx / tail, i = rot + (idx - hd * tail);
-      qrow[(size_t)hd * d + i] = from_float<T>(load_split_sum(row + (size_t)hd * d + i, splits, split_stride));
-    }
-  if (!do_write) return;
-  for (int idx = threadIdx.x; idx < nkv * tail; idx += 256) {
-    const int g = idx / tail, i = rot + (idx - g * tail);
-    k_pages[(((size_t)page * nkv + g) * page_size + off) * d + i] =
-        from_float<T>(load_split_sum(row + (size_t)(nh + g) * d + i, splits, split_stride));
-  }
-  for (int idx = threadIdx.x; idx < nkv * d; idx += 256) {
-    const int g = idx / d, i = idx - g * d;
-    v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] =
-        from_float<T>(load_split_sum(row + (size_t)(nh + nkv + g) * d + i, splits, split_stride));
-  }
+  if (!is_q || copy_q_tail)           // values beyond the rotated part are plain copies
+    for (int i = rot + lane; i < d; i += 64) dst[i] = from_float<T>(load_split_sum(x + i, splits, split_stride));
 }
 
 // src: [splits, src_rows, row_stride] of src_dtype; q_out, pages: act_dtype.
@@ -312,12 +296,14 @@ extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int
   if (!inv_freq) rot = 0;
   const size_t stride = (size_t)src_rows * row_stride;
   const int copy_q_tail = (src != q_out || splits > 1) ? 1 : 0;
-  int lph = 1;
-  while (lph < (rot >> 1) && lph < 256) lph <<= 1;
-#define ROPE_LAUNCH(TS, T)                                                                                        \
-  rope_kv_append_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, splits, stride, (T*)q_out, q_stride, positions, \
-                                                      slots, inv_freq, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
-                                                      d, rot, page_size, num_pages, write_kv, copy_q_tail, lph)
+  const int heads = nh + (write_kv ? 2 * nkv : 0);
+  if ((heads + 3) / 4 > 65535) return IA_ERR_UNSUPPORTED;
+  const dim3 grid(N, (heads + 3) / 4);
+#define ROPE_LAUNCH(TS, T)                                                                                         \
+  rope_kv_append_kernel<TS, T><<<grid, 256, 0, stream>>>((const TS*)src, splits, stride, (T*)q_out, q_stride,      \
+                                                         positions, slots, inv_freq, (T*)k_pages, (T*)v_pages,     \
+                                                         row_stride, nh, nkv, d, rot, page_size, num_pages,        \
+                                                         write_kv, copy_q_tail)
   if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_LAUNCH(float, float);
   else if (act_dtype == IA_BF16 && src_dtype == IA_BF16) ROPE_LAUNCH(bf16_t, bf16_t);
   else if (act_dtype == IA_BF16 && src_dtype == IA_F32) ROPE_LAUNCH(float, bf16_t);

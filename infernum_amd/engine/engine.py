@@ -29,8 +29,23 @@ class OutOfPages(RuntimeError):
     """The pool has too few free pages (or state slots) for this step; nothing was changed."""
 
 
+class _DecodeGraph:
+    """A recorded decode step of one shape: its int32 inputs, the recorded launches, its logits."""
+
+    __slots__ = ("inputs", "graph", "logits")
+
+    def __init__(self, inputs: torch.Tensor, graph: "torch.cuda.CUDAGraph", logits: torch.Tensor):
+        self.inputs, self.graph, self.logits = inputs, graph, logits
+
+
 class Engine:
-    def __init__(self, model: DecoderModel, cache_config: CacheConfig):
+    """``use_graphs``: steps in which every request brings one token are recorded into a HIP graph per shape
+    (number of requests, width of the block tables, number of wanted rows) the second time the shape comes,
+    and replayed from then on: one launch instead of some hundred.  The step's int32 arrays are copied into
+    the graph's own input buffer first; pages, state and weights are where they always are.  Models with a
+    part that is not marked ``graph_safe`` (one that reads device memory on the host, say) run without."""
+
+    def __init__(self, model: DecoderModel, cache_config: CacheConfig, use_graphs: bool = True):
         self.model = model
         self.rt: Runtime = model.rt
         self.spec = model.spec
@@ -38,6 +53,11 @@ class Engine:
                                   dtype=self.rt.dtype, device=self.rt.device)
         self.views = self.cache.views()
         self.steps_run = 0
+        self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and model.graph_safe()
+        self._graphs: Dict[tuple, _DecodeGraph] = {}
+        self._shape_seen: Dict[tuple, int] = {}
+        self._graph_pool = None
+        self.graph_replays = 0
 
     # ---- building ------------------------------------------------------------------
     @staticmethod
@@ -54,7 +74,7 @@ class Engine:
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", cache_config: Optional[CacheConfig] = None,
-                        device: Any = "cuda:0", **runtime_kw: Any) -> "Engine":
+                        device: Any = "cuda:0", use_graphs: bool = True, **runtime_kw: Any) -> "Engine":
         """Model class by config.json's model_type, weights from the folder's safetensors."""
         from .. import models  # noqa: F401  (registers the architectures)
         from ..config.registry import load_config, model_spec_for
@@ -65,14 +85,15 @@ class Engine:
         config = load_config(model_dir)
         model = DecoderModel(model_spec_for(config), rt)
         load_weights(model, model_dir)
-        eng = cls(model, cache_config or CacheConfig())
+        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs)
         eng.config = config
         return eng
 
     @classmethod
     def from_config(cls, config: Any, seed: int = 0, dtype: Any = "bfloat16",
                     cache_config: Optional[CacheConfig] = None, device: Any = "cuda:0",
-                    spec_kw: Optional[Dict[str, Any]] = None, **runtime_kw: Any) -> "Engine":
+                    spec_kw: Optional[Dict[str, Any]] = None, use_graphs: bool = True,
+                    **runtime_kw: Any) -> "Engine":
         """Random weights made on the device from (config, seed); nothing is read or written."""
         from .. import models  # noqa: F401
         from ..config.registry import model_spec_for
@@ -82,7 +103,7 @@ class Engine:
         load_library("core")
         model = DecoderModel(model_spec_for(config, **(spec_kw or {})), rt)
         random_weights_on_device(model, seed)
-        eng = cls(model, cache_config or CacheConfig())
+        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs)
         eng.config = config
         return eng
 
@@ -114,13 +135,57 @@ class Engine:
                 cache.admit(e.request)
             ok = cache.reserve(e.request, len(e.tokens))
             assert ok
-        packed = pack_step(cache, entries)
-        ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
-        logits = self.model.forward(ctx, self.views)
-        for e in packed.batch:
+        if all(len(e.tokens) == 1 for e in entries):
+            logits = self._decode_step(entries)
+        else:
+            packed = pack_step(cache, entries)
+            ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
+            logits = self.model.forward(ctx, self.views)
+        for e in entries:
             cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
         return logits
+
+    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Every request brings one token.  Block tables are widened to a power of two of pages, and the
+        kernels are told that width as the longest length, so that a shape's launches are the same from
+        step to step, recorded or not."""
+        cache = self.cache
+        widths = []
+        for g in cache.groups:
+            need = max(len(g.tables[e.request].pages) for e in entries)
+            w = 8
+            while w < need:
+                w *= 2
+            widths.append(w)
+        width = max(widths) if widths else None
+        packed = pack_step(cache, entries, bt_width=width)
+        limit = (width or 0) * cache.page_size
+        key = (len(entries), width, packed.num_logit_rows)
+        g = self._graphs.get(key)
+        if g is not None:
+            g.inputs.copy_(torch.from_numpy(packed.host))
+            g.graph.replay()
+            self.graph_replays += 1
+            return g.logits.clone()
+        seen = self._shape_seen.get(key, 0)
+        self._shape_seen[key] = seen + 1
+        inputs = torch.from_numpy(packed.host).to(self.rt.device)
+        ctx = packed.context(inputs)
+        ctx.max_total_len = max(limit, ctx.max_total_len)
+        if not self.use_graphs or seen < 1:
+            return self.model.forward(ctx, self.views)
+        # second time this shape comes: record it (kernels were loaded by the first, eager run)
+        torch.cuda.synchronize(self.rt.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self.model.forward(ctx, self.views)
+        if self._graph_pool is None:
+            self._graph_pool = graph.pool()
+        self._graphs[key] = _DecodeGraph(inputs, graph, logits)
+        graph.replay()
+        self.graph_replays += 1
+        return logits.clone()
 
     def decode_greedy(self, requests: Sequence[Hashable], tokens: Sequence[int]) -> List[int]:
         """One decode step for requests that each bring one token; returns each one's next token (argmax)."""

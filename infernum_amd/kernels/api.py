@@ -304,10 +304,11 @@ def _attn(d: int) -> ctypes.CDLL:
 
 
 def decode_splits(batch: int, nh: int, nkv: int, max_len: int) -> int:
-    """Parts the keys of a request are cut into, so that a small batch still fills the GPU."""
+    """Parts the keys of a request are cut into, so that a small batch still fills the GPU: about 512
+    workgroups (of four waves, each wave one tile of 16 keys at a time), at least 4 tiles a workgroup."""
     groups = batch * nkv * ((nh // nkv + 15) // 16)
     tiles = max(1, (max_len + 15) // 16)
-    return max(1, min((1024 + groups - 1) // groups, (tiles + 1) // 2, 64))
+    return max(1, min((512 + groups - 1) // groups, (tiles + 3) // 4, 64))
 
 
 def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,

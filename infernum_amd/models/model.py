@@ -54,6 +54,12 @@ class DecoderModel:
                 if a != b:
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_of}: {a} != {b}")
 
+    def graph_safe(self) -> bool:
+        """True when every part may be recorded into a HIP graph (it launches kernels on the current stream
+        and reads nothing back from the device on the host)."""
+        return all(getattr(part, "graph_safe", False) for _, part in self._parts) and \
+            all(getattr(b, "graph_safe", False) for b in self.blocks)
+
     # ---- weights -------------------------------------------------------------
     def expected_weights(self) -> Dict[str, WeightSpec]:
         """Full tensor name -> what is expected of it."""

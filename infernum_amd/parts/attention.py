@@ -27,6 +27,7 @@ from .linear import linear
 
 
 class Attention(Mixer):
+    graph_safe = True
     def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[Mapping[str, Any]] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, kernels: str = "auto", init_std: float = 0.02):

@@ -175,6 +175,9 @@ class Part:
     """Base of all parts.  ``weights`` lists what it wants; ``load`` receives them."""
 
     category = "part"
+    # True when ``forward`` only launches kernels on the current stream with shapes that follow from the
+    # step's sizes, and reads nothing from the device on the host: such a step can be recorded and replayed.
+    graph_safe = False
 
     def __init__(self, rt: Runtime, **params: Any):
         self.rt = rt
@@ -250,6 +253,7 @@ class Block:
     """
 
     category = "block"
+    graph_safe = False
 
     def __init__(self, rt: Runtime, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
                  feed_forward_norm: Norm, extra: Mapping[str, Part]):

@@ -16,6 +16,7 @@ from .base import Block, CacheView, StepContext, register_part
 
 
 class PreNormBlock(Block):
+    graph_safe = True
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
                 cache: CacheView) -> torch.Tensor:
         n = self.mixer_norm.forward(h, pending)

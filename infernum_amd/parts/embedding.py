@@ -19,6 +19,7 @@ from .linear import linear
 
 
 class TokenEmbedding(Embedding):
+    graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02):
         super().__init__(rt)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
@@ -37,6 +38,7 @@ class TokenEmbedding(Embedding):
 
 
 class LinearHead(Head):
+    graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, fallback: Optional[str] = None,
                  tied: bool = False, init_std: float = 0.02):
         super().__init__(rt)

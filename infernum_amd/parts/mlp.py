@@ -15,6 +15,7 @@ from .linear import linear
 
 
 class SwiGLUFeedForward(FeedForward):
+    graph_safe = True
     def __init__(self, rt: Runtime, hidden_size: int, intermediate_size: int, init_std: float = 0.02):
         super().__init__(rt)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

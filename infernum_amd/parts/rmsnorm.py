@@ -16,6 +16,7 @@ from .base import Norm, Runtime, WeightSpec, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
     def __init__(self, rt: Runtime, size: int, eps: float, init: tuple = ("ones",)):
         super().__init__(rt)
         self.size = int(size)

@@ -56,6 +56,7 @@ def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Ma
 
 class RotaryEmbedding(PositionEncoding):
     """Half-split rotary encoding of the first ``rotary_dim`` values of a head."""
+    graph_safe = True
 
     def __init__(self, rt: Runtime, head_dim: int, theta: float, scaling: Optional[Mapping[str, Any]] = None,
                  rotary_dim: Optional[int] = None):
@@ -69,6 +70,7 @@ class RotaryEmbedding(PositionEncoding):
 
 class NoPositionEncoding(PositionEncoding):
     """Queries and keys are used as they are."""
+    graph_safe = True
 
     def __init__(self, rt: Runtime, **_: Any):
         super().__init__(rt)

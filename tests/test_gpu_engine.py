@@ -144,3 +144,39 @@ def test_trace_run_program(models, tmp_path):
                 row += 1
             pos[e["id"]] = base + len(e["tokens"])
     _check(got, ref, "float32", "trace_run A float32 mixed")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_recorded_decode_steps_equal_eager_ones(models, name, dtype):
+    """Decode steps replayed from a HIP graph give the bits of the same steps launched one by one; every
+    replay is checked, with eager steps (portions of prompts) and synchronisations between them."""
+    from infernum_amd import CacheConfig, Engine, StepEntry
+    d, cfg, reqs, ref = models[(name, dtype, "mixed")]
+    eager = Engine.from_pretrained(d, dtype=dtype, use_graphs=False,
+                                   cache_config=CacheConfig(page_size=PAGE[name], num_pages=128, num_state_slots=8))
+    graphed = Engine.from_pretrained(d, dtype=dtype, use_graphs=True,
+                                     cache_config=CacheConfig(page_size=PAGE[name], num_pages=128, num_state_slots=8))
+    assert graphed.use_graphs and not eager.use_graphs
+    names = sorted(reqs, key=lambda r: -len(reqs[r]))[:3]      # the three longest: 41 + 40 tokens at least
+    fed = {r: 0 for r in names}
+    for r in names:                                   # prompts in one step each
+        n = 20 + 7 * names.index(r)
+        for eng in (eager, graphed):
+            eng.step([StepEntry(r, reqs[r][:n], [])])
+        fed[r] = n
+    for it in range(40):
+        live = names if it % 7 else names[:2]         # the batch size changes now and then: another shape
+        entries = [StepEntry(r, reqs[r][fed[r]:fed[r] + 1], [0]) for r in live]
+        a, b = eager.step(entries), graphed.step(entries)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), it
+        for r in live:
+            fed[r] += 1
+        if it % 9 == 4:                               # an eager step of another kind between replays
+            for eng in (eager, graphed):
+                eng.step([StepEntry("x", reqs[names[0]][:11], [10])])
+                eng.end("x")
+    assert graphed.graph_replays >= 30
+    got = {(r, fed[r] - 1): graphed.step([StepEntry(r, reqs[r][fed[r]:fed[r] + 1], [0])])[0].cpu() for r in names[:1]}
+    _check({(names[0], fed[names[0]]): got[(names[0], fed[names[0]] - 1)]}, ref, dtype, f"{name} {dtype} recorded decode")
