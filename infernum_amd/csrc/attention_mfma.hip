@@ -25,6 +25,7 @@
 // zeroed (values) or masked (scores): a stale or poisoned page never leaks in.
 // A key that is needed but has no page in the block table gives NaN, not a fault.
 #include "common.h"
+#include <stdlib.h>
 
 #ifndef IA_HEAD_DIM
 #error "compile with -DIA_HEAD_DIM=<head size>"
@@ -268,54 +269,292 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 }
 
 // ----------------------------------------------------------------------- prefill
-// grid (num_tiles, nkv * ceil(G / GH), 64 / (16 * CT / GH)), 64 threads.
+// grid (num_tiles, nkv * ceil(G / CT)), 256 threads.
 // tiles[i] = (request, first row of a block of 64 rows among the request's new tokens).
-extern "C" __global__ __launch_bounds__(64) void attn_prefill_kernel(
+// A workgroup takes 64 rows x CT query heads of one key/value head: wave w takes rows 16 w .. 16 w + 15 for
+// all CT heads.  Keys and values go through LDS in tiles of 32 keys, loaded once per workgroup and read by
+// its four waves; the loads of the next tile are in flight while the matrix cores work on this one.
+//   S^T[key, col] = K[key, :] . Q[col, :]       v_mfma_f32_16x16x32_bf16 over 32 head dims a step
+//   O^T[dim, col] += V^T[dim, key] P^T[key, col] one v_mfma_f32_16x16x32_bf16 over the 32 keys of a tile
+// The accumulators of the two S^T tiles of 16 keys leave lane (col, qd) with the keys 4 qd .. 4 qd + 3 and
+// 16 + 4 qd .. 16 + 4 qd + 3; the values are laid into LDS in that order of keys, so the probabilities go
+// from registers to registers.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+#define PF_WAVES 4
+#define PF_KT 32
+#define PF_KROW (HD + 8)        // bf16 per key row in LDS: 16 bytes of padding spread the banks
+#define PF_VROW 40              // bf16 per dim row of V^T in LDS (32 keys + 8 of padding)
+#define PF_CT_MAX (HD <= 128 ? 4 : 2)
+#define PF_LAZY 6.0f            // log2 of how far the running maximum may run ahead of the reference point
+
+template <int CT>
+__global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
     const int* __restrict__ seq_starts, const int* __restrict__ seq_ctx, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, float scale_log2,
-    int window, int GH) {
-  constexpr int CT = PREFILL_CT;
-  const int lane = threadIdx.x, j = lane & 15, qd = lane >> 4;
+    int window) {
+  __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KT][PF_KROW];
+  __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD][PF_VROW];
+  __shared__ int s_poison;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, qd = lane >> 4;
   const int sidx = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
-  const int G = nh / nkv, HC = (G + GH - 1) / GH, TT = CT / GH;
+  const int G = nh / nkv, HC = (G + CT - 1) / CT;
   const int g = blockIdx.y / HC, hc = blockIdx.y - g * HC;
-  const int rb = row0 + blockIdx.z * TT * 16;
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
-  if (rb >= qlen) return;
-  s16x4 qreg[CT][NS];
+  const int rows_here = (qlen - row0) < 64 ? (qlen - row0) : 64;      // rows of this workgroup (>= 1)
+  const int rb = row0 + wave * 16;                                     // first row of this wave
+  if (tid == 0) s_poison = 0;
+
+  // ---- queries of this wave: CT heads x 16 rows, as B operands (col = row j of head c)
+  // steps of 32 head dims; a head size that is an odd multiple of 16 ends with a step whose upper half
+  // is zero in both operands (lanes qd >= 2 bring zeros), so one kind of instruction serves all sizes
+  constexpr int NS32 = (HD + 31) / 32;
+  constexpr bool HALF_LAST = (HD % 32) != 0;
+  bf16x8_t q32[CT][NS32];
   int pos[CT], lo[CT];
   f32x4 o[CT][NS];
-  float m[CT], l[CT];
+  float m[CT];
+  f32x4 lacc[CT];           // sum of the probabilities of a column, from a product with a tile of ones
+  const int row = rb + j;
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
-    const int hh = c % GH, tt = c / GH;
-    const int hj = hc * GH + hh, row = rb + tt * 16 + j;
+    const int hj = hc * CT + c;
     const bool ok = hj < G && row < qlen;
     pos[c] = ok ? ctx + row : -1;
     lo[c] = (window > 0 && pos[c] - window + 1 > 0) ? pos[c] - window + 1 : 0;
-    if (ok) load_row_operand(q + (size_t)(qstart + row) * q_row_stride + (size_t)(g * G + hj) * HD, qd, qreg[c]);
-    else zero_row_operand(qreg[c]);
+    const uint16_t* qrow = q + (size_t)(qstart + (ok ? row : row0)) * q_row_stride + (size_t)(g * G + (ok ? hj : 0)) * HD;
+#pragma unroll
+    for (int st = 0; st < NS32; ++st) {
+      const bool real = ok && !(HALF_LAST && st == NS32 - 1 && qd >= 2);
+      const uint4 v = real ? *reinterpret_cast<const uint4*>(qrow + st * 32 + qd * 8) : make_uint4(0u, 0u, 0u, 0u);
+      q32[c][st] = __builtin_bit_cast(bf16x8_t, v);
+    }
     m[c] = -INFINITY;
-    l[c] = 0.f;
+    lacc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int n = 0; n < NS; ++n) o[c][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
-  const int last_row = (rb + TT * 16 < qlen ? rb + TT * 16 : qlen) - 1;
-  const int key_hi = ctx + last_row;
-  const int key_lo = (window > 0 && ctx + rb - window + 1 > 0) ? ctx + rb - window + 1 : 0;
+  const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+
+  // ---- keys the workgroup needs: those its rows may see
+  const int key_hi = ctx + row0 + rows_here - 1;
+  const int key_lo = (window > 0 && ctx + row0 - window + 1 > 0) ? ctx + row0 - window + 1 : 0;
+  const int wave_hi = ctx + rb + 15;                                    // last key any row of this wave sees
+  const int wave_lo = (window > 0 && ctx + rb - window + 1 > 0) ? ctx + rb - window + 1 : 0;
+  const int wave_lo_last = (window > 0 && ctx + rb + 15 - window + 1 > 0) ? ctx + rb + 15 - window + 1 : 0;
+  const bool wave_live = rb < qlen;
   const int* bt = block_tables + (size_t)sidx * bt_stride;
-  for (int t = key_lo / 16; t <= key_hi / 16; ++t)
-    attn_tile<CT>(t * 16, key_lo, key_hi, bt, ps, num_pages, nkv, g, k_pages, v_pages, qreg, pos, lo, scale_log2, o, m,
-                  l, lane);
+  const int t_begin = key_lo / PF_KT, t_end = key_hi / PF_KT;          // inclusive
+
+  // staging: K tile = 32 keys x HD/8 pieces of 16 bytes; V^T tile = HD dims x 8 quads of 4 keys (8 bytes)
+  constexpr int KPIECES = PF_KT * (HD / 8), KPT = (KPIECES + PF_WAVES * 64 - 1) / (PF_WAVES * 64);
+  constexpr int VPIECES = HD * 8, VPT = (VPIECES + PF_WAVES * 64 - 1) / (PF_WAVES * 64);
+  uint4 kreg[KPT];
+  uint2 vreg[VPT];
+  bool bad = false;
+  // Page numbers are read one tile ahead of the keys and values they lead to, so that a tile's loads
+  // do not wait for the block table: pgk[i] for the key row of K piece i, pgv for this thread's quad of V.
+  // -2: the keys are not needed (outside the rows' range).
+  int pgk[KPT], pgv;
+  // page size: a shift when it is a power of two (the usual case), a division otherwise
+  const int ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;
+  auto page_index = [&](int key) { return ps_shift >= 0 ? key >> ps_shift : key / ps; };
+  auto page_offset = [&](int key) { return ps_shift >= 0 ? key & (ps - 1) : key % ps; };
+  const size_t page_elems = (size_t)nkv * ps * HD;                 // elements of one page (all heads)
+  // what does not change from tile to tile
+  int k_row[KPT], k_col[KPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    const int pc = tid + i * PF_WAVES * 64;
+    k_row[i] = pc / (HD / 8);
+    k_col[i] = (pc - k_row[i] * (HD / 8)) * 8;
+  }
+  const int v_quad = tid & 7;
+  const uint16_t* k_base = k_pages + (size_t)g * ps * HD;
+  const uint16_t* v_base = v_pages + (size_t)g * HD * ps;
+  auto clampk = [&](int key) { return key < key_lo ? key_lo : (key > key_hi ? key_hi : key); };
+  // per thread, once: where its pieces lie within a page row / a tile
+  int k_off[KPT];                      // column of the piece within its key row
+  size_t v_dim_off[VPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) k_off[i] = k_col[i];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int dim = (tid + i * PF_WAVES * 64) >> 3;
+    v_dim_off[i] = (size_t)(dim < HD ? dim : HD - 1) * ps;
+  }
+  auto load_pages = [&](int t) {
+    const int t0 = t * PF_KT;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) pgk[i] = bt[page_index(clampk(t0 + k_row[i]))];
+    pgv = bt[page_index(clampk(t0 + v_quad * 4))];        // clamping stays within the quad's page when it is needed
+  };
+  auto load_tile = [&](int t) {
+    const int t0 = t * PF_KT;
+    const int key0 = t0 + v_quad * 4;
+    if (t0 >= key_lo && t0 + PF_KT - 1 <= key_hi) {
+      // every key of the tile is one of the request's: no clamping, no masks
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const bool page_ok = (unsigned)pgk[i] < (unsigned)num_pages;
+        bad |= !page_ok && (KPIECES % (PF_WAVES * 64) == 0 || tid + i * PF_WAVES * 64 < KPIECES);
+        const int key = t0 + (k_row[i] & (PF_KT - 1));
+        kreg[i] = *reinterpret_cast<const uint4*>(k_base + (size_t)(page_ok ? pgk[i] : 0) * page_elems +
+                                                  page_offset(key) * HD + k_off[i]);
+      }
+      const bool vpage_ok = (unsigned)pgv < (unsigned)num_pages;
+      bad |= !vpage_ok;
+      const uint16_t* vq = v_base + (size_t)(vpage_ok ? pgv : 0) * page_elems + page_offset(key0);
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) vreg[i] = *reinterpret_cast<const uint2*>(vq + v_dim_off[i]);
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int key = t0 + k_row[i], keyc = clampk(key);
+      const bool need = key == keyc && (KPIECES % (PF_WAVES * 64) == 0 || tid + i * PF_WAVES * 64 < KPIECES);
+      const bool page_ok = (unsigned)pgk[i] < (unsigned)num_pages;
+      bad |= need && !page_ok;
+      const uint4 v = *reinterpret_cast<const uint4*>(k_base + (size_t)(page_ok ? pgk[i] : 0) * page_elems +
+                                                     page_offset(keyc) * HD + k_off[i]);
+      kreg[i] = need && page_ok ? v : make_uint4(0u, 0u, 0u, 0u);
+    }
+    const bool vneed = key0 + 3 >= key_lo && key0 <= key_hi;
+    const bool vpage_ok = (unsigned)pgv < (unsigned)num_pages;
+    bad |= vneed && !vpage_ok;
+    // keys outside the request's range are not its data: zero them (16 bits each)
+    const uint32_t m0 = (key0 >= key_lo && key0 <= key_hi) ? 0x0000ffffu : 0u;
+    const uint32_t m1 = (key0 + 1 >= key_lo && key0 + 1 <= key_hi) ? 0xffff0000u : 0u;
+    const uint32_t m2 = (key0 + 2 >= key_lo && key0 + 2 <= key_hi) ? 0x0000ffffu : 0u;
+    const uint32_t m3 = (key0 + 3 >= key_lo && key0 + 3 <= key_hi) ? 0xffff0000u : 0u;
+    const uint32_t mx = vpage_ok ? (m0 | m1) : 0u, my = vpage_ok ? (m2 | m3) : 0u;
+    // the quad lies within one page (the page size is a multiple of 4); its place there is the same for all dims
+    const uint16_t* vq = v_base + (size_t)(vpage_ok ? pgv : 0) * page_elems + page_offset(clampk(key0) & ~3);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const uint2 v = *reinterpret_cast<const uint2*>(vq + v_dim_off[i]);
+      vreg[i] = make_uint2(v.x & mx, v.y & my);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int pc = tid + i * PF_WAVES * 64;
+      const int kr = pc / (HD / 8), dp = pc - kr * (HD / 8);
+      if (pc < KPIECES) *reinterpret_cast<uint4*>(&ks[buf][kr][dp * 8]) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int pc = tid + i * PF_WAVES * 64;
+      const int dim = pc >> 3, quad = pc & 7;
+      // quad = 4 kt + qd holds the keys 16 kt + 4 qd .. + 3: they go to the places 8 qd + 4 kt .. + 3
+      if (pc < VPIECES) *reinterpret_cast<uint2*>(&vs[buf][dim][(quad & 3) * 8 + (quad >> 2) * 4]) = vreg[i];
+    }
+  };
+
+  load_pages(t_begin);
+  load_tile(t_begin);
+  if (t_begin < t_end) load_pages(t_begin + 1);
+  store_tile(0);
+  __syncthreads();
+  for (int t = t_begin; t <= t_end; ++t) {
+    const int buf = (t - t_begin) & 1;
+    const bool more = t < t_end;
+    if (more) {
+      load_tile(t + 1);                        // with the page numbers read a round ago
+      if (t + 2 <= t_end) load_pages(t + 2);
+    }
+    const int t0 = t * PF_KT;
+    if (wave_live && t0 <= wave_hi && t0 + PF_KT - 1 >= wave_lo) {
+      // ---- S^T = K Q^T for the two tiles of 16 keys
+      f32x4 sc[CT][2];
+#pragma unroll
+      for (int c = 0; c < CT; ++c) { sc[c][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; sc[c][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const uint16_t* krow = &ks[buf][kt * 16 + j][0];
+#pragma unroll
+        for (int st = 0; st < NS32; ++st) {
+          const bool real = !(HALF_LAST && st == NS32 - 1 && qd >= 2);
+          const uint4 kv = real ? *reinterpret_cast<const uint4*>(krow + st * 32 + qd * 8) : make_uint4(0u, 0u, 0u, 0u);
+          const bf16x8_t ka = __builtin_bit_cast(bf16x8_t, kv);
+#pragma unroll
+          for (int c = 0; c < CT; ++c) sc[c][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q32[c][st], sc[c][kt], 0, 0, 0);
+        }
+      }
+      // ---- softmax statistics per column; probabilities as the B operand of the second product.
+      // Only tiles that touch the diagonal or a window's lower edge need the mask (the same for the whole wave).
+      const bool need_mask = (t0 + PF_KT - 1 > ctx + rb) || (window > 0 && t0 < wave_lo_last) || rb + 15 >= qlen;
+      bf16x8_t pb[CT];
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        float sv[8];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sv[kt * 4 + r] = sc[c][kt][r];
+        if (need_mask) {
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int kr = t0 + kt * 16 + 4 * qd + r;
+              const bool ok = pos[c] >= 0 && kr <= pos[c] && kr >= lo[c];
+              sv[kt * 4 + r] = ok ? sv[kt * 4 + r] : -INFINITY;
+            }
+        }
+        // the scale is positive: the maximum is taken of the raw scores and scaled once
+        float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, IA_WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE)) * scale_log2;
+        // The reference point of the exponentials follows the running maximum lazily: it moves only when the
+        // maximum has grown by more than 2^PF_LAZY, so probabilities stay below 2^PF_LAZY (exact in fp32 and in
+        // the relative rounding of bf16) and the accumulators are rescaled rarely.
+        const bool move = tmax > m[c] + PF_LAZY;           // also the first tile (m = -inf) and never for -inf
+        const float m_new = move ? tmax : m[c];
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        // probabilities are rounded to bf16 by the hardware conversion (nearest even); their sum is taken by the
+        // matrix cores of the same rounded values (a product with a tile of ones), so that numerator and
+        // denominator of the softmax agree and the vector units are spared the additions
+        uint32_t pk[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          f32x2_t e = {__builtin_amdgcn_exp2f(fmaf(sv[2 * r], scale_log2, -m_safe)),
+                       __builtin_amdgcn_exp2f(fmaf(sv[2 * r + 1], scale_log2, -m_safe))};
+          pk[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(e, bf16x2_t));
+        }
+        if (__any(move)) {
+          const float corr = __builtin_amdgcn_exp2f(m[c] - m_safe);      // 1 for the columns that did not move
+          lacc[c] *= corr;
+#pragma unroll
+          for (int n = 0; n < NS; ++n) o[c][n] *= corr;
+        }
+        m[c] = m_new;
+        pb[c] = __builtin_bit_cast(bf16x8_t, make_uint4(pk[0], pk[1], pk[2], pk[3]));
+        lacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[c], lacc[c], 0, 0, 0);
+      }
+      // ---- O^T += V^T P^T
+#pragma unroll
+      for (int n = 0; n < NS; ++n) {
+        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&vs[buf][n * 16 + j][qd * 8]));
+#pragma unroll
+        for (int c = 0; c < CT; ++c) o[c][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[c], o[c][n], 0, 0, 0);
+      }
+    }
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+  if (bad) s_poison = 1;      // a key that is needed has no page in the block table: the result is NaN
+  __syncthreads();
+  const bool poison = s_poison != 0;
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     if (pos[c] < 0) continue;
-    const int hh = c % GH, tt = c / GH;
-    const int row = rb + tt * 16 + j;
-    const float inv = 1.0f / l[c];
-    uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride + (size_t)(g * G + hc * GH + hh) * HD + 4 * qd;
+    const float inv = poison ? __uint_as_float(0x7fc00000u) : 1.0f / lacc[c][0];
+    uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride + (size_t)(g * G + hc * CT + c) * HD + 4 * qd;
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
       uint2 w;
@@ -361,22 +600,33 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
                                int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
                                float scale, int window, hipStream_t stream) {
   if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
-      bt_stride <= 0)
+      bt_stride <= 0 || !(scale > 0.f))
     return IA_ERR_BAD_ARG;
   if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
   if (num_tiles == 0) return IA_OK;
-  constexpr int CT = PREFILL_CT;
   const int G = nh / nkv;
-  int GH = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
-  if (GH > CT) GH = CT;
-  const int HC = (G + GH - 1) / GH, TT = CT / GH;
-  if (nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
+  // query heads of one key/value head that a wave takes together: two keep a wave's accumulators within 256
+  // vector registers, so that two waves share a SIMD and one's softmax overlaps the other's products
+  int CT = G >= 2 ? 2 : 1;
+  if (const char* e = getenv("IA_PF_CT")) { int v = atoi(e); if (v == 1 || v == 2 || (v == 4 && PF_CT_MAX == 4)) CT = v; }   // experiment
+  const int HC = (G + CT - 1) / CT;
+  if ((long long)nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid(num_tiles, nkv * HC, 64 / (16 * TT));
-  attn_prefill_kernel<<<grid, 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
-                                               (const uint16_t*)v_pages, (uint16_t*)out, out_row_stride, seq_starts,
-                                               seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages,
-                                               scale_log2, window, GH);
+  dim3 grid(num_tiles, nkv * HC);
+#define PF_LAUNCH(C)                                                                                              \
+  attn_prefill_kernel<C><<<grid, PF_WAVES * 64, 0, stream>>>(                                                     \
+      (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
+      out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window)
+  if (CT == 1) PF_LAUNCH(1);
+  else if (CT == 2) PF_LAUNCH(2);
+  else {
+#if IA_HEAD_DIM <= 128
+    PF_LAUNCH(4);
+#else
+    return IA_ERR_UNSUPPORTED;
+#endif
+  }
+#undef PF_LAUNCH
   IA_LAUNCH_CHECK();
   return IA_OK;
 }

@@ -108,7 +108,10 @@ def library_plan(name: str) -> Dict:
         d = int(name[len("attn_d"):])
         if d not in SUPPORTED_HEAD_DIMS:
             raise BuildError(f"no MFMA attention kernel for head size {d}: supported are multiples of 16 up to 256")
-        return {"sources": ["attention_mfma.hip"], "defines": [f"-DIA_HEAD_DIM={d}"]}
+        # accumulators of the matrix cores in ordinary vector registers: the softmax rescales them with
+        # vector instructions, which cannot reach the accumulation registers
+        return {"sources": ["attention_mfma.hip"],
+                "defines": [f"-DIA_HEAD_DIM={d}", "-mllvm", "-amdgpu-mfma-vgpr-form"]}
     raise BuildError(f"unknown library {name!r}")
 
 
