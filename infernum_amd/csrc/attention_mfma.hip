@@ -25,7 +25,6 @@
 // zeroed (values) or masked (scores): a stale or poisoned page never leaks in.
 // A key that is needed but has no page in the block table gives NaN, not a fault.
 #include "common.h"
-#include <stdlib.h>
 
 #ifndef IA_HEAD_DIM
 #error "compile with -DIA_HEAD_DIM=<head size>"
@@ -282,26 +281,29 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
-#define PF_WAVES 4
-#define PF_KT 32
+#define PF_KT (HD <= 128 ? 64 : 32)   // keys per round of the main loop (one barrier), in parts of 32
+#define PF_SUBS (PF_KT / 32)
+#define PF_QPT (PF_KT / 4)             // quads of 4 keys per round
 #define PF_KROW (HD + 8)        // bf16 per key row in LDS: 16 bytes of padding spread the banks
 #define PF_VROW 40              // bf16 per dim row of V^T in LDS (32 keys + 8 of padding)
 #define PF_CT_MAX (HD <= 128 ? 4 : 2)
 #define PF_LAZY 6.0f            // log2 of how far the running maximum may run ahead of the reference point
 
-template <int CT>
-__global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
+template <int CT, int HGW>
+__global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
     const int* __restrict__ seq_starts, const int* __restrict__ seq_ctx, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, float scale_log2,
     int window) {
   __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KT][PF_KROW];
-  __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD][PF_VROW];
+  __shared__ __attribute__((aligned(16))) uint16_t vs[2][PF_SUBS][HD][PF_VROW];
   __shared__ int s_poison;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, qd = lane >> 4;
+  constexpr int PF_THREADS = 4 * HGW * 64;
+  const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, qd = lane >> 4;
+  const int wave = (tid >> 6) & 3, hgw = tid >> 8;      // group of 16 rows, group of CT heads
   const int sidx = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
-  const int G = nh / nkv, HC = (G + CT - 1) / CT;
+  const int G = nh / nkv, HC = (G + CT * HGW - 1) / (CT * HGW);
   const int g = blockIdx.y / HC, hc = blockIdx.y - g * HC;
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
   const int rows_here = (qlen - row0) < 64 ? (qlen - row0) : 64;      // rows of this workgroup (>= 1)
@@ -321,7 +323,7 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   const int row = rb + j;
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
-    const int hj = hc * CT + c;
+    const int hj = (hc * HGW + hgw) * CT + c;
     const bool ok = hj < G && row < qlen;
     pos[c] = ok ? ctx + row : -1;
     lo[c] = (window > 0 && pos[c] - window + 1 > 0) ? pos[c] - window + 1 : 0;
@@ -350,8 +352,8 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   const int t_begin = key_lo / PF_KT, t_end = key_hi / PF_KT;          // inclusive
 
   // staging: K tile = 32 keys x HD/8 pieces of 16 bytes; V^T tile = HD dims x 8 quads of 4 keys (8 bytes)
-  constexpr int KPIECES = PF_KT * (HD / 8), KPT = (KPIECES + PF_WAVES * 64 - 1) / (PF_WAVES * 64);
-  constexpr int VPIECES = HD * 8, VPT = (VPIECES + PF_WAVES * 64 - 1) / (PF_WAVES * 64);
+  constexpr int KPIECES = PF_KT * (HD / 8), KPT = (KPIECES + PF_THREADS - 1) / (PF_THREADS);
+  constexpr int VPIECES = HD * PF_QPT, VPT = (VPIECES + PF_THREADS - 1) / (PF_THREADS);
   uint4 kreg[KPT];
   uint2 vreg[VPT];
   bool bad = false;
@@ -368,11 +370,11 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   int k_row[KPT], k_col[KPT];
 #pragma unroll
   for (int i = 0; i < KPT; ++i) {
-    const int pc = tid + i * PF_WAVES * 64;
+    const int pc = tid + i * PF_THREADS;
     k_row[i] = pc / (HD / 8);
     k_col[i] = (pc - k_row[i] * (HD / 8)) * 8;
   }
-  const int v_quad = tid & 7;
+  const int v_quad = tid & (PF_QPT - 1);
   const uint16_t* k_base = k_pages + (size_t)g * ps * HD;
   const uint16_t* v_base = v_pages + (size_t)g * HD * ps;
   auto clampk = [&](int key) { return key < key_lo ? key_lo : (key > key_hi ? key_hi : key); };
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   for (int i = 0; i < KPT; ++i) k_off[i] = k_col[i];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int dim = (tid + i * PF_WAVES * 64) >> 3;
+    const int dim = (tid + i * PF_THREADS) / PF_QPT;
     v_dim_off[i] = (size_t)(dim < HD ? dim : HD - 1) * ps;
   }
   auto load_pages = [&](int t) {
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
 #pragma unroll
       for (int i = 0; i < KPT; ++i) {
         const bool page_ok = (unsigned)pgk[i] < (unsigned)num_pages;
-        bad |= !page_ok && (KPIECES % (PF_WAVES * 64) == 0 || tid + i * PF_WAVES * 64 < KPIECES);
+        bad |= !page_ok && (KPIECES % (PF_THREADS) == 0 || tid + i * PF_THREADS < KPIECES);
         const int key = t0 + (k_row[i] & (PF_KT - 1));
         kreg[i] = *reinterpret_cast<const uint4*>(k_base + (size_t)(page_ok ? pgk[i] : 0) * page_elems +
                                                   page_offset(key) * HD + k_off[i]);
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int key = t0 + k_row[i], keyc = clampk(key);
-      const bool need = key == keyc && (KPIECES % (PF_WAVES * 64) == 0 || tid + i * PF_WAVES * 64 < KPIECES);
+      const bool need = key == keyc && (KPIECES % (PF_THREADS) == 0 || tid + i * PF_THREADS < KPIECES);
       const bool page_ok = (unsigned)pgk[i] < (unsigned)num_pages;
       bad |= need && !page_ok;
       const uint4 v = *reinterpret_cast<const uint4*>(k_base + (size_t)(page_ok ? pgk[i] : 0) * page_elems +
@@ -442,16 +444,17 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      const int pc = tid + i * PF_WAVES * 64;
+      const int pc = tid + i * PF_THREADS;
       const int kr = pc / (HD / 8), dp = pc - kr * (HD / 8);
       if (pc < KPIECES) *reinterpret_cast<uint4*>(&ks[buf][kr][dp * 8]) = kreg[i];
     }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const int pc = tid + i * PF_WAVES * 64;
-      const int dim = pc >> 3, quad = pc & 7;
-      // quad = 4 kt + qd holds the keys 16 kt + 4 qd .. + 3: they go to the places 8 qd + 4 kt .. + 3
-      if (pc < VPIECES) *reinterpret_cast<uint2*>(&vs[buf][dim][(quad & 3) * 8 + (quad >> 2) * 4]) = vreg[i];
+      const int pc = tid + i * PF_THREADS;
+      const int dim = pc / PF_QPT, quad = pc & (PF_QPT - 1), sub = quad >> 3, q8 = quad & 7;
+      // within a part of 32 keys, quad q8 = 4 kt + qd holds the keys 16 kt + 4 qd .. + 3: they go to the places
+      // 8 qd + 4 kt .. + 3
+      if (pc < VPIECES) *reinterpret_cast<uint2*>(&vs[buf][sub][dim][(q8 & 3) * 8 + (q8 >> 2) * 4]) = vreg[i];
     }
   };
 
@@ -467,15 +470,17 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
       load_tile(t + 1);                        // with the page numbers read a round ago
       if (t + 2 <= t_end) load_pages(t + 2);
     }
-    const int t0 = t * PF_KT;
-    if (wave_live && t0 <= wave_hi && t0 + PF_KT - 1 >= wave_lo) {
+#pragma unroll
+    for (int sub = 0; sub < PF_SUBS; ++sub) {
+    const int t0 = t * PF_KT + sub * 32;
+    if (wave_live && t0 <= wave_hi && t0 + 31 >= wave_lo && t0 <= key_hi) {
       // ---- S^T = K Q^T for the two tiles of 16 keys
       f32x4 sc[CT][2];
 #pragma unroll
       for (int c = 0; c < CT; ++c) { sc[c][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; sc[c][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
-        const uint16_t* krow = &ks[buf][kt * 16 + j][0];
+        const uint16_t* krow = &ks[buf][sub * 32 + kt * 16 + j][0];
 #pragma unroll
         for (int st = 0; st < NS32; ++st) {
           const bool real = !(HALF_LAST && st == NS32 - 1 && qd >= 2);
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
       }
       // ---- softmax statistics per column; probabilities as the B operand of the second product.
       // Only tiles that touch the diagonal or a window's lower edge need the mask (the same for the whole wave).
-      const bool need_mask = (t0 + PF_KT - 1 > ctx + rb) || (window > 0 && t0 < wave_lo_last) || rb + 15 >= qlen;
+      const bool need_mask = (t0 + 31 > ctx + rb) || (window > 0 && t0 < wave_lo_last) || rb + 15 >= qlen;
       bf16x8_t pb[CT];
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
@@ -539,10 +544,11 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
       // ---- O^T += V^T P^T
 #pragma unroll
       for (int n = 0; n < NS; ++n) {
-        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&vs[buf][n * 16 + j][qd * 8]));
+        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&vs[buf][sub][n * 16 + j][qd * 8]));
 #pragma unroll
         for (int c = 0; c < CT; ++c) o[c][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[c], o[c][n], 0, 0, 0);
       }
+    }
     }
     if (more) store_tile(buf ^ 1);
     __syncthreads();
@@ -554,7 +560,8 @@ __global__ __launch_bounds__(PF_WAVES * 64) void attn_prefill_kernel(
   for (int c = 0; c < CT; ++c) {
     if (pos[c] < 0) continue;
     const float inv = poison ? __uint_as_float(0x7fc00000u) : 1.0f / lacc[c][0];
-    uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride + (size_t)(g * G + hc * CT + c) * HD + 4 * qd;
+    uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride +
+                     (size_t)(g * G + (hc * HGW + hgw) * CT + c) * HD + 4 * qd;
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
       uint2 w;
@@ -605,23 +612,27 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
   if (num_tiles == 0) return IA_OK;
   const int G = nh / nkv;
-  // query heads of one key/value head that a wave takes together: two keep a wave's accumulators within 256
-  // vector registers, so that two waves share a SIMD and one's softmax overlaps the other's products
+  // A wave takes 16 rows of CT query heads of one key/value head; two heads keep its accumulators within 256
+  // vector registers, so that two waves share a SIMD and one's softmax overlaps the other's products.  With
+  // four or more heads to a key/value head a workgroup has a second set of four waves for the next CT heads:
+  // twice the rows of Q per tile of keys that is brought in.
   int CT = G >= 2 ? 2 : 1;
-  if (const char* e = getenv("IA_PF_CT")) { int v = atoi(e); if (v == 1 || v == 2 || (v == 4 && PF_CT_MAX == 4)) CT = v; }   // experiment
-  const int HC = (G + CT - 1) / CT;
+  int HGW = G >= 2 * CT ? 2 : 1;
+  const int HC = (G + CT * HGW - 1) / (CT * HGW);
   if ((long long)nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(num_tiles, nkv * HC);
-#define PF_LAUNCH(C)                                                                                              \
-  attn_prefill_kernel<C><<<grid, PF_WAVES * 64, 0, stream>>>(                                                     \
+#define PF_LAUNCH(C, W)                                                                                           \
+  attn_prefill_kernel<C, W><<<grid, 4 * W * 64, 0, stream>>>(                                                     \
       (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
       out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window)
-  if (CT == 1) PF_LAUNCH(1);
-  else if (CT == 2) PF_LAUNCH(2);
+  if (CT == 1 && HGW == 1) PF_LAUNCH(1, 1);
+  else if (CT == 1) PF_LAUNCH(1, 2);
+  else if (CT == 2 && HGW == 1) PF_LAUNCH(2, 1);
+  else if (CT == 2) PF_LAUNCH(2, 2);
   else {
 #if IA_HEAD_DIM <= 128
-    PF_LAUNCH(4);
+    if (HGW == 1) PF_LAUNCH(4, 1); else PF_LAUNCH(4, 2);
 #else
     return IA_ERR_UNSUPPORTED;
 #endif
