@@ -123,7 +123,8 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
     float4 ds[RN_MAXV];
 #pragma unroll
     for (int c = 0; c < RN_MAXV; ++c) ds[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int k = 0; k < splits; ++k) {
+#pragma unroll 4
+    for (int k = 0; k < splits; ++k) {           // unrolled: the loads of several parts are in flight together
 #pragma unroll
       for (int c = 0; c < RN_MAXV; ++c) {
         const int i = (threadIdx.x + c * NT) * 4;
@@ -235,6 +236,7 @@ extern "C" int ia_residual_add(float* h, const void* delta, int act_dtype, int N
 template <typename TS>
 __device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t split_stride) {
   float v = to_float(p[0]);
+#pragma unroll 4
   for (int k = 1; k < splits; ++k) v += to_float(p[k * split_stride]);
   return v;
 }

@@ -47,12 +47,15 @@ template <> __device__ __forceinline__ void store_out<float>(float* p, float v) 
 template <> __device__ __forceinline__ void store_out<uint16_t>(uint16_t* p, float v) { *p = float_to_bf16_bits(v); }
 
 // part != nullptr: fp32 partial tiles go to part[split, m, n]; else the result goes to C (one split only).
-template <int MT, typename TO>
+// GLU (one split only): a wave takes 16 rows n of the first half of W and the 16 rows N/2 + n of the second,
+// and stores silu(first) * second to C[m, n], n < N/2.
+template <int MT, bool GLU, typename TO>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ X,
                                                                     const uint16_t* __restrict__ W,
                                                                     TO* __restrict__ C, float* __restrict__ part,
                                                                     int M, int N, int K, int chunks_per_split) {
   constexpr int XROW = SK_KC + SK_XPAD;
+  constexpr int TPW = GLU ? 2 : 1;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][XROW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
@@ -61,12 +64,17 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   const int nchunks = (K + SK_KC - 1) / SK_KC;
   const int c0 = split * chunks_per_split;
   const int c1 = min(nchunks, c0 + chunks_per_split);
+  const int NO = GLU ? N / 2 : N;                      // columns of the result
 
-  const int n_row = (n_base + r < N) ? n_base + r : N - 1;
-  const uint16_t* wrow = W + (size_t)n_row * K;
-  f32x4 acc[MT];
+  const int n_row = (n_base + r < NO) ? n_base + r : NO - 1;
+  const uint16_t* wrow[TPW];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < TPW; ++t) wrow[t] = W + ((size_t)n_row + (size_t)t * NO) * K;
+  f32x4 acc[TPW][MT];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   // the chunk of X is MT*16 rows of 256 values = MT*512 pieces of 16 bytes, spread over the 256 threads
   constexpr int XPIECES = MT * 16 * (SK_KC / 8);
@@ -91,13 +99,15 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
       *reinterpret_cast<uint4*>(&xs[buf][row][kk]) = xreg[i];
     }
   };
-  uint4 wcur[SK_NLD], wnext[SK_NLD];
-  auto load_w = [&](int c, uint4 (&dst)[SK_NLD]) {
+  uint4 wcur[TPW][SK_NLD], wnext[TPW][SK_NLD];
+  auto load_w = [&](int c, uint4 (&dst)[TPW][SK_NLD]) {
 #pragma unroll
-    for (int i = 0; i < SK_NLD; ++i) {
-      const int k = c * SK_KC + (i * 4 + q) * 8;
-      dst[i] = (k < K) ? load_stream_16(wrow + k) : make_uint4(0u, 0u, 0u, 0u);
-    }
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int i = 0; i < SK_NLD; ++i) {
+        const int k = c * SK_KC + (i * 4 + q) * 8;
+        dst[t][i] = (k < K) ? load_stream_16(wrow[t] + k) : make_uint4(0u, 0u, 0u, 0u);
+      }
   };
 
   if (c0 < c1) {
@@ -116,17 +126,21 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
     }
 #pragma unroll
     for (int i = 0; i < SK_NLD; ++i) {
-      const bf16x8 wv = __builtin_bit_cast(bf16x8, wcur[i]);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const uint4 xv = *reinterpret_cast<const uint4*>(&xs[buf][mt * 16 + r][(i * 4 + q) * 8]);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, __builtin_bit_cast(bf16x8, xv), acc[mt], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < TPW; ++t)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wcur[t][i]),
+                                                               __builtin_bit_cast(bf16x8, xv), acc[t][mt], 0, 0, 0);
       }
     }
     if (more) {
       store_x(buf ^ 1);
 #pragma unroll
-      for (int i = 0; i < SK_NLD; ++i) wcur[i] = wnext[i];
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int i = 0; i < SK_NLD; ++i) wcur[t][i] = wnext[t][i];
     }
     __syncthreads();
   }
@@ -136,20 +150,27 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     if (m >= M) continue;
-    if (part) {
+    if (GLU) {
+      TO* o = C + (size_t)m * NO + n;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float gt = acc[0][mt][e], up = acc[TPW - 1][mt][e];
+        if (n + e < NO) store_out<TO>(o + e, gt / (1.0f + expf(-gt)) * up);
+      }
+    } else if (part) {
       float* o = part + ((size_t)split * M + m) * N + n;
       if (n + 3 < N && (N & 3) == 0) {
-        *reinterpret_cast<f32x4*>(o) = acc[mt];
+        *reinterpret_cast<f32x4*>(o) = acc[0][mt];
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (n + e < N) o[e] = acc[mt][e];
+          if (n + e < N) o[e] = acc[0][mt][e];
       }
     } else {
       TO* o = C + (size_t)m * N + n;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (n + e < N) store_out<TO>(o + e, acc[mt][e]);
+        if (n + e < N) store_out<TO>(o + e, acc[0][mt][e]);
     }
   }
 }
@@ -187,17 +208,18 @@ static int skinny_splits(int N, int K) {
 // Number of K splits the kernel uses for a weight [N, K] (a function of N and K only).
 extern "C" int ia_gemm_skinny_splits(int N, int K) { return (N > 0 && K > 0) ? skinny_splits(N, K) : 0; }
 
-template <typename TO>
+template <bool GLU, typename TO>
 static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K, int splits,
                          hipStream_t stream) {
   const int nchunks = (K + SK_KC - 1) / SK_KC;
   const int cps = (nchunks + splits - 1) / splits;
-  dim3 grid((N + SK_BN - 1) / SK_BN, splits);
+  const int NO = GLU ? N / 2 : N;
+  dim3 grid((NO + SK_BN - 1) / SK_BN, splits);
   switch ((M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 2: gemm_skinny_kernel<2, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 3: gemm_skinny_kernel<3, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 4: gemm_skinny_kernel<4, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 1: gemm_skinny_kernel<1, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 2: gemm_skinny_kernel<2, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 3: gemm_skinny_kernel<3, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 4: gemm_skinny_kernel<4, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
     default: return IA_ERR_UNSUPPORTED;
   }
   IA_LAUNCH_CHECK();
@@ -228,15 +250,20 @@ extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dty
   if (out_dtype != IA_F32 && out_dtype != IA_BF16) return IA_ERR_BAD_ARG;
   const int splits = skinny_splits(N, K);
   if (splits > 65535) return IA_ERR_UNSUPPORTED;
-  const bool via_workspace = splits > 1 || epilogue != SK_EPI_NONE || C == nullptr;
-  if (via_workspace && (!workspace || workspace_floats < (size_t)splits * M * N)) return IA_ERR_BAD_ARG;
   const uint16_t* x = (const uint16_t*)X;
   const uint16_t* w = (const uint16_t*)W;
-  if (!via_workspace) {
-    if (out_dtype == IA_F32) return launch_skinny<float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
-    return launch_skinny<uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
+  if (splits == 1 && epilogue == SK_EPI_SWIGLU && C != nullptr) {
+    // one pass: both halves of W in the same wave, the activation in the epilogue
+    if (out_dtype == IA_F32) return launch_skinny<true, float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
+    return launch_skinny<true, uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
   }
-  const int rc = launch_skinny<float>(x, w, nullptr, workspace, M, N, K, splits, stream);
+  const bool via_workspace = splits > 1 || epilogue != SK_EPI_NONE || C == nullptr;
+  if (via_workspace && (!workspace || workspace_floats < (size_t)splits * M * N)) return IA_ERR_BAD_ARG;
+  if (!via_workspace) {
+    if (out_dtype == IA_F32) return launch_skinny<false, float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
+    return launch_skinny<false, uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
+  }
+  const int rc = launch_skinny<false, float>(x, w, nullptr, workspace, M, N, K, splits, stream);
   if (rc != IA_OK || C == nullptr) return rc;
   if (out_dtype == IA_F32) return launch_join<float>(workspace, (float*)C, M, N, splits, epilogue, stream);
   return launch_join<uint16_t>(workspace, (uint16_t*)C, M, N, splits, epilogue, stream);

@@ -248,7 +248,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     _need(epilogue is None or N % 2 == 0, "gemm_skinny: the swiglu epilogue needs an even N")
     splits = gemm_skinny_splits(N, K)
     ws = None
-    if splits > 1 or epilogue is not None:
+    if splits > 1:
         ws = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
     if keep_split and epilogue is None and splits > 1:
         _ok(_core().ia_gemm_skinny(_p(a), _p(w), None, 0, M, N, K, 0, _p(ws), ctypes.c_size_t(ws.numel()),
