@@ -113,15 +113,38 @@ def time_decode(engine, batch, steps, warmup, prompt_len=PROMPT_LEN):
     return dt, ctx_mid
 
 
+def time_prefill(engine, cfg, dtype: str, repeats: int = 3) -> dict:
+    """One prompt of 2,048 tokens in one step, logits at its last place; the best of a few runs after the first."""
+    import torch
+    from infernum_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
+    best = None
+    for i in range(repeats):
+        sync()
+        t0 = time.perf_counter()
+        engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
+        sync()
+        t = time.perf_counter() - t0
+        engine.end(f"p{i}")
+        if i > 0:
+            best = t if best is None else min(best, t)
+    flops = prefill_flops(cfg, PREFILL_TOKENS)
+    return {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
+            "frac": round(flops / best / (PEAK_TFLOPS[dtype] * 1e12), 4)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=240)      # 16 + 240 = the 256 generated tokens of the workload
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (both are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only the prefill of 2,048 tokens, a few times (for profiles); prints its record alone")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
@@ -137,7 +160,7 @@ def main() -> int:
     cfg = LlamaConfig.from_dict(raw)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
-    max_batch = max(a.batch, 1 if a.no_points else 64)
+    max_batch = 1 if a.prefill_only else max(a.batch, 1 if a.no_points else 64)
     tokens_needed = max(max_batch * (PROMPT_LEN + a.steps + a.warmup + PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
     t_load = time.perf_counter()
     engine = Engine.from_config(cfg, seed=0, dtype=dtype,
@@ -147,6 +170,10 @@ def main() -> int:
                                 max_tokens_per_step=8192)
     sync()
     print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
+
+    if a.prefill_only:
+        print(json.dumps({"prefill": time_prefill(engine, cfg, a.dtype, repeats=max(3, a.warmup))}))
+        return 0
 
     # ---- the timed K steps at the headline batch ---------------------------------
     dt, ctx_mid = time_decode(engine, a.batch, a.steps, a.warmup)
@@ -175,23 +202,7 @@ def main() -> int:
             d, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)))
             points[f"decode_b{b}"] = round(b * steps / d, 2)
         out["points"] = points
-        # ---- prefill of one 2,048-token prompt ---------------------------------------
-        from infernum_amd.engine import StepEntry
-        g = torch.Generator().manual_seed(7)
-        prompt = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
-        best = None
-        for i in range(3):
-            sync()
-            t0 = time.perf_counter()
-            engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
-            sync()
-            t = time.perf_counter() - t0
-            engine.end(f"p{i}")
-            if i > 0:
-                best = t if best is None else min(best, t)
-        flops = prefill_flops(cfg, PREFILL_TOKENS)
-        out["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
-                          "frac": round(flops / best / (PEAK_TFLOPS[a.dtype] * 1e12), 4)}
+        out["prefill"] = time_prefill(engine, cfg, a.dtype)
     print(json.dumps(out))
     return 0
 

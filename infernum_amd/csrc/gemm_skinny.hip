@@ -47,19 +47,22 @@ template <> __device__ __forceinline__ void store_out<float>(float* p, float v) 
 template <> __device__ __forceinline__ void store_out<uint16_t>(uint16_t* p, float v) { *p = float_to_bf16_bits(v); }
 
 // part != nullptr: fp32 partial tiles go to part[split, m, n]; else the result goes to C (one split only).
-// GLU (one split only): a wave takes 16 rows n of the first half of W and the 16 rows N/2 + n of the second,
-// and stores silu(first) * second to C[m, n], n < N/2.
+// GLU (one split only): a workgroup takes 32 columns n of the result; waves 0 and 1 multiply with the rows n
+// of the first half of W, waves 2 and 3 with the rows N/2 + n of the second half; the halves meet in LDS and
+// silu(first) * second goes to C[m, n], n < N/2.
 template <int MT, bool GLU, typename TO>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ X,
                                                                     const uint16_t* __restrict__ W,
                                                                     TO* __restrict__ C, float* __restrict__ part,
                                                                     int M, int N, int K, int chunks_per_split) {
   constexpr int XROW = SK_KC + SK_XPAD;
-  constexpr int TPW = GLU ? 2 : 1;
+  constexpr int TPW = 1;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][XROW];
+  __shared__ f32x4 glu_up[GLU ? 2 : 1][GLU ? MT : 1][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
-  const int n_base = blockIdx.x * SK_BN + wave * 16;
+  const int half = GLU ? wave >> 1 : 0;                // which half of W this wave multiplies with
+  const int n_base = GLU ? blockIdx.x * (SK_BN / 2) + (wave & 1) * 16 : blockIdx.x * SK_BN + wave * 16;
   const int split = blockIdx.y;
   const int nchunks = (K + SK_KC - 1) / SK_KC;
   const int c0 = split * chunks_per_split;
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   const int n_row = (n_base + r < NO) ? n_base + r : NO - 1;
   const uint16_t* wrow[TPW];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t) wrow[t] = W + ((size_t)n_row + (size_t)t * NO) * K;
+  for (int t = 0; t < TPW; ++t) wrow[t] = W + ((size_t)n_row + (size_t)half * NO) * K;
   f32x4 acc[TPW][MT];
 #pragma unroll
   for (int t = 0; t < TPW; ++t)
@@ -146,16 +149,25 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   }
   // lane holds D[i = 4 q + e][j = r]: i counts rows of W in the tile, j rows of X
   const int n = n_base + 4 * q;
+  if (GLU) {
+    if (half == 1) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) glu_up[wave & 1][mt][lane] = acc[0][mt];
+    }
+    __syncthreads();
+    if (half == 1) return;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     if (m >= M) continue;
     if (GLU) {
+      const f32x4 up = glu_up[wave & 1][mt][lane];
       TO* o = C + (size_t)m * NO + n;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float gt = acc[0][mt][e], up = acc[TPW - 1][mt][e];
-        if (n + e < NO) store_out<TO>(o + e, gt / (1.0f + expf(-gt)) * up);
+        const float gt = acc[0][mt][e];
+        if (n + e < NO) store_out<TO>(o + e, gt / (1.0f + expf(-gt)) * up[e]);
       }
     } else if (part) {
       float* o = part + ((size_t)split * M + m) * N + n;
@@ -214,7 +226,8 @@ static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* par
   const int nchunks = (K + SK_KC - 1) / SK_KC;
   const int cps = (nchunks + splits - 1) / splits;
   const int NO = GLU ? N / 2 : N;
-  dim3 grid((NO + SK_BN - 1) / SK_BN, splits);
+  const int cols = GLU ? SK_BN / 2 : SK_BN;           // columns of the result per workgroup
+  dim3 grid((NO + cols - 1) / cols, splits);
   switch ((M + 15) / 16) {
     case 1: gemm_skinny_kernel<1, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
     case 2: gemm_skinny_kernel<2, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
