@@ -106,6 +106,20 @@ def test_mixed_with_page_reuse(models, name, dtype):
     assert eng.cache.free_pages(0) == num_pages
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_no_fast_kernel_takes(tmp_path, dtype):
+    """Head size 20, width 100, feed-forward width 150, vocabulary 333, pages of 5 tokens: every kernel either
+    takes the size or hands over to a plain one; the logits are right all the same."""
+    d = str(tmp_path / "D")
+    TM.write_tiny("D", d, dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    cfg, w = P.read_model(d)
+    reqs = TT.make_requests(cfg["vocab_size"], (23, 70, 9), seed=4)
+    ref = {r: P.forward(cfg, w, toks) for r, toks in reqs.items()}
+    for trace in (TT.trace_whole(reqs), TT.trace_portions(reqs), TT.trace_tail_one_by_one(reqs, 12)):
+        got = TT.run_steps(_engine(d, dtype, 5, 40), trace)
+        _check(got, ref, dtype, f"D {dtype}")
+
+
 def test_cutting_does_not_change_fp32_logits(models):
     """In the 32-bit path a position's logits are the same bits however the tokens
     are cut into steps: each output is one chain of operations in a fixed order."""

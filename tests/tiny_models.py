@@ -32,13 +32,22 @@ TINY_C = dict(
     max_window_layers=2,
 )
 
+# D: sizes that no fast kernel takes: a head size that is no multiple of 16, a width and a feed-forward
+# width that are no multiples of 4, an odd vocabulary: the plain kernels (or the library product) must serve.
+TINY_D = dict(
+    model_type="llama", num_hidden_layers=2, hidden_size=100, num_attention_heads=5, num_key_value_heads=5,
+    head_dim=20, intermediate_size=150, vocab_size=333, rope_theta=10000.0, rms_norm_eps=1e-5,
+    tie_word_embeddings=True, max_position_embeddings=512,
+)
+
 SPEC_KW = {
     "A": dict(norm_init=("ones",)),
     "B": dict(norm_init=("uniform", 0.5, 1.5)),
     "C": dict(norm_init=("uniform", 0.5, 1.5), init_std=0.05),
+    "D": dict(norm_init=("uniform", 0.5, 1.5), init_std=0.05),
 }
-RAW = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEED = {"A": 0, "B": 1, "C": 2}
+RAW = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+SEED = {"A": 0, "B": 1, "C": 2, "D": 3}
 
 
 def tiny_config(name: str) -> LlamaConfig:
