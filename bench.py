@@ -134,6 +134,57 @@ def time_prefill(engine, cfg, dtype: str, repeats: int = 3) -> dict:
             "frac": round(flops / best / (PEAK_TFLOPS[dtype] * 1e12), 4)}
 
 
+LLAMA_1B = dict(
+    model_type="llama", num_hidden_layers=16, hidden_size=2048, num_attention_heads=32, num_key_value_heads=8,
+    head_dim=64, intermediate_size=8192, vocab_size=128256, rope_theta=500000.0, rms_norm_eps=1e-5,
+    tie_word_embeddings=True, max_position_embeddings=131072,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+
+
+def serve(a) -> int:
+    """Continuous batching of 128 requests on the Llama-3.2-1B shape: prompts of 64 to 2,048 tokens, 32 to 512
+    new tokens each (uniform, seeded), greedy, context 4,096.  Prints one JSON line of its own."""
+    import random
+    import torch
+    from infernum_amd import BatchConfig, CacheConfig, Engine, GenerateOptions, LlamaConfig, Runtime
+    cfg = LlamaConfig.from_dict(LLAMA_1B)
+    bc = BatchConfig(max_batch_size=a.serve_batch, max_prefill_tokens=a.serve_chunk, block_size=PAGE_SIZE,
+                     num_blocks=a.serve_blocks, max_tokens_per_step=a.serve_chunk + a.serve_batch)
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16",
+                                cache_config=CacheConfig(page_size=bc.block_size, num_pages=bc.num_blocks,
+                                                         num_state_slots=bc.max_batch_size),
+                                max_tokens_per_step=bc.max_tokens_per_step)
+    rt = Runtime(engine, None, bc, max_seq_len=CONTEXT_LEN)
+    rng = random.Random(0)
+    jobs = [([rng.randrange(cfg.vocab_size) for _ in range(rng.randint(64, 2048))], rng.randint(32, 512))
+            for _ in range(a.serve_requests)]
+    # a short warm-up so that kernels are loaded and the common decode shapes are recorded
+    rt.generate_batch([j[0][:64] for j in jobs[:4]], GenerateOptions(max_new_tokens=4))
+    sync()
+    t0 = time.perf_counter()
+    seqs = [rt.submit(p, GenerateOptions(max_new_tokens=n)) for p, n in jobs]
+    steps = set_back = 0
+    while not rt.scheduler.is_idle():
+        plan = rt.step()
+        steps += 1
+        set_back += len(plan.set_back)
+    sync()
+    dt = time.perf_counter() - t0
+    gen = sum(len(s.generated_ids) for s in seqs)
+    prompt = sum(len(j[0]) for j in jobs)
+    assert all(s.error is None and len(s.generated_ids) == n for s, (_, n) in zip(seqs, jobs))
+    print(json.dumps({"metric": "continuous batching, Llama-3.2-1B shape", "requests": len(jobs),
+                      "generated_tokens": gen, "prompt_tokens": prompt, "seconds": round(dt, 3),
+                      "generated_tok_per_s": round(gen / dt, 1), "all_tok_per_s": round((gen + prompt) / dt, 1),
+                      "steps": steps, "ms_per_step": round(dt / steps * 1e3, 3), "set_back": set_back,
+                      "graph_replays": engine.graph_replays, "max_batch": bc.max_batch_size,
+                      "chunk": bc.max_prefill_tokens, "num_blocks": bc.num_blocks, "dtype": "bf16",
+                      "data": "synthetic"}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,11 +196,19 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the prefill of 2,048 tokens, a few times (for profiles); prints its record alone")
+    ap.add_argument("--serve", action="store_true",
+                    help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
+    ap.add_argument("--serve-requests", type=int, default=128)
+    ap.add_argument("--serve-batch", type=int, default=64)
+    ap.add_argument("--serve-chunk", type=int, default=1024)
+    ap.add_argument("--serve-blocks", type=int, default=16384)
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
         return 2
 
+    if a.serve:
+        return serve(a)
     import torch
     from infernum_amd import CacheConfig, Engine, LlamaConfig
 

@@ -271,6 +271,12 @@ class CacheManager:
     def token_slots(self, group: int, req: Hashable, start: int, n: int) -> np.ndarray:
         """page * page_size + offset of positions start .. start+n-1 (pages must be reserved)."""
         g = self.groups[group]
+        if n == 1:                                   # a decoded token: no arrays needed
+            t = g.tables[req].pages
+            i = start // g.page_size
+            if i >= len(t) or t[i] < 0:
+                raise PageError(f"request {req!r} has no page for position {start}")
+            return np.asarray([t[i] * g.page_size + start % g.page_size], dtype=np.int32)
         pos = np.arange(start, start + n, dtype=np.int64)
         pages = np.asarray(g.tables[req].pages, dtype=np.int64)
         idx = pos // g.page_size

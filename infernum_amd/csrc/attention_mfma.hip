@@ -64,93 +64,114 @@ __device__ __forceinline__ void zero_row_operand(s16x4 (&reg)[NS]) {
   for (int s = 0; s < NS; ++s) reg[s] = (s16x4){0, 0, 0, 0};
 }
 
-__device__ __forceinline__ float bf16_round(float x) { return bf16_bits_to_float(float_to_bf16_bits(x)); }
-
-// One tile of 16 keys, t0 .. t0+15, for CT column tiles.
-//   pos[c], lo[c]: this lane's column (lane % 16) of tile c sees keys lo .. pos; pos < 0: no such column
-//   key_lo, key_hi: keys outside are not data of this request (wave-uniform)
-template <int CT>
-__device__ __forceinline__ void attn_tile(int t0, int key_lo, int key_hi, const int* __restrict__ bt, int ps,
-                                          int num_pages, int nkv, int g, const uint16_t* __restrict__ k_pages,
-                                          const uint16_t* __restrict__ v_pages, const s16x4 (&q)[CT][NS],
-                                          const int (&pos)[CT], const int (&lo)[CT], float scale_log2,
-                                          f32x4 (&o)[CT][NS], float (&m)[CT], float (&l)[CT], int lane) {
-  const int j = lane & 15, qd = lane >> 4;
-  // ---- S^T = K Q^T
-  const int key = t0 + j;
-  const int keyc = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
-  const int page = bt[keyc / ps];
-  const bool page_ok = (unsigned)page < (unsigned)num_pages;
-  const bool needed = key >= key_lo && key <= key_hi;
-  const uint16_t* krow = k_pages + (((size_t)(page_ok ? page : 0) * nkv + g) * ps + (keyc % ps)) * HD;
-  s16x4 kreg[NS];
-  load_row_operand(krow, qd, kreg);
-  const bool poison = __any(needed && !page_ok);
-  f32x4 s[CT];
-#pragma unroll
-  for (int c = 0; c < CT; ++c) {
-    s[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int st = 0; st < NS; ++st) s[c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[st], q[c][st], s[c], 0, 0, 0);
-  }
-  // ---- softmax statistics of each column; probabilities as the B operand of the next product
-  const int kg = t0 + 4 * qd;   // this lane holds the keys kg .. kg+3 of its column
-  s16x4 pb[CT];
-#pragma unroll
-  for (int c = 0; c < CT; ++c) {
-    float sv[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int kr = kg + r;
-      const bool ok = pos[c] >= 0 && kr <= pos[c] && kr >= lo[c];
-      sv[r] = ok ? s[c][r] * scale_log2 : -INFINITY;
-    }
-    float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, IA_WAVE));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE));
-    const float m_new = fmaxf(m[c], tmax);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    float p[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) p[r] = bf16_round(exp2f(sv[r] - m_safe));
-    const float corr = exp2f(m[c] - m_safe);
-    float psum = (p[0] + p[1]) + (p[2] + p[3]);
-    psum += __shfl_xor(psum, 16, IA_WAVE);
-    psum += __shfl_xor(psum, 32, IA_WAVE);
-    l[c] = l[c] * corr + psum;
-    if (poison) l[c] = __uint_as_float(0x7fc00000u);
-    m[c] = m_new;
-#pragma unroll
-    for (int n = 0; n < NS; ++n) o[c][n] *= corr;
-    pb[c] = as_s16x4((uint32_t)float_to_bf16_bits(p[0]) | ((uint32_t)float_to_bf16_bits(p[1]) << 16),
-                     (uint32_t)float_to_bf16_bits(p[2]) | ((uint32_t)float_to_bf16_bits(p[3]) << 16));
-  }
-  // ---- O^T += V^T P^T
-  const int kgc = kg < key_lo ? (key_lo & ~3) : (kg > key_hi ? (key_hi & ~3) : kg);
-  const int pagev = bt[kgc / ps];
-  const bool pagev_ok = (unsigned)pagev < (unsigned)num_pages;
-  const uint16_t* vbase = v_pages + ((size_t)(pagev_ok ? pagev : 0) * nkv + g) * HD * ps + (kgc % ps);
-  // keep the values of keys key_lo .. key_hi, zero the others (16 bits each)
-  uint32_t mlo = 0u, mhi = 0u;
-  if (kg == kgc) {
-    mlo = ((kg >= key_lo && kg <= key_hi) ? 0x0000ffffu : 0u) | ((kg + 1 >= key_lo && kg + 1 <= key_hi) ? 0xffff0000u : 0u);
-    mhi = ((kg + 2 >= key_lo && kg + 2 <= key_hi) ? 0x0000ffffu : 0u) | ((kg + 3 >= key_lo && kg + 3 <= key_hi) ? 0xffff0000u : 0u);
-  }
-#pragma unroll
-  for (int n = 0; n < NS; ++n) {
-    const uint2 v = *reinterpret_cast<const uint2*>(vbase + (size_t)(n * 16 + j) * ps);
-    const s16x4 vreg = as_s16x4(v.x & mlo, v.y & mhi);
-#pragma unroll
-    for (int c = 0; c < CT; ++c) o[c][n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg, pb[c], o[c][n], 0, 0, 0);
-  }
-}
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 // ------------------------------------------------------------------------ decode
 // grid (B, nkv * ceil(G/16), num_splits), 256 threads.  Token b is row b of q and out.  The four waves of a
 // workgroup take every fourth tile of 16 keys of the workgroup's part of the keys and join what they found
 // through LDS (in the order of the waves), so that few requests still put many waves to work without more
-// partial results in memory.
+// partial results in memory.  The workgroup's slice of the block table is brought into LDS once, so that the
+// loads of keys and values wait for no other global load, and a wave's next tile is in flight while it
+// works on this one.
 #define DEC_WAVES 4
+#define DEC_BT_LDS 4096          // block-table entries kept in LDS (a longer slice is read from global memory)
+
+struct DecTile {                 // 16 keys as they come from memory: operands of the two products
+  s16x4 k[NS];
+  uint2 v[NS];
+  bool bad;                      // a key that is needed has no page
+};
+
+struct DecGeom {                 // what does not change from tile to tile
+  const uint16_t* k_base;        // pages of this key/value head
+  const uint16_t* v_base;
+  const int* bt_global;
+  const int* bt_lds;
+  int bt_first, bt_count;        // the slice [bt_first, bt_first + bt_count) of the table lies in bt_lds
+  size_t page_elems;
+  int ps, ps_shift, num_pages, key_lo, key_hi;
+};
+
+__device__ __forceinline__ int dec_page(const DecGeom& G, int key) {
+  const int idx = G.ps_shift >= 0 ? key >> G.ps_shift : key / G.ps;
+  const int rel = idx - G.bt_first;
+  return (unsigned)rel < (unsigned)G.bt_count ? G.bt_lds[rel] : G.bt_global[idx];
+}
+__device__ __forceinline__ int dec_offset(const DecGeom& G, int key) {
+  return G.ps_shift >= 0 ? key & (G.ps - 1) : key % G.ps;
+}
+
+__device__ __forceinline__ void dec_load(const DecGeom& G, int t0, int j, int qd, DecTile& T) {
+  const int key = t0 + j;
+  const int keyc = key < G.key_lo ? G.key_lo : (key > G.key_hi ? G.key_hi : key);
+  const int page = dec_page(G, keyc);
+  const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
+  load_row_operand(G.k_base + (size_t)(page_ok ? page : 0) * G.page_elems + (size_t)dec_offset(G, keyc) * HD, qd, T.k);
+  const int kg = t0 + 4 * qd;    // this lane brings the values of the keys kg .. kg+3 (one quad, one page)
+  const int kgc = kg < G.key_lo ? (G.key_lo & ~3) : (kg > G.key_hi ? (G.key_hi & ~3) : kg);
+  const int pagev = dec_page(G, kgc);
+  const bool pagev_ok = (unsigned)pagev < (unsigned)G.num_pages;
+  const uint16_t* vq = G.v_base + (size_t)(pagev_ok ? pagev : 0) * G.page_elems + dec_offset(G, kgc);
+  // keep the values of keys key_lo .. key_hi, zero the others (16 bits each)
+  uint32_t mlo = 0u, mhi = 0u;
+  if (kg == kgc && pagev_ok) {
+    mlo = ((kg >= G.key_lo && kg <= G.key_hi) ? 0x0000ffffu : 0u) | ((kg + 1 >= G.key_lo && kg + 1 <= G.key_hi) ? 0xffff0000u : 0u);
+    mhi = ((kg + 2 >= G.key_lo && kg + 2 <= G.key_hi) ? 0x0000ffffu : 0u) | ((kg + 3 >= G.key_lo && kg + 3 <= G.key_hi) ? 0xffff0000u : 0u);
+  }
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const uint2 v = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
+    T.v[n] = make_uint2(v.x & mlo, v.y & mhi);
+  }
+  const bool k_needed = key == keyc, v_needed = kg + 3 >= G.key_lo && kg <= G.key_hi;
+  T.bad = (k_needed && !page_ok) || (v_needed && !pagev_ok);
+}
+
+// One tile of 16 keys, t0 .. t0+15, against the 16 columns (heads) of this wave.
+//   pos, lo: this lane's column sees keys lo .. pos; pos < 0: no such column
+__device__ __forceinline__ void dec_compute(int t0, const DecTile& T, const s16x4 (&q)[NS], int pos, int lo, int qd,
+                                            float scale_log2, f32x4 (&o)[NS], float& m, float& l) {
+  // ---- S^T = K Q^T
+  f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < NS; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(T.k[st], q[st], s, 0, 0, 0);
+  // ---- softmax statistics of the column; probabilities as the B operand of the next product
+  const int kg = t0 + 4 * qd;   // this lane holds the keys kg .. kg+3 of its column
+  float sv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int kr = kg + r;
+    const bool ok = pos >= 0 && kr <= pos && kr >= lo;
+    sv[r] = ok ? s[r] * scale_log2 : -INFINITY;
+  }
+  float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, IA_WAVE));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE));
+  const float m_new = fmaxf(m, tmax);
+  const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+  // probabilities rounded to bf16 (hardware conversion, nearest even); their sum is taken of the rounded values
+  const f32x2_t e0 = {__builtin_amdgcn_exp2f(sv[0] - m_safe), __builtin_amdgcn_exp2f(sv[1] - m_safe)};
+  const f32x2_t e1 = {__builtin_amdgcn_exp2f(sv[2] - m_safe), __builtin_amdgcn_exp2f(sv[3] - m_safe)};
+  const uint32_t p0 = __builtin_bit_cast(uint32_t, __builtin_convertvector(e0, bf16x2_t));
+  const uint32_t p1 = __builtin_bit_cast(uint32_t, __builtin_convertvector(e1, bf16x2_t));
+  float psum = (__uint_as_float(p0 << 16) + __uint_as_float(p0 & 0xffff0000u)) +
+               (__uint_as_float(p1 << 16) + __uint_as_float(p1 & 0xffff0000u));
+  psum += __shfl_xor(psum, 16, IA_WAVE);
+  psum += __shfl_xor(psum, 32, IA_WAVE);
+  const float corr = __builtin_amdgcn_exp2f(m - m_safe);
+  l = l * corr + psum;
+  if (__any(T.bad)) l = __uint_as_float(0x7fc00000u);
+  m = m_new;
+  const s16x4 pb = as_s16x4(p0, p1);
+  // ---- O^T = O^T corr + V^T P^T
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    o[n] *= corr;
+    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(as_s16x4(T.v[n].x, T.v[n].y), pb, o[n], 0, 0, 0);
+  }
+}
+
 extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o,
@@ -158,6 +179,7 @@ extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
     int bt_stride, int nh, int nkv, int ps, int num_pages, float scale_log2, int window, int num_splits) {
   __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
   __shared__ f32x4 s_o[DEC_WAVES][NS][64];
+  __shared__ int s_bt[DEC_BT_LDS];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, qd = lane >> 4;
   const int G = nh / nkv, HT = (G + 15) / 16;
   const int g = blockIdx.y / HT, ht = blockIdx.y - g * HT;
@@ -167,24 +189,61 @@ extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
   const int hj = ht * 16 + j;
   const bool col_ok = hj < G;
   const int h = g * G + hj;
-  s16x4 qreg[1][NS];
-  if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg[0]);
-  else zero_row_operand(qreg[0]);
-  const int pos[1] = {col_ok ? p : -1};
-  const int lo[1] = {lo0};
-  f32x4 o[1][NS];
-#pragma unroll
-  for (int n = 0; n < NS; ++n) o[0][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float m[1] = {-INFINITY}, l[1] = {0.f};
   const int t_first = lo0 / 16, t_last = p / 16;
   const int per = (t_last - t_first + 1 + num_splits - 1) / num_splits;
   const int ta = t_first + split * per;
   const int tb = (ta + per < t_last + 1) ? ta + per : t_last + 1;
   const int* bt = block_tables + (size_t)b * bt_stride;
-  for (int t = ta + wave; t < tb; t += DEC_WAVES)
-    attn_tile<1>(t * 16, lo0, p, bt, ps, num_pages, nkv, g, k_pages, v_pages, qreg, pos, lo, scale_log2, o, m, l, lane);
+
+  DecGeom geo;
+  geo.ps = ps;
+  geo.ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;
+  geo.num_pages = num_pages;
+  geo.key_lo = lo0;
+  geo.key_hi = p;
+  geo.page_elems = (size_t)nkv * ps * HD;
+  geo.k_base = k_pages + (size_t)g * ps * HD;
+  geo.v_base = v_pages + (size_t)g * HD * ps;
+  geo.bt_global = bt;
+  geo.bt_lds = s_bt;
+  // the slice of the block table that this workgroup's keys need
+  {
+    const int k_from = ta * 16 < lo0 ? lo0 : ta * 16, k_to = tb * 16 - 1 > p ? p : tb * 16 - 1;
+    const int first = geo.ps_shift >= 0 ? k_from >> geo.ps_shift : k_from / ps;
+    const int last = geo.ps_shift >= 0 ? k_to >> geo.ps_shift : k_to / ps;
+    int count = ta < tb ? last - first + 1 : 0;
+    if (count > DEC_BT_LDS) count = DEC_BT_LDS;
+    geo.bt_first = first;
+    geo.bt_count = count;
+    for (int i = threadIdx.x; i < count; i += DEC_WAVES * 64) s_bt[i] = bt[first + i];
+  }
+  s16x4 qreg[NS];
+  if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg);
+  else zero_row_operand(qreg);
+  const int pos = col_ok ? p : -1;
+  f32x4 o[NS];
+#pragma unroll
+  for (int n = 0; n < NS; ++n) o[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  __syncthreads();
+  // two tiles in flight: the loads of the next tile of this wave are issued before this one is worked on
+  DecTile A, B;
+  int t = ta + wave;
+  if (t < tb) dec_load(geo, t * 16, j, qd, A);
+  while (t < tb) {
+    const bool more1 = t + DEC_WAVES < tb;
+    if (more1) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, B);
+    dec_compute(t * 16, A, qreg, pos, lo0, qd, scale_log2, o, m, l);
+    t += DEC_WAVES;
+    if (!more1) break;
+    const bool more2 = t + DEC_WAVES < tb;
+    if (more2) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, A);
+    dec_compute(t * 16, B, qreg, pos, lo0, qd, scale_log2, o, m, l);
+    t += DEC_WAVES;
+    if (!more2) break;
+  }
   // ---- join the waves: common maximum, rescale, add in the order of the waves
-  if (qd == 0) { s_m[wave][j] = m[0]; s_l[wave][j] = l[0]; }
+  if (qd == 0) { s_m[wave][j] = m; s_l[wave][j] = l; }
   __syncthreads();
   float M = s_m[0][j];
 #pragma unroll
@@ -195,9 +254,9 @@ extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
     const float mw = s_m[w][j];
     L += (mw == -INFINITY ? 0.f : exp2f(mw - M)) * s_l[w][j];
   }
-  const float f = (m[0] == -INFINITY) ? 0.f : exp2f(m[0] - M);
+  const float f = (m == -INFINITY) ? 0.f : exp2f(m - M);
 #pragma unroll
-  for (int n = 0; n < NS; ++n) s_o[wave][n][lane] = o[0][n] * f;
+  for (int n = 0; n < NS; ++n) s_o[wave][n][lane] = o[n] * f;
   __syncthreads();
   if (!col_ok) return;
   // wave w finishes the slices n = w, w + 4, ... of the head
@@ -279,8 +338,6 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 // 16 + 4 qd .. 16 + 4 qd + 3; the values are laid into LDS in that order of keys, so the probabilities go
 // from registers to registers.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
 #define PF_KT (HD <= 128 ? 64 : 32)   // keys per round of the main loop (one barrier), in parts of 32
 #define PF_SUBS (PF_KT / 32)
 #define PF_QPT (PF_KT / 4)             // quads of 4 keys per round

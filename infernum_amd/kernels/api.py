@@ -48,8 +48,30 @@ def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_fixed_stream: Optional[ctypes.c_void_p] = None
+
+
 def _stream() -> ctypes.c_void_p:
+    if _fixed_stream is not None:
+        return _fixed_stream
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class on_current_stream:
+    """Within this block every kernel call launches on the stream that is current at its entry, looked up
+    once (the lookup costs as much as several launches).  Enter it anew inside a graph capture: the capture
+    has a stream of its own."""
+
+    def __enter__(self):
+        global _fixed_stream
+        self._before = _fixed_stream
+        _fixed_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        global _fixed_stream
+        _fixed_stream = self._before
+        return False
 
 
 def _ok(code: int, what: str) -> None:

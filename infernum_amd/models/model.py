@@ -95,6 +95,11 @@ class DecoderModel:
     # ---- one step --------------------------------------------------------------
     def forward(self, ctx: StepContext, views: List[CacheView]) -> torch.Tensor:
         """Runs the tokens of ``ctx`` and returns fp32 logits [R, V] at ctx.logit_rows."""
+        from ..kernels.api import on_current_stream
+        with on_current_stream():
+            return self._forward(ctx, views)
+
+    def _forward(self, ctx: StepContext, views: List[CacheView]) -> torch.Tensor:
         h = self.embedding.forward(ctx)
         pending: Optional[torch.Tensor] = None
         for e, view in zip(self.spec.schedule, views):
