@@ -127,3 +127,12 @@ def test_command_line(folders):
     assert "Decoding: greedy (argmax)" in proc.stdout and "KV cache: enabled" in proc.stdout
     assert " ".join(map(str, want)) in proc.stdout
     assert "Generated 6 tokens in" in proc.stdout
+
+
+def test_bench_command_line(folders):
+    d, cfg, w = folders["B"]
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "bench"), d, "12", "--dtype", "f32",
+                           "--prefill", "40"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert "12 tokens in" in proc.stdout and "tok/s" in proc.stdout and "prefill 40 tokens" in proc.stdout
+    assert "Model loaded: 3 layers, 128 hidden, dtype=f32" in proc.stderr
