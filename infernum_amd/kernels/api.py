@@ -419,21 +419,7 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
     return out
 
 
-# ------------------------------------------------------- which fast kernels are built
-_has: Dict[str, bool] = {}
-
-
-def gemm_skinny_available() -> bool:
-    if "skinny" not in _has:
-        _has["skinny"] = hasattr(_core(), "ia_gemm_skinny")
-    return _has["skinny"]
-
-
+# ---------------------------------------------------- which head sizes the MFMA kernels take
 def attention_mfma_available(d: int) -> bool:
-    """Whether the MFMA attention kernels exist for head size d (built on first use)."""
-    import os
-    key = f"attn{d}"
-    if key not in _has:
-        _has[key] = (d in _build.SUPPORTED_HEAD_DIMS
-                     and os.path.isfile(os.path.join(_build.CSRC_DIR, "attention_mfma.hip")))
-    return _has[key]
+    """Whether the MFMA attention kernels take head size d (their library is built at its first use)."""
+    return d in _build.SUPPORTED_HEAD_DIMS

@@ -183,8 +183,6 @@ def test_gemm_generic(M, N, K_):
 @pytest.mark.parametrize("N,K_", [(250, 96), (384, 176), (4096, 4096), (1000, 14336), (16, 8), (129, 1000)])
 def test_gemm_skinny(M, N, K_):
     api = K()
-    if not api.gemm_skinny_available():
-        pytest.skip("skinny kernel not built")
     a, w = _rand(M, K_, dtype=torch.bfloat16, seed=6), _rand(N, K_, dtype=torch.bfloat16, seed=7)
     want = a.double() @ w.double().t()
     outf = torch.full((M, N), float("nan"), device=DEV)
