@@ -187,3 +187,147 @@ def test_state_slot_is_zeroed_when_taken_again(toy):
     eng.end("b")
     again = eng.step([StepEntry("c", [1, 2, 3, 4, 5], [4])]).cpu()
     assert torch.equal(a, again)
+
+
+# ------------------------------------------------------------------------------------------------
+# A feed-forward with routing and another position encoding, again defined here and not in the framework.
+from infernum_amd.parts import FeedForward, PositionEncoding        # noqa: E402
+
+
+class RoutedFeedForward(FeedForward):
+    """Two experts, the one with the larger router logit (fp32) serves the token:
+    y = swiglu_e(x), e = argmax(x W_r^T).  Written with torch operations: it is a toy."""
+
+    def __init__(self, rt, hidden_size, intermediate_size, num_experts=2):
+        super().__init__(rt)
+        self.H, self.I, self.E = hidden_size, intermediate_size, num_experts
+
+    def weights(self):
+        w = {"router.weight": WeightSpec((self.E, self.H), ("normal", 0.5), follows_compute_dtype=False)}
+        for e in range(self.E):
+            w[f"experts.{e}.gate_up.weight"] = WeightSpec((2 * self.I, self.H), ("normal", 0.1))
+            w[f"experts.{e}.down.weight"] = WeightSpec((self.H, self.I), ("normal", 0.1))
+        return w
+
+    def load(self, tensors):
+        self.t = tensors
+
+    def forward(self, x, ctx):
+        logits = x.float() @ self.t["router.weight"].float().t()
+        choice = logits.argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for e in range(self.E):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                gu = x[rows].float() @ self.t[f"experts.{e}.gate_up.weight"].float().t()
+                g, u = gu[:, :self.I], gu[:, self.I:]
+                act = (g / (1 + torch.exp(-g)) * u).to(x.dtype)
+                out[rows] = (act.float() @ self.t[f"experts.{e}.down.weight"].float().t()).to(x.dtype)
+        return out
+
+
+class SlowedPartialRotary(PositionEncoding):
+    """Rotates the first half of each head only, with every frequency divided by ``slow``: what the attention
+    kernels need of a position encoding is its table of frequencies and how many values it rotates."""
+    graph_safe = True
+
+    def __init__(self, rt, head_dim, theta, slow):
+        super().__init__(rt)
+        self.rotary_dim = head_dim // 2
+        i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        self.inv_freq = (theta ** (-2.0 * i / self.rotary_dim) / slow).to(torch.float32).to(rt.device)
+
+
+@dataclass(frozen=True)
+class Toy2Config:
+    vocab_size: int = 77
+    hidden_size: int = 64
+    num_heads: int = 2
+    intermediate_size: int = 40
+    slow: float = 4.0
+    model_type: str = "toy-routed"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return Toy2Config(**{k: v for k, v in raw.items() if k in Toy2Config.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy2_spec(cfg: Toy2Config) -> ModelSpec:
+    H, d = cfg.hidden_size, cfg.hidden_size // cfg.num_heads
+    norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "init": ("uniform", 0.5, 1.5)}, prefix)
+    layers = []
+    for i in range(2):
+        layers.append(LayerSpec(
+            "prenorm",
+            PartSpec("attention", {"hidden_size": H, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_heads,
+                                   "head_dim": d, "init_std": 0.1,
+                                   "position": {"kind": "slowed_partial_rope",
+                                                "params": {"head_dim": d, "theta": 100.0, "slow": cfg.slow}}},
+                     f"l.{i}.attn."),
+            PartSpec("routed", {"hidden_size": H, "intermediate_size": cfg.intermediate_size}, f"l.{i}.moe.")
+            if i == 1 else PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size,
+                                               "init_std": 0.1}, f"l.{i}.ff."),
+            norm(f"l.{i}.n1."), norm(f"l.{i}.n2.")))
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.5}, "emb."),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn."),
+                     head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.1}, "head."))
+
+
+def plain_forward2(cfg: Toy2Config, w, ids):
+    W = {k: v.double() for k, v in w.items()}
+    H, nh = cfg.hidden_size, cfg.num_heads
+    d = H // nh
+    rot = d // 2
+    T = len(ids)
+    i = torch.arange(rot // 2, dtype=torch.float64)
+    freqs = (100.0 ** (-2.0 * i / rot) / cfg.slow).to(torch.float32).double()
+    pos = torch.arange(T)
+    h = P.embedding(W["emb.weight"], ids)
+    for l in range(2):
+        n = P.rms_norm(h, W[f"l.{l}.n1.weight"], 1e-5)
+        p = f"l.{l}.attn."
+        q = P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d)
+        k = P.linear(n, W[p + "k_proj.weight"]).reshape(T, nh, d)
+        v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, nh, d)
+        q = torch.cat([P.rope(q[..., :rot], pos, freqs), q[..., rot:]], -1)
+        k = torch.cat([P.rope(k[..., :rot], pos, freqs), k[..., rot:]], -1)
+        a = P.causal_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, H)
+        h = h + P.linear(a, W[p + "o_proj.weight"])
+        m = P.rms_norm(h, W[f"l.{l}.n2.weight"], 1e-5)
+        if l == 0:
+            h = h + P.linear(P.swiglu(P.linear(m, W["l.0.ff.gate_proj.weight"]), P.linear(m, W["l.0.ff.up_proj.weight"])),
+                             W["l.0.ff.down_proj.weight"])
+        else:
+            choice = P.linear(m, W["l.1.moe.router.weight"]).argmax(-1)
+            out = torch.zeros_like(m)
+            for t in range(T):
+                e = int(choice[t])
+                gu = P.linear(m[t:t + 1], W[f"l.1.moe.experts.{e}.gate_up.weight"])
+                I = cfg.intermediate_size
+                out[t] = P.linear(P.swiglu(gu[:, :I], gu[:, I:]), W[f"l.1.moe.experts.{e}.down.weight"])[0]
+            h = h + out
+    return P.linear(P.rms_norm(h, W["fn.weight"], 1e-5), W["head.weight"])
+
+
+def test_routed_feed_forward_and_another_position_encoding(tmp_path):
+    register_part("feed_forward", "routed", RoutedFeedForward, replace=True)
+    register_part("position", "slowed_partial_rope", SlowedPartialRotary, replace=True)
+    register_architecture("toy-routed", Toy2Config, toy2_spec, replace=True)
+    cfg = Toy2Config()
+    d = write_random_model(cfg, str(tmp_path / "toy2"), seed=9, dtype=torch.float32)
+    _, w = P.read_model(d)
+    eng = Engine.from_pretrained(d, dtype="float32", cache_config=CacheConfig(page_size=4, num_pages=64,
+                                                                              num_state_slots=4))
+    assert not eng.use_graphs                 # the routed feed-forward is not marked as safe to record
+    reqs = TT.make_requests(cfg.vocab_size, (41, 9, 30), seed=6)
+    ref = {r: plain_forward2(cfg, w, t) for r, t in reqs.items()}
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("portions", TT.trace_portions(reqs)),
+                        ("tail", TT.trace_tail_one_by_one(reqs, 10))):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy2 {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= 3e-5 * rms, (name, worst / rms, where)
