@@ -398,6 +398,21 @@ def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
     assert err <= 2e-2, err
 
 
+@pytest.mark.parametrize("splits", [1, 3])
+def test_attention_mfma_decode_block_table_longer_than_its_lds_slice(splits):
+    """18,000 keys in pages of 4: 4,500 block-table entries, more than the 4,096 the decode kernel keeps in LDS;
+    the rest is read from global memory.  One far key is loud, so a wrong page shows."""
+    nh, nkv, d, ps = 4, 2, 32, 4
+    lens = [18000, 5]
+    case = _paged_case(nh, nkv, d, ps, lens, [1, 1], torch.bfloat16, seed=3, scale_one=(0, 17001, 6.0))
+    out = torch.full((2, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    K().attention_decode(case["q"], case["kp"], case["vp"], out, case["positions"], case["bt"], nh, nkv, d, scale,
+                         0, max(lens), num_splits=splits)
+    want = _ref_attention(case, nh, nkv, d, scale, 0)
+    assert (out.double().cpu() - want).abs().max().item() <= 2e-2
+
+
 def test_attention_mfma_far_key_stale_pages_and_missing_page():
     """A far key carries the softmax; pages hold NaN wherever this request has no data;
     a needed key without a page gives NaN instead of a fault."""
