@@ -32,6 +32,11 @@ LLAMA_8B = dict(
     rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
                       original_max_position_embeddings=8192),
 )
+LLAMA_13B = dict(
+    model_type="llama", num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=40,
+    intermediate_size=13824, vocab_size=32000, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+    max_position_embeddings=4096,
+)
 CONTEXT_LEN = 4096
 PROMPT_LEN = 512
 PREFILL_TOKENS = 2048
@@ -196,6 +201,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the prefill of 2,048 tokens, a few times (for profiles); prints its record alone")
+    ap.add_argument("--shape", default="8b", choices=["8b", "13b"],
+                    help="8b: Llama-3.1-8B (the default, the headline); 13b: Llama-2-13B (40 key/value heads)")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every request's prompt")
     ap.add_argument("--serve", action="store_true",
                     help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
     ap.add_argument("--serve-requests", type=int, default=128)
@@ -212,7 +220,7 @@ def main() -> int:
     import torch
     from infernum_amd import CacheConfig, Engine, LlamaConfig
 
-    raw = dict(LLAMA_8B)
+    raw = dict(LLAMA_8B if a.shape == "8b" else LLAMA_13B)
     full_layers = raw["num_hidden_layers"]
     if a.layers:
         raw["num_hidden_layers"] = a.layers
@@ -220,7 +228,7 @@ def main() -> int:
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
     max_batch = 1 if a.prefill_only else max(a.batch, 1 if a.no_points else 64)
-    tokens_needed = max(max_batch * (PROMPT_LEN + a.steps + a.warmup + PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
+    tokens_needed = max(max_batch * (a.prompt_len + a.steps + a.warmup + PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
     t_load = time.perf_counter()
     engine = Engine.from_config(cfg, seed=0, dtype=dtype,
                                 cache_config=CacheConfig(page_size=PAGE_SIZE,
@@ -235,20 +243,21 @@ def main() -> int:
         return 0
 
     # ---- the timed K steps at the headline batch ---------------------------------
-    dt, ctx_mid = time_decode(engine, a.batch, a.steps, a.warmup)
+    dt, ctx_mid = time_decode(engine, a.batch, a.steps, a.warmup, a.prompt_len)
     ms_per_step = dt / a.steps * 1e3
     value = a.batch * a.steps / dt
     achieved = decode_bytes(cfg, ctx_mid, elem) / (dt / a.steps) / 1e9
     out = {
-        "metric": "decode tok/s @ batch 8, Llama-3-8B shape", "value": round(value, 2), "unit": "tokens/s",
+        "metric": f"decode tok/s @ batch {a.batch}, {'Llama-3-8B' if a.shape == '8b' else 'Llama-2-13B'} shape", "value": round(value, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
         "config": {
-            "model": "llama-3.1-8b-shape-random", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
+            "model": "llama-3.1-8b-shape-random" if a.shape == "8b" else "llama-2-13b-shape-random", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
             "hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads, "num_kv_heads": cfg.num_kv_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
-            "global_batch": a.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "page_size": PAGE_SIZE,
-            "parallelism": "none", "sampling": "greedy", "rope": "llama3(8,1,4,8192) theta 5e5",
+            "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LEN, "page_size": PAGE_SIZE,
+            "parallelism": "none", "sampling": "greedy",
+            "rope": "llama3(8,1,4,8192) theta 5e5" if a.shape == "8b" else "theta 1e4",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -258,7 +267,7 @@ def main() -> int:
         points = {}
         for b in (1, 64):
             steps = max(16, min(a.steps, 64))
-            d, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)))
+            d, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)), a.prompt_len)
             points[f"decode_b{b}"] = round(b * steps / d, 2)
         out["points"] = points
         out["prefill"] = time_prefill(engine, cfg, a.dtype)
