@@ -15,14 +15,13 @@ from __future__ import annotations
 
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
-import numpy as np
 import torch
 
 from ..cache import CacheConfig, CacheManager
 from ..models.model import DecoderModel
-from ..parts.base import Runtime, StepContext
+from ..parts.base import Runtime
 
-from .batch import PackedStep, StepEntry, StepError, check_entries, pack_step
+from .batch import StepEntry, StepError, check_entries, pack_step  # noqa: F401  (StepError is part of this module's face)
 
 
 class OutOfPages(RuntimeError):

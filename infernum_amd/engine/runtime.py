@@ -19,11 +19,10 @@ import os
 from typing import Any, Callable, Iterator, List, Optional, Sequence, Union
 
 from ..cache import CacheConfig
-from ..sampling.params import GenerateOptions, SamplingParams
+from ..sampling.params import GenerateOptions
 from ..sampling.sampler import RowRequest
 from .engine import Engine, StepEntry
-from .scheduler import (BatchConfig, FinishReason, GenerationEvent, Scheduler, SchedulerOutput, SequencePhase,
-                        SequenceState, TokenSender)
+from .scheduler import BatchConfig, Scheduler, SchedulerOutput, SequencePhase, SequenceState, TokenSender
 
 Prompt = Union[str, Sequence[int]]
 

@@ -24,7 +24,6 @@ MAX_LIVE_REQUESTS = 4
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, stream: IO[str], done: IO[str],
            page_size: int = PAGE_SIZE, poison: bool = False) -> int:
-    import numpy as np
     from ..cache import CacheConfig
     from .engine import Engine, StepEntry
 

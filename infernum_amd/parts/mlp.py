@@ -9,7 +9,6 @@ from typing import Dict, Optional
 
 import torch
 
-from ..kernels import api as K
 from .base import FeedForward, Runtime, StepContext, WeightSpec, register_part
 from .linear import linear
 

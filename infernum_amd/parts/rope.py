@@ -19,7 +19,7 @@ fp32 product of the fp32 position and the fp32 frequency.
 from __future__ import annotations
 
 import math
-from typing import Any, Dict, Mapping, Optional
+from typing import Any, Mapping, Optional
 
 import torch
 

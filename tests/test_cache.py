@@ -4,7 +4,7 @@ import random
 
 import pytest
 
-from infernum_amd.cache import (NO_PAGE, BlockTable, CacheConfig, CacheManager, PageAllocator, PageError,
+from infernum_amd.cache import (NO_PAGE, CacheConfig, CacheManager, PageAllocator, PageError,
                                 StateSlotPool, pages_for)
 from infernum_amd.parts import CacheSpec, StateSpec
 

@@ -7,7 +7,7 @@ import torch
 
 import plain_llama as P
 import tiny_models as TM
-from part_harness import DEV, DTYPES, TOL, Steps, build, dense, rel_err, runtime
+from part_harness import DEV, TOL, Steps, build, dense, rel_err, runtime
 
 pytestmark = pytest.mark.gpu
 BOTH = pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

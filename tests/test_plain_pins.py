@@ -2,8 +2,6 @@
 reference's text.  Each test is chosen so that a plausible mistake fails it."""
 import math
 
-import numpy as np
-import pytest
 import torch
 
 import plain_llama as P

@@ -4,7 +4,7 @@ import random
 import pytest
 
 from fake_engine import CpuSampler, FakeEngine, reference_generation
-from infernum_amd.engine import (BatchConfig, FinishReason, GenerationError, Runtime, Scheduler, SequencePhase)
+from infernum_amd.engine import BatchConfig, FinishReason, GenerationError, Runtime, SequencePhase
 from infernum_amd.sampling import GenerateOptions, SamplingParams
 
 

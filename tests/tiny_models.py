@@ -5,9 +5,6 @@ size, feed-forward width (no power of two), vocabulary, eps, theta, rope scaling
 tied or separate head, norm weights.  C adds a sliding window on some layers, a
 head size that is no power of two and an explicit head_dim.
 """
-import os
-import tempfile
-
 import torch
 
 from infernum_amd.config import LlamaConfig
