@@ -39,6 +39,7 @@ CORE_SOURCES = [
     "elementwise.hip",
     "gemm_generic.hip",
     "gemm_skinny.hip",
+    "gemm_mfma.hip",
     "attention_generic.hip",
     "sampling.hip",
 ]

@@ -1,0 +1,224 @@
+// C[M, N] = X[M, K] * W[N, K]^T in bf16 with fp32 accumulation for many rows (prefill), on
+// v_mfma_f32_32x32x16_bf16 with both operands tiled through LDS.
+//
+// A workgroup of WAVES_M x WAVES_N waves owns a BM x BN tile of C; a wave owns (BM / WAVES_M) x
+// (BN / WAVES_N) of it as 32 x 32 accumulator tiles.  K is walked in steps of 64.  The BM x 64 tile of X and
+// the BN x 64 tile of W of a later step go from global memory straight into a free stage of a ring of LDS
+// buffers (global_load_lds_dwordx4: no registers and no LDS store instructions on the way) while the matrix
+// cores work on this step; one barrier a step.
+//
+// Both matrices have K contiguous, which is what the operands want: lane (i, h) = (lane % 32, lane / 32) of
+// an operand holds the 8 values k = 16 s + 8 h .. + 7 of row i, one 16-byte LDS read.  A load instruction
+// of a wave fills 1,024 consecutive bytes of LDS, lane by lane, which is 8 rows of 128 bytes without
+// padding; so that the reads of rows i, i + 1, .. do not all fall on the same banks, the 16-byte piece c of
+// row r lies at position c ^ (r % 8) of its row: the lane that fills position p of row r fetches piece
+// p ^ (r % 8) from global memory.
+//
+// Workgroups are numbered so that the ones running together share rows of W and X in L2.
+//
+// K must be a multiple of 64; M and N are arbitrary (rows beyond them are read from the last valid row and
+// not stored).  A result row depends on its own row of X only; how rows are grouped into tiles does not
+// change it.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define GM_BK 64
+#define GM_ROW_BYTES (GM_BK * 2)
+
+typedef const __attribute__((address_space(1))) void* gm_global_ptr;
+typedef __attribute__((address_space(3))) void* gm_lds_ptr;
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X,
+                                                                           const uint16_t* __restrict__ W,
+                                                                           uint16_t* __restrict__ C, int M, int N,
+                                                                           int K, int tiles_m, int tiles_n) {
+  constexpr int WAVES = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // tile of a wave
+  constexpr int TM = WM / 32, TN = WN / 32;             // in accumulator tiles of 32 x 32
+  constexpr int ROWS = BM + BN;                         // rows staged per step (X rows, then W rows)
+  constexpr int STAGE_BYTES = ROWS * GM_ROW_BYTES;
+  constexpr int FILLS = ROWS / 8;                       // load instructions per step, 8 rows each
+  constexpr int FPW = FILLS / WAVES;                    // per wave
+  constexpr int KS = GM_BK / 16;                        // matrix-core steps per staged step
+  static_assert(FILLS % WAVES == 0, "loads must divide over the waves");
+  static_assert(BM % (8 * WAVES) == 0, "a load index must be all X or all W");
+  extern __shared__ __attribute__((aligned(1024))) char lds[];   // [STAGES][ROWS][128 bytes]
+
+  // workgroups go to the 8 dies in turn (workgroup i to die i % 8), and each die has an L2 of its own:
+  // give every die one contiguous run of tiles, so that W is read from memory once and not once per die
+  const int total = tiles_m * tiles_n;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int bid = xcd * (total >> 3) + min(xcd, total & 7) + idx;
+  // 8 tiles of M under one tile of N at a time
+  const int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int group = bid / per_group, in_group = bid - group * per_group;
+  const int group_rows = min(GROUP, tiles_m - group * GROUP);
+  const int tm = group * GROUP + in_group % group_rows;
+  const int tn = in_group / group_rows;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int li = lane & 31, lh = lane >> 5;
+
+  // ---- staging: load f of this wave fills rows 8 (f WAVES + wave) .. + 7; this lane fills position
+  // lane % 8 of row lane / 8 of them.  Byte offsets from X or W.
+  uint32_t src[FPW];
+#pragma unroll
+  for (int f = 0; f < FPW; ++f) {
+    const int row = 8 * (f * WAVES + wave) + (lane >> 3);
+    const int piece = (lane & 7) ^ (row & 7);
+    const int r = (8 * f * WAVES < BM) ? min(m0 + row, M - 1) : min(n0 + row - BM, N - 1);
+    src[f] = ((uint32_t)r * (uint32_t)K + (uint32_t)piece * 8u) * 2u;
+  }
+#define GM_FILL(f, kt, buf)                                                                                  \
+  __builtin_amdgcn_global_load_lds(                                                                         \
+      (gm_global_ptr)(reinterpret_cast<const char*>((8 * (f) * WAVES < BM) ? X : W) + (size_t)(kt) * GM_ROW_BYTES + \
+                      src[f]),                                                                              \
+      (gm_lds_ptr)(lds + (buf) * STAGE_BYTES + 1024 * ((f) * WAVES + wave)), 16, 0, 0)
+
+  // W is the first operand: accumulator register r of lane (j, h) = (lane % 32, lane / 32) of tile [a][b] is
+  // the product for n = 32 a + 8 (r / 4) + 4 h + r % 4 and m = 32 b + j, four neighbours in a row of C at a time
+  f32x16 acc[TN][TM];
+#pragma unroll
+  for (int a = 0; a < TN; ++a)
+#pragma unroll
+    for (int b = 0; b < TM; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+  // stage j of LDS holds steps j, j + STAGES, ..: while step kt is worked on, step kt + STAGES - 1 is
+  // fetched into the stage that step kt - 1 has left
+  const int ksteps = K / GM_BK;
+#pragma unroll
+  for (int j = 0; j < STAGES - 1; ++j)
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) GM_FILL(f, min(j, ksteps - 1), j);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * FPW) : "memory");
+  __syncthreads();
+
+  // piece 2 s + h of row i lies at position (2 s + h) ^ (i % 8); tiles start at multiples of 32 rows
+  const int xrow = (wm * WM + li) * GM_ROW_BYTES;
+  const int wrow = (BM + wn * WN + li) * GM_ROW_BYTES;
+  int swz[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) swz[s] = ((2 * s + lh) ^ (li & 7)) * 16;
+
+  int buf = 0, fill_buf = STAGES - 1;
+  for (int kt = 0; kt < ksteps; ++kt) {
+    const char* xa = lds + buf * STAGE_BYTES + xrow;
+    const char* wb = lds + buf * STAGE_BYTES + wrow;
+    // past the end the last step is fetched again, into a stage that is not read any more
+    const int kt_fill = min(kt + STAGES - 1, ksteps - 1);
+    bf16x8 wf[2][TN], xf[2][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a) wf[0][a] = *reinterpret_cast<const bf16x8*>(wb + a * 32 * GM_ROW_BYTES + swz[0]);
+#pragma unroll
+    for (int b = 0; b < TM; ++b) xf[0][b] = *reinterpret_cast<const bf16x8*>(xa + b * 32 * GM_ROW_BYTES + swz[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    // The order below is kept as written (nothing moves across a sched_barrier): the reads of the next
+    // operands and the loads of the next step go between the matrix instructions of this one, so that
+    // none of them is waited for with the matrix cores idle.
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      constexpr int MF = TN * TM, RD = TN + TM;
+#pragma unroll
+      for (int g = 0; g < MF; ++g) {
+        if (s + 1 < KS) {
+#pragma unroll
+          for (int r = (g * RD) / MF; r < ((g + 1) * RD) / MF; ++r) {
+            if (r < TN)
+              wf[(s + 1) & 1][r] = *reinterpret_cast<const bf16x8*>(wb + r * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
+            else
+              xf[(s + 1) & 1][r - TN] =
+                  *reinterpret_cast<const bf16x8*>(xa + (r - TN) * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
+          }
+        }
+#pragma unroll
+        for (int f = (g * FPW) / MF; f < ((g + 1) * FPW) / MF; ++f)
+          if (s == 0) GM_FILL(f, kt_fill, fill_buf);   // all of them early
+        acc[g / TM][g % TM] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][g / TM], xf[s & 1][g % TM], acc[g / TM][g % TM], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // the next step's loads must have landed; the ones issued since may still be on their way
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * FPW) : "memory");
+    __syncthreads();
+    buf = (buf + 1 == STAGES) ? 0 : buf + 1;
+    fill_buf = (fill_buf + 1 == STAGES) ? 0 : fill_buf + 1;
+  }
+
+  // ---- C
+  const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+  for (int a = 0; a < TN; ++a)
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+      const int m = m0 + wm * WM + b * 32 + li;
+      if (m >= M) continue;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * WN + a * 32 + 8 * g + 4 * lh;
+        uint16_t* dstp = C + (size_t)m * N + n;
+        if (vec_ok && n + 3 < N) {
+          uint2 v;
+          v.x = (uint32_t)float_to_bf16_bits(acc[a][b][4 * g]) | ((uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 1]) << 16);
+          v.y = (uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 2]) | ((uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 3]) << 16);
+          *reinterpret_cast<uint2*>(dstp) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) dstp[e] = float_to_bf16_bits(acc[a][b][4 * g + e]);
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES>
+static int launch_gemm_mfma(const uint16_t* x, const uint16_t* w, uint16_t* c, int M, int N, int K,
+                            hipStream_t stream) {
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const size_t lds_bytes = (size_t)STAGES * (BM + BN) * GM_ROW_BYTES;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  if ((long long)tiles_m * tiles_n > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
+  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES><<<tiles_m * tiles_n, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
+      x, w, c, M, N, K, tiles_m, tiles_n);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// X [M, K], W [N, K], C [M, N]: bf16, contiguous.  tile: 0 = chosen here, 1 = 256 x 256 (two stages),
+// 2 = 128 x 256 (three stages), 3 = 128 x 128 (four stages).
+extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int tile,
+                            hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || (K % GM_BK) != 0) return IA_ERR_UNSUPPORTED;
+  // rows are addressed with 32-bit byte offsets
+  if ((unsigned long long)M * K * 2 > 0xffffffffULL || (unsigned long long)N * K * 2 > 0xffffffffULL)
+    return IA_ERR_UNSUPPORTED;
+  const uint16_t* x = (const uint16_t*)X;
+  const uint16_t* w = (const uint16_t*)W;
+  uint16_t* c = (uint16_t*)C;
+  if (tile == 0) {
+    // the largest tile that still gives every compute unit about two workgroups
+    const long long t256 = (long long)((M + 255) / 256) * ((N + 255) / 256);
+    const long long t128 = (long long)((M + 127) / 128) * ((N + 255) / 256);
+    tile = t256 >= 512 ? 1 : (t128 >= 128 ? 2 : 3);
+  }
+  if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2>(x, w, c, M, N, K, stream);
+  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3>(x, w, c, M, N, K, stream);
+  if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4>(x, w, c, M, N, K, stream);
+  return IA_ERR_BAD_ARG;
+}

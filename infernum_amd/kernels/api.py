@@ -239,6 +239,33 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.T
     return out
 
 
+MFMA_GEMM_TILES = {"auto": 0, "256x256": 1, "128x256": 2, "128x128": 3}
+
+
+def gemm_mfma_supported(M: int, N: int, K: int) -> bool:
+    """Sizes the LDS-tiled MFMA product takes: K in steps of 64, rows addressed with 32-bit byte offsets."""
+    return M >= 1 and N >= 1 and K >= 64 and K % 64 == 0 and M * K * 2 < 2 ** 32 and N * K * 2 < 2 ** 32
+
+
+def gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, tile: str = "auto") -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T, bf16 with fp32 accumulation, for many rows (prefill): both operands
+    tiled through LDS, ``v_mfma_f32_32x32x16_bf16``.  A row of the result depends on its own row of ``a`` only."""
+    _dev(a, w, out)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_mfma: shapes")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_mfma: bf16 operands")
+    _need(a.is_contiguous() and w.is_contiguous(), "gemm_mfma: contiguous operands")
+    _need(gemm_mfma_supported(M, N, K), f"gemm_mfma: M={M} N={N} K={K} not supported (K % 64 == 0, below 4 GiB)")
+    _need(tile in MFMA_GEMM_TILES, f"gemm_mfma: unknown tile {tile!r}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N),
+          f"gemm_mfma: out must be contiguous bf16 [{M}, {N}]")
+    _ok(_core().ia_gemm_mfma(_p(a), _p(w), _p(out), M, N, K, MFMA_GEMM_TILES[tile], _stream()), "gemm_mfma")
+    return out
+
+
 SKINNY_MAX_M = 64
 EPILOGUE = {None: 0, "swiglu": 1}
 

@@ -9,7 +9,10 @@ fp32: the hand-written fp32 kernel, always (no reduced-precision matrix mode).
 bf16: up to 64 rows the hand-written MFMA kernel that streams the weight once;
 above that the library product (hipBLASLt through torch), as the reference uses
 its library there; an fp32 result of many rows comes 64 rows at a time from the
-hand-written kernel.
+hand-written kernel.  ``set_prefill_gemm("mfma")`` (or INFERNUM_PREFILL_GEMM=mfma
+in the environment) sends the many-row bf16 products to the hand-written
+LDS-tiled MFMA kernel instead, where it takes the size (K in steps of 64); it is
+correct at every size but slower than the library so far, hence not the default.
 
 ``epilogue="swiglu"`` returns silu(y[:, :N/2]) * y[:, N/2:]; the decode kernel
 does it while it joins its partial sums, the other paths in a kernel of its own.
@@ -18,12 +21,32 @@ does it while it joins its partial sums, the other paths in a kernel of its own.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional, Union
 
 import torch
 
 from ..kernels import api as K
 from ..kernels.api import SplitSum
+
+
+PREFILL_GEMMS = ("library", "mfma")
+_prefill_gemm = os.environ.get("INFERNUM_PREFILL_GEMM", "library")
+if _prefill_gemm not in PREFILL_GEMMS:
+    raise ValueError(f"INFERNUM_PREFILL_GEMM={_prefill_gemm!r}: one of {PREFILL_GEMMS}")
+
+
+def set_prefill_gemm(name: str) -> str:
+    """Chooses the bf16 product for more than 64 rows; returns the previous choice."""
+    global _prefill_gemm
+    if name not in PREFILL_GEMMS:
+        raise ValueError(f"prefill gemm {name!r}: one of {PREFILL_GEMMS}")
+    previous, _prefill_gemm = _prefill_gemm, name
+    return previous
+
+
+def prefill_gemm() -> str:
+    return _prefill_gemm
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -41,7 +64,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     elif x.dtype != torch.bfloat16:
         raise K.KernelError(f"linear: dtype {x.dtype} is not supported")
     elif out_dtype == torch.bfloat16:
-        y = torch.mm(x, w.t())                      # library product, fp32 accumulation
+        if _prefill_gemm == "mfma" and x.is_contiguous() and K.gemm_mfma_supported(M, N, Kdim):
+            y = K.gemm_mfma(x, w)
+        else:
+            y = torch.mm(x, w.t())                  # library product, fp32 accumulation
     elif K.gemm_skinny_supported(1, N, Kdim) and x.is_contiguous():
         # fp32 result from bf16 operands, many rows: 64 rows at a time through the skinny kernel
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)

@@ -235,6 +235,69 @@ def test_gemm_skinny_refuses_what_it_cannot_do():
         api.gemm_skinny(_rand(4, 64, dtype=torch.bfloat16), _rand(33, 64, dtype=torch.bfloat16), epilogue="swiglu")
 
 
+@pytest.mark.parametrize("tile", ["auto", "256x256", "128x256", "128x128"])
+@pytest.mark.parametrize("M,N,K_", [(65, 250, 64), (300, 1003, 192), (257, 516, 1024), (1, 7, 128), (640, 384, 320)])
+def test_gemm_mfma(tile, M, N, K_):
+    """The LDS-tiled product at sizes that fill no tile: edges in M and N, N that is no multiple of 4 (scalar
+    stores), one step of K and many, every tile shape."""
+    api = K()
+    a, w = _rand(M, K_, dtype=torch.bfloat16, seed=8), _rand(N, K_, dtype=torch.bfloat16, scale=0.1, seed=9)
+    want = a.double() @ w.double().t()
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    api.gemm_mfma(a, w, out, tile=tile)
+    # fp32 accumulation, one rounding to bf16
+    bound = 2e-5 * math.sqrt(K_) * 0.1 + 2.0 ** -8 * want.abs()
+    assert bool(((out.double() - want).abs() <= bound).all())
+    # a row's result does not depend on the rows beside it, nor on the tile shape
+    last = api.gemm_mfma(a[M - 1:M].contiguous(), w, tile=tile)
+    assert torch.equal(last[0], out[M - 1])
+    assert torch.equal(api.gemm_mfma(a, w, tile="128x128"), out)
+
+
+def test_gemm_mfma_picks_out_one_product():
+    """One large entry in a and one in w, at the last row, column and k: a wrong swizzle, stage or edge row
+    would move or lose it."""
+    api = K()
+    M, N, K_ = 515, 771, 448
+    a = torch.zeros(M, K_, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(N, K_, dtype=torch.bfloat16, device=DEV)
+    spots = [(0, 0, 0), (M - 1, N - 1, K_ - 1), (256, 255, 64), (129, 513, 71), (300, 2, 447)]
+    for i, (m, n, k) in enumerate(spots):
+        a[m, k] = 1 + i
+        w[n, k] = 2
+    want = a.float() @ w.float().t()
+    assert torch.equal(api.gemm_mfma(a, w).float(), want)
+
+
+def test_gemm_mfma_refuses_what_it_cannot_do():
+    api = K()
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma(_rand(80, 96, dtype=torch.bfloat16), _rand(32, 96, dtype=torch.bfloat16))      # K % 64
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma(_rand(80, 64), _rand(32, 64))                                                  # fp32
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma(_rand(80, 128, dtype=torch.bfloat16)[:, :64], _rand(32, 64, dtype=torch.bfloat16))
+
+
+def test_linear_with_the_hand_written_prefill_gemm():
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")   # the package exports the function under this name
+    x, w = _rand(200, 256, dtype=torch.bfloat16, seed=3), _rand(330, 256, dtype=torch.bfloat16, scale=0.1, seed=4)
+    lib = L.linear(x, w)
+    previous = L.set_prefill_gemm("mfma")
+    try:
+        own = L.linear(x, w)
+        act = L.linear(x, w, epilogue="swiglu")
+        odd = L.linear(x[:, :200].contiguous(), w[:, :200].contiguous())   # K = 200: the library takes it
+    finally:
+        L.set_prefill_gemm(previous)
+    want = x.double() @ w.double().t()
+    bound = 2e-5 * 16 * 0.1 + 2.0 ** -8 * want.abs()
+    assert bool(((own.double() - want).abs() <= bound).all()) and bool(((lib.double() - want).abs() <= bound).all())
+    assert torch.equal(act, K().swiglu(own, torch.empty(200, 165, dtype=torch.bfloat16, device=DEV)))
+    assert tuple(odd.shape) == (200, 330)
+
+
 def test_rope_from_partial_sums():
     """The rotary kernel joins a split product itself: same pages and queries as from the joined tensor."""
     api = K()
