@@ -18,6 +18,8 @@ recurrent state.
 """
 from __future__ import annotations
 
+import ctypes
+import re
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -25,82 +27,51 @@ import numpy as np
 import torch
 
 from ..parts.base import CacheSpec, CacheView, StateSpec
-from .pages import NO_PAGE, BlockTable, PageAllocator, PageError, pages_for
+from . import native
+from .pages import NO_PAGE, BlockTable, PageAllocator, PageError, pages_for  # noqa: F401  (NO_PAGE: part of this module's face)
+
+_KINDS = {"full": 0, "window": 1}
 
 
 class CacheGroup:
-    """Host bookkeeping of one group: its allocator and its requests' block tables."""
+    """One group as the host sees it: what kind it is, which schedule entries own pages in it, and its pool
+    (the tables themselves are kept natively by the manager)."""
 
-    def __init__(self, index: int, kind: str, window: int, page_size: int, num_pages: int):
+    def __init__(self, index: int, kind: str, window: int, page_size: int):
         self.index, self.kind, self.window = index, kind, int(window)
         self.page_size = int(page_size)
-        self.allocator = PageAllocator(num_pages)
-        self.tables: Dict[Hashable, BlockTable] = {}
         self.entries: List[int] = []         # schedule entries that own pages in this group
-
-    def pages_missing(self, req: Hashable, n_new: int) -> int:
-        t = self.tables[req]
-        return max(0, pages_for(t.num_tokens + n_new, self.page_size) - len(t.pages))
-
-    def grow(self, req: Hashable, n_new: int) -> bool:
-        t = self.tables[req]
-        got = self.allocator.allocate_many(self.pages_missing(req, n_new))
-        if got is None:
-            return False
-        t.pages.extend(got)
-        return True
-
-    def advance(self, req: Hashable, n_new: int) -> List[int]:
-        """Count n_new more tokens as stored; returns the pages a window has passed (now free)."""
-        t = self.tables[req]
-        t.num_tokens += n_new
-        if t.num_tokens > len(t.pages) * self.page_size:
-            raise PageError(f"request {req!r} stored {t.num_tokens} tokens in {len(t.pages)} pages")
-        freed: List[int] = []
-        if self.kind == "window" and self.window > 0:
-            # the next query stands at position num_tokens and sees keys >= num_tokens - window + 1
-            first_needed = max(0, t.num_tokens - self.window + 1) // self.page_size
-            while t.first_live < min(first_needed, len(t.pages)):
-                p = t.pages[t.first_live]
-                if p != NO_PAGE:
-                    self.allocator.free(p)
-                    freed.append(p)
-                    t.pages[t.first_live] = NO_PAGE
-                t.first_live += 1
-        return freed
-
-    def release(self, req: Hashable) -> List[int]:
-        t = self.tables.pop(req)
-        freed = t.live_pages()
-        for p in freed:
-            self.allocator.free(p)
-        return freed
+        self.allocator: Optional[PageAllocator] = None
 
 
 class StateSlotPool:
-    """Indices of per-request state records of fixed size."""
+    """Indices of per-request state records of fixed size (alone, or the slots of a cache manager)."""
 
-    def __init__(self, num_slots: int):
+    def __init__(self, num_slots: int, _view: Optional[ctypes.c_void_p] = None):
+        self._lib = native.lib()
         self.num_slots = int(num_slots)
-        self._free = list(range(self.num_slots - 1, -1, -1))
-        self._used = bytearray(self.num_slots)
+        if _view is not None:
+            self._h, self._owned = _view, False
+        else:
+            self._h = ctypes.c_void_p(self._lib.ia_cache_create(0, None, None, 1, 1, self.num_slots))
+            self._owned = True
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self._h:
+            self._lib.ia_cache_destroy(self._h)
+            self._h = None
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return int(self._lib.ia_cache_num_free_slots(self._h))
 
     def acquire(self) -> Optional[int]:
-        if not self._free:
-            return None
-        s = self._free.pop()
-        self._used[s] = 1
-        return s
+        s = int(self._lib.ia_cache_acquire_slot(self._h))
+        return None if s < 0 else s
 
     def release(self, slot: int) -> None:
-        if not 0 <= slot < self.num_slots or not self._used[slot]:
-            raise PageError(f"state slot {slot} is released twice or was never taken")
-        self._used[slot] = 0
-        self._free.append(slot)
+        if self._lib.ia_cache_release_slot(self._h, int(slot)) != 0:
+            raise PageError(self._lib.ia_cache_error(self._h).decode())
 
 
 @dataclass
@@ -113,7 +84,9 @@ class CacheConfig:
 
 class CacheManager:
     """``needs[i]`` = (CacheSpec or None, StateSpec or None) of schedule entry i;
-    ``cache_of[i]`` = the entry whose cache entry i reads, or None."""
+    ``cache_of[i]`` = the entry whose cache entry i reads, or None.
+
+    Requests are named by any hashable value here and by a number in the native bookkeeping."""
 
     def __init__(self, needs: Sequence[Tuple[Optional[CacheSpec], Optional[StateSpec]]],
                  cache_of: Sequence[Optional[int]], config: CacheConfig, dtype: torch.dtype = torch.float32,
@@ -122,6 +95,8 @@ class CacheManager:
         self.page_size = int(config.page_size)
         if self.page_size <= 0:
             raise ValueError("page_size must be positive")
+        if config.num_pages <= 0:
+            raise ValueError("a page pool needs at least one page")
         self.device = device
         self.dtype = dtype
         self.groups: List[CacheGroup] = []
@@ -134,16 +109,31 @@ class CacheManager:
             if cs is None:
                 self._entry_group.append(-1)
                 continue
+            if cs.kind not in _KINDS:
+                raise ValueError(f"cache kind {cs.kind!r}: one of {sorted(_KINDS)}")
             key = cs.group_key()
             if key not in key_to_group:
                 key_to_group[key] = len(self.groups)
-                self.groups.append(CacheGroup(len(self.groups), cs.kind, cs.window, self.page_size, config.num_pages))
+                self.groups.append(CacheGroup(len(self.groups), cs.kind, cs.window, self.page_size))
             g = key_to_group[key]
             self.groups[g].entries.append(i)
             self._entry_group.append(g)
-        self.slots = StateSlotPool(config.num_state_slots)
-        self._slot_of: Dict[Hashable, int] = {}
-        self._tokens: Dict[Hashable, int] = {}
+        # the bookkeeping itself, natively
+        self._lib = native.lib()
+        G = len(self.groups)
+        kinds = (ctypes.c_int * max(G, 1))(*[_KINDS[g.kind] for g in self.groups])
+        windows = (ctypes.c_int * max(G, 1))(*[g.window for g in self.groups])
+        self._h = ctypes.c_void_p(self._lib.ia_cache_create(G, kinds, windows, self.page_size, int(config.num_pages),
+                                                            int(config.num_state_slots)))
+        if not self._h:
+            raise ValueError("the cache could not be created: page_size, num_pages must be positive, slots not negative")
+        for g in self.groups:
+            g.allocator = PageAllocator(0, _view=self._lib.ia_cache_group_pool(self._h, g.index))
+        self.slots = StateSlotPool(config.num_state_slots, _view=self._h)
+        self._ids: Dict[Hashable, int] = {}          # request -> its number in the native bookkeeping
+        self._names: Dict[int, Hashable] = {}
+        self._next_id = 0
+        self._per_group = (ctypes.c_int * max(G, 1))()
         # device memory
         self.k_pages: List[Optional[torch.Tensor]] = [None] * len(needs)
         self.v_pages: List[Optional[torch.Tensor]] = [None] * len(needs)
@@ -160,91 +150,142 @@ class CacheManager:
                     self.state[i] = torch.zeros((config.num_state_slots,) + tuple(ss.shape), dtype=ss.dtype,
                                                 device=device)
 
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.ia_cache_destroy(self._h)
+            self._h = None
+
+    def _fail(self) -> None:
+        """Raise the native call's error, with the request's own name in place of its number."""
+        msg = self._lib.ia_cache_error(self._h).decode()
+        msg = re.sub(r"request #(\d+)", lambda m: f"request {self._names.get(int(m.group(1)), m.group(0))!r}", msg)
+        raise PageError(msg)
+
+    def _id(self, req: Hashable) -> int:
+        i = self._ids.get(req)
+        if i is None:
+            raise PageError(f"request {req!r} is not admitted")
+        return i
+
+    def native_handle(self) -> ctypes.c_void_p:
+        return self._h
+
+    def request_id(self, req: Hashable) -> int:
+        """The request's number in the native bookkeeping."""
+        return self._id(req)
+
     # ---- requests -------------------------------------------------------------
     def has(self, req: Hashable) -> bool:
-        return req in self._slot_of
+        return req in self._ids
 
     def requests(self) -> List[Hashable]:
-        return list(self._slot_of)
+        return list(self._ids)
 
     def admit(self, req: Hashable) -> bool:
         """Give the request empty block tables and a state slot; False when no slot is free."""
-        if req in self._slot_of:
+        if req in self._ids:
             raise PageError(f"request {req!r} is admitted twice")
-        slot = self.slots.acquire()
-        if slot is None:
+        rid = self._next_id
+        slot = int(self._lib.ia_cache_admit(self._h, rid))
+        if slot == native.HOST_ERROR:
+            self._fail()
+        if slot < 0:
             return False
-        self._slot_of[req] = slot
-        self._tokens[req] = 0
-        for g in self.groups:
-            g.tables[req] = BlockTable()
+        self._next_id += 1
+        self._ids[req] = rid
+        self._names[rid] = req
         for st in self.state:
             if st is not None:
                 st[slot].zero_()
         return True
 
     def state_slot(self, req: Hashable) -> int:
-        return self._slot_of[req]
+        return int(self._lib.ia_cache_state_slot(self._h, self._id(req)))
 
     def num_tokens(self, req: Hashable) -> int:
-        return self._tokens[req]
+        return int(self._lib.ia_cache_num_tokens(self._h, self._id(req)))
 
     def pages_needed(self, req: Optional[Hashable], n_new: int) -> List[int]:
         """Per group, the pages that n_new more tokens of the request would take from the pool
         (a request that is not admitted yet holds nothing)."""
-        if req is not None and req in self._slot_of:
-            return [g.pages_missing(req, n_new) for g in self.groups]
-        return [pages_for(n_new, g.page_size) for g in self.groups]
+        rid = self._ids.get(req) if req is not None else None
+        self._lib.ia_cache_pages_needed(self._h, int(rid is not None), rid or 0, int(n_new), self._per_group)
+        return list(self._per_group[:len(self.groups)])
 
     def tokens_that_fit(self, req: Optional[Hashable], promised: Optional[Sequence[int]] = None) -> int:
         """How many more tokens of the request the pool can hold, with ``promised[g]`` pages of
         every group already spoken for."""
-        best = 1 << 60
-        for i, g in enumerate(self.groups):
-            avail = g.allocator.num_free - (promised[i] if promised is not None else 0)
-            if req is not None and req in self._slot_of:
-                t = g.tables[req]
-                room = (len(t.pages) + max(avail, 0)) * g.page_size - t.num_tokens
-            else:
-                room = max(avail, 0) * g.page_size
-            best = min(best, room)
-        return max(best, 0)
+        rid = self._ids.get(req) if req is not None else None
+        prom = (ctypes.c_int * max(len(self.groups), 1))(*promised) if promised is not None else None
+        return int(self._lib.ia_cache_tokens_that_fit(self._h, int(rid is not None), rid or 0, prom))
 
     def can_reserve(self, req: Hashable, n_new: int) -> bool:
-        return all(g.allocator.can_allocate(g.pages_missing(req, n_new)) for g in self.groups)
+        return self._lib.ia_cache_can_reserve(self._h, self._id(req), int(n_new)) == 1
 
     def reserve(self, req: Hashable, n_new: int) -> bool:
         """Pages for the next n_new tokens in every group, or nothing at all."""
-        if not self.can_reserve(req, n_new):
-            return False
-        for g in self.groups:
-            ok = g.grow(req, n_new)
-            assert ok
-        return True
+        return self._lib.ia_cache_reserve(self._h, self._id(req), int(n_new)) == 1
+
+    def step_fits(self, reqs: Sequence[Hashable], q_lens: Sequence[int]) -> bool:
+        """Whether the pools and the state slots can take a whole step: ``q_lens[i]`` more tokens of
+        ``reqs[i]``, admitted or not."""
+        n = len(reqs)
+        ids = [self._ids.get(r) for r in reqs]
+        return self._lib.ia_cache_step_fits(
+            self._h, n, (ctypes.c_int64 * max(n, 1))(*[i or 0 for i in ids]),
+            (ctypes.c_int * max(n, 1))(*[int(i is not None) for i in ids]), (ctypes.c_int * max(n, 1))(*q_lens)) == 1
+
+    def _step_arrays(self, reqs: Sequence[Hashable], q_lens: Sequence[int]):
+        n = len(reqs)
+        return n, (ctypes.c_int64 * max(n, 1))(*[self._id(r) for r in reqs]), (ctypes.c_int * max(n, 1))(*q_lens)
+
+    def reserve_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int]) -> bool:
+        """Pages for ``q_lens[i]`` more tokens of every ``reqs[i]`` (all admitted), or nothing at all."""
+        rc = self._lib.ia_cache_reserve_step(self._h, *self._step_arrays(reqs, q_lens))
+        if rc == native.HOST_ERROR:
+            self._fail()
+        return rc == 1
+
+    def commit_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int]) -> None:
+        """``commit`` for every request of a step."""
+        if self._lib.ia_cache_commit_step(self._h, *self._step_arrays(reqs, q_lens)) != 0:
+            self._fail()
+        self._poison()
 
     def commit(self, req: Hashable, n_new: int) -> None:
         """The n_new tokens are stored; pages that a window has passed go back to the pool."""
-        self._tokens[req] += n_new
-        for g in self.groups:
-            self._poison(g, g.advance(req, n_new))
+        if self._lib.ia_cache_commit(self._h, self._id(req), int(n_new)) != 0:
+            self._fail()
+        self._poison()
 
     def release(self, req: Hashable) -> None:
         """The request is over (finished, cancelled or preempted): everything it holds goes back."""
-        slot = self._slot_of.pop(req, None)
-        if slot is None:
+        rid = self._ids.get(req)
+        if rid is None:
             raise PageError(f"request {req!r} is released but not admitted")
-        del self._tokens[req]
-        for g in self.groups:
-            self._poison(g, g.release(req))
-        self.slots.release(slot)
+        if self._lib.ia_cache_release(self._h, rid) != 0:
+            self._fail()
+        del self._ids[req]
+        del self._names[rid]
+        self._poison()
 
-    def _poison(self, g: CacheGroup, pages: List[int]) -> None:
-        if not self.config.poison_freed_pages or not pages or self.device is None:
+    def _poison(self) -> None:
+        """Fill the pages that the last commit or release gave back with NaN (when asked to)."""
+        if not self.config.poison_freed_pages or self.device is None:
             return
-        idx = torch.tensor(pages, dtype=torch.long, device=self.device)
-        for e in g.entries:
-            self.k_pages[e].index_fill_(0, idx, float("nan"))
-            self.v_pages[e].index_fill_(0, idx, float("nan"))
+        n = int(self._lib.ia_cache_last_freed(self._h, None, 0))
+        if n == 0:
+            return
+        pairs = (ctypes.c_int * (2 * n))()
+        self._lib.ia_cache_last_freed(self._h, pairs, n)
+        for g in self.groups:
+            pages = [pairs[2 * i + 1] for i in range(n) if pairs[2 * i] == g.index]
+            if not pages:
+                continue
+            idx = torch.tensor(pages, dtype=torch.long, device=self.device)
+            for e in g.entries:
+                self.k_pages[e].index_fill_(0, idx, float("nan"))
+                self.v_pages[e].index_fill_(0, idx, float("nan"))
 
     # ---- what a step needs --------------------------------------------------------
     def free_pages(self, group: int = 0) -> int:
@@ -254,35 +295,41 @@ class CacheManager:
         return min((g.allocator.num_free for g in self.groups), default=1 << 30)
 
     def block_table(self, group: int, req: Hashable) -> BlockTable:
-        return self.groups[group].tables[req]
+        """A copy of the request's block table in the group."""
+        rid = self._id(req)
+        tokens, first = ctypes.c_int64(0), ctypes.c_int(0)
+        n = int(self._lib.ia_cache_table(self._h, int(group), rid, None, 0, ctypes.byref(tokens), ctypes.byref(first)))
+        if n == native.HOST_ERROR:
+            self._fail()
+        pages = (ctypes.c_int * max(n, 1))()
+        self._lib.ia_cache_table(self._h, int(group), rid, pages, n, None, None)
+        return BlockTable(list(pages[:n]), tokens.value, first.value)
+
+    def num_pages_held(self, group: int, req: Hashable) -> int:
+        """Length of the request's block table in the group (pages given back by a window count)."""
+        n = int(self._lib.ia_cache_table(self._h, int(group), self._id(req), None, 0, None, None))
+        if n == native.HOST_ERROR:
+            self._fail()
+        return n
 
     def block_table_rows(self, group: int, reqs: Sequence[Hashable], width: Optional[int] = None) -> np.ndarray:
         """int32 [len(reqs), width], NO_PAGE where a request holds no page."""
-        g = self.groups[group]
+        tables = [self.block_table(group, r).pages for r in reqs]
         if width is None:
-            width = max((len(g.tables[r].pages) for r in reqs), default=1)
+            width = max((len(t) for t in tables), default=1)
         width = max(width, 1)
         out = np.full((len(reqs), width), NO_PAGE, dtype=np.int32)
-        for i, r in enumerate(reqs):
-            p = g.tables[r].pages
+        for i, p in enumerate(tables):
             out[i, :len(p)] = p
         return out
 
     def token_slots(self, group: int, req: Hashable, start: int, n: int) -> np.ndarray:
         """page * page_size + offset of positions start .. start+n-1 (pages must be reserved)."""
-        g = self.groups[group]
-        if n == 1:                                   # a decoded token: no arrays needed
-            t = g.tables[req].pages
-            i = start // g.page_size
-            if i >= len(t) or t[i] < 0:
-                raise PageError(f"request {req!r} has no page for position {start}")
-            return np.asarray([t[i] * g.page_size + start % g.page_size], dtype=np.int32)
-        pos = np.arange(start, start + n, dtype=np.int64)
-        pages = np.asarray(g.tables[req].pages, dtype=np.int64)
-        idx = pos // g.page_size
-        if n and (idx[-1] >= len(pages) or (pages[idx] < 0).any()):
-            raise PageError(f"request {req!r} has no page for positions {start}..{start + n - 1}")
-        return (pages[idx] * g.page_size + pos % g.page_size).astype(np.int32)
+        out = np.empty(max(n, 0), dtype=np.int32)
+        if self._lib.ia_cache_token_slots(self._h, int(group), self._id(req), int(start), int(n),
+                                          out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))) != 0:
+            self._fail()
+        return out
 
     def views(self) -> List[CacheView]:
         """One CacheView per schedule entry."""
@@ -296,20 +343,7 @@ class CacheManager:
     # ---- invariants (tests) ---------------------------------------------------------
     def check(self) -> None:
         """Every page is free or held by exactly one request; counts agree."""
-        for g in self.groups:
-            held: Dict[int, Hashable] = {}
-            for r, t in g.tables.items():
-                for p in t.live_pages():
-                    if p in held:
-                        raise PageError(f"group {g.index}: page {p} is held by {held[p]!r} and {r!r}")
-                    if not g.allocator.is_used(p):
-                        raise PageError(f"group {g.index}: page {p} of {r!r} is marked free")
-                    held[p] = r
-                if t.num_tokens > len(t.pages) * g.page_size:
-                    raise PageError(f"group {g.index}: {r!r} holds too few pages")
-            if len(held) != g.allocator.num_used:
-                raise PageError(f"group {g.index}: {g.allocator.num_used} pages in use, {len(held)} held: a page is lost")
-        if len(self._slot_of) != self.slots.num_slots - self.slots.num_free:
-            raise PageError("state slots in use do not match the admitted requests")
-        if len(set(self._slot_of.values())) != len(self._slot_of):
-            raise PageError("two requests share a state slot")
+        if self._lib.ia_cache_check(self._h) != 0:
+            self._fail()
+        if int(self._lib.ia_cache_num_requests(self._h)) != len(self._ids):
+            raise PageError("the native bookkeeping and the names of the requests disagree")

@@ -5,10 +5,16 @@ empty, and a loud failure on a double free or a page outside the pool, as
 infernum/src/block_allocator.rs:27-110; the in-use flags make the double-free
 check O(1).  A request's pages per group are a block table: page numbers in the
 order of positions, ``page_size`` tokens each (block_allocator.rs:119-198).
+
+The bookkeeping itself is native (``csrc/host_core.cpp``); the classes here are
+its Python face.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import List, Optional
+
+from . import native
 
 NO_PAGE = -1
 
@@ -18,47 +24,51 @@ class PageError(RuntimeError):
 
 
 class PageAllocator:
-    def __init__(self, num_pages: int):
-        if num_pages <= 0:
-            raise ValueError("a page pool needs at least one page")
-        self.num_pages = int(num_pages)
-        self._free: List[int] = list(range(self.num_pages - 1, -1, -1))   # pop() gives 0 first
-        self._in_use = bytearray(self.num_pages)
+    """A pool of ``num_pages`` pages; ``_view`` wraps a pool that a cache manager owns."""
+
+    def __init__(self, num_pages: int, _view: Optional[int] = None):
+        self._lib = native.lib()
+        if _view is not None:
+            self._h, self._owned = ctypes.c_void_p(_view), False
+        else:
+            if num_pages <= 0:
+                raise ValueError("a page pool needs at least one page")
+            self._h, self._owned = ctypes.c_void_p(self._lib.ia_pool_create(int(num_pages))), True
+        self.num_pages = int(self._lib.ia_pool_num_pages(self._h))
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self._h:
+            self._lib.ia_pool_destroy(self._h)
+            self._h = None
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return int(self._lib.ia_pool_num_free(self._h))
 
     @property
     def num_used(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.num_free
 
     def can_allocate(self, n: int) -> bool:
-        return n <= len(self._free)
+        return n <= self.num_free
 
     def allocate(self) -> Optional[int]:
-        if not self._free:
-            return None
-        p = self._free.pop()
-        self._in_use[p] = 1
-        return p
+        p = int(self._lib.ia_pool_allocate(self._h))
+        return None if p < 0 else p
 
     def allocate_many(self, n: int) -> Optional[List[int]]:
         """n pages or none at all."""
-        if n > len(self._free):
+        out = (ctypes.c_int * max(n, 1))()
+        if not self._lib.ia_pool_allocate_many(self._h, int(n), out):
             return None
-        return [self.allocate() for _ in range(n)]
+        return list(out[:n])
 
     def free(self, page: int) -> None:
-        if not 0 <= page < self.num_pages:
-            raise PageError(f"page {page} is outside the pool of {self.num_pages}")
-        if not self._in_use[page]:
-            raise PageError(f"page {page} is freed twice")
-        self._in_use[page] = 0
-        self._free.append(page)
+        if self._lib.ia_pool_free(self._h, int(page)) != 0:
+            raise PageError(self._lib.ia_pool_error(self._h).decode())
 
     def is_used(self, page: int) -> bool:
-        return bool(self._in_use[page])
+        return bool(self._lib.ia_pool_is_used(self._h, int(page)))
 
 
 def pages_for(num_tokens: int, page_size: int) -> int:
@@ -66,15 +76,15 @@ def pages_for(num_tokens: int, page_size: int) -> int:
 
 
 class BlockTable:
-    """Pages of one request in one group.  ``pages[i]`` holds positions
-    [i * page_size, (i + 1) * page_size); NO_PAGE where a window has passed."""
+    """Pages of one request in one group (a copy of the native table at the time it was asked for).
+    ``pages[i]`` holds positions [i * page_size, (i + 1) * page_size); NO_PAGE where a window has passed."""
 
     __slots__ = ("pages", "num_tokens", "first_live")
 
-    def __init__(self) -> None:
-        self.pages: List[int] = []
-        self.num_tokens = 0
-        self.first_live = 0      # pages before this index have been given back
+    def __init__(self, pages: Optional[List[int]] = None, num_tokens: int = 0, first_live: int = 0) -> None:
+        self.pages: List[int] = list(pages or [])
+        self.num_tokens = int(num_tokens)
+        self.first_live = int(first_live)      # pages before this index have been given back
 
     def live_pages(self) -> List[int]:
         return [p for p in self.pages[self.first_live:] if p != NO_PAGE]

@@ -44,6 +44,9 @@ CORE_SOURCES = [
     "sampling.hip",
 ]
 HEADERS = ["common.h"]
+# The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
+HOST_SOURCES = ["host_core.cpp"]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
 # Head sizes whose attention library `build_all` compiles ahead of time.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)
@@ -60,6 +63,15 @@ def _say(msg: str) -> None:
 
 def find_hipcc() -> Optional[str]:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def find_cxx() -> Optional[str]:
+    """A C++ compiler for the host library; hipcc (a clang) serves when there is no other."""
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 find_hipcc()):
         if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
             return cand
     return None
@@ -91,18 +103,20 @@ def _existing(files: Sequence[str]) -> List[str]:
     return [f for f in files if os.path.isfile(os.path.join(CSRC_DIR, f))]
 
 
-def _fingerprint(sources: Sequence[str], defines: Sequence[str]) -> str:
+def _fingerprint(sources: Sequence[str], defines: Sequence[str], host: bool = False) -> str:
     h = hashlib.sha256()
-    for f in list(sources) + _existing(HEADERS):
+    for f in list(sources) + ([] if host else _existing(HEADERS)):
         with open(os.path.join(CSRC_DIR, f), "rb") as fh:
             h.update(f.encode())
             h.update(fh.read())
-    h.update(" ".join(HIPCC_FLAGS + list(defines)).encode())
+    h.update(" ".join((CXX_FLAGS if host else HIPCC_FLAGS) + list(defines)).encode())
     return h.hexdigest()
 
 
 def library_plan(name: str) -> Dict:
-    """Sources and defines of a library by its name ('core' or 'attn_d<D>')."""
+    """Sources and defines of a library by its name ('core', 'attn_d<D>' or 'host')."""
+    if name == "host":
+        return {"sources": _existing(HOST_SOURCES), "defines": [], "host": True}
     if name == "core":
         return {"sources": _existing(CORE_SOURCES), "defines": []}
     if name.startswith("attn_d"):
@@ -130,8 +144,32 @@ def _heartbeat(stop: threading.Event, what: str) -> None:
         _say(f"still compiling {what} ({time.time() - t0:.0f} s)")
 
 
+def _compile_host_library(name: str, plan: Dict) -> str:
+    cxx = find_cxx()
+    if cxx is None:
+        raise BuildError("no C++ compiler found for the host library (looked at $CXX, g++, c++, clang++, hipcc)")
+    out = library_path(name)
+    tmp_dir = tempfile.mkdtemp(prefix=f"ia_{name}_", dir=lib_dir())
+    t0 = time.time()
+    try:
+        tmp_out = os.path.join(tmp_dir, "lib.so")
+        cmd = [cxx] + CXX_FLAGS + ["-shared", "-o", tmp_out] + [os.path.join(CSRC_DIR, f) for f in plan["sources"]]
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, cwd=tmp_dir)
+        if r.returncode != 0:
+            raise BuildError(f"{os.path.basename(cxx)} failed on {', '.join(plan['sources'])}:\n{r.stderr[-6000:]}")
+        os.replace(tmp_out, out)
+        with open(_stamp_path(name), "w") as f:
+            json.dump({"fingerprint": _fingerprint(plan["sources"], plan["defines"], host=True)}, f)
+    finally:
+        shutil.rmtree(tmp_dir, ignore_errors=True)
+    _say(f"built {os.path.basename(out)} in {time.time() - t0:.1f} s")
+    return out
+
+
 def compile_library(name: str) -> str:
     """Compile one library now, whether or not it is there already."""
+    if library_plan(name).get("host"):
+        return _compile_host_library(name, library_plan(name))
     hipcc = find_hipcc()
     if hipcc is None:
         raise BuildError("hipcc not found: the HIP kernels cannot be compiled (looked at $HIPCC, PATH, /opt/rocm/bin)")
@@ -177,19 +215,20 @@ def ensure(name: str) -> str:
     if os.path.isfile(out):
         try:
             with open(_stamp_path(name)) as f:
-                if json.load(f).get("fingerprint") == _fingerprint(plan["sources"], plan["defines"]):
+                if json.load(f).get("fingerprint") == _fingerprint(plan["sources"], plan["defines"],
+                                                                   host=bool(plan.get("host"))):
                     return out
         except (OSError, ValueError):
             pass
-        if find_hipcc() is None:
-            _say(f"{os.path.basename(out)} may be older than its sources and hipcc is not here: using it as is")
+        if (find_cxx() if plan.get("host") else find_hipcc()) is None:
+            _say(f"{os.path.basename(out)} may be older than its sources and no compiler is here: using it as is")
             return out
     return compile_library(name)
 
 
 def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> List[str]:
     """Compile every library (the core one, and attention for the given head sizes)."""
-    names = ["core"]
+    names = ["host", "core"]
     if os.path.isfile(os.path.join(CSRC_DIR, "attention_mfma.hip")):
         names += [f"attn_d{d}" for d in head_dims]
     workers = max(1, min(4, int(os.environ.get("MAX_JOBS", "8"))))

@@ -12,16 +12,18 @@ infernum-cuda/src/inner/cuda/paged_kv_cache.rs:158-159.)
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheManager, native
 from ..parts.base import StepContext
 
 PREFILL_TILE_ROWS = 64      # query rows per workgroup tile of the MFMA prefill attention
+POW2_WIDTH = -1             # for pack_step's bt_width
 
 
 class StepError(ValueError):
@@ -33,10 +35,6 @@ class StepEntry:
     request: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)     # places among ``tokens`` whose logits are wanted
-
-
-def _align4(n: int) -> int:
-    return (n + 3) & ~3
 
 
 @dataclass
@@ -91,43 +89,32 @@ def check_entries(entries: Sequence[StepEntry], vocab_size: int, max_tokens: int
 
 def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optional[int] = None) -> PackedStep:
     """Pages for the entries' tokens must be reserved already.  ``bt_width`` widens the block
-    tables to a fixed number of columns (filled with NO_PAGE)."""
-    order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
+    tables to a fixed number of columns (filled with NO_PAGE); ``POW2_WIDTH`` to the power of two
+    (at least 8) that holds the longest table of any group.  The arrays are laid out natively
+    (``ia_cache_pack_step``); the buffer returned is a copy of the native one."""
+    n = len(entries)
+    G = len(cache.groups)
+    q_lens_in = [len(e.tokens) for e in entries]
+    want_counts = [len(e.want) for e in entries]
+    tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=sum(q_lens_in))
+    wants = np.fromiter((w for e in entries for w in e.want), dtype=np.int32, count=sum(want_counts))
+    S = 8 + 2 * G
+    meta = np.empty(7 + 2 * S + G + 2 * n, dtype=np.int32)
+    lib, h = native.lib(), cache.native_handle()
+    i32 = ctypes.POINTER(ctypes.c_int32)
+    rc = lib.ia_cache_pack_step(
+        h, n, (ctypes.c_int64 * max(n, 1))(*[cache.request_id(e.request) for e in entries]),
+        (ctypes.c_int * max(n, 1))(*q_lens_in), tokens.ctypes.data_as(i32), (ctypes.c_int * max(n, 1))(*want_counts),
+        wants.ctypes.data_as(i32), int(bt_width or 0), PREFILL_TILE_ROWS, meta.ctypes.data_as(i32), int(meta.size))
+    if rc != 0:
+        cache._fail()
+    total, num_decode, num_tiles, num_rows = (int(v) for v in meta[:4])
+    offsets = [int(v) for v in meta[7:7 + S]]
+    sizes = [int(v) for v in meta[7 + S:7 + 2 * S]]
+    cols = [int(v) for v in meta[7 + 2 * S:7 + 2 * S + G]]
+    order = [int(v) for v in meta[7 + 2 * S + G:7 + 2 * S + G + n]]
+    ctx_lens = [int(v) for v in meta[7 + 2 * S + G + n:7 + 2 * S + G + 2 * n]]
+    host = np.ctypeslib.as_array(lib.ia_cache_packed(h), shape=(total,)).copy()
     batch = [entries[i] for i in order]
-    B = len(batch)
-    num_decode = sum(1 for e in batch if len(e.tokens) == 1)
-    q_lens = [len(e.tokens) for e in batch]
-    ctx_lens = [cache.num_tokens(e.request) for e in batch]
-    starts = np.zeros(B + 1, dtype=np.int32)
-    starts[1:] = np.cumsum(q_lens)
-    start_of = {e.request: int(starts[i]) for i, e in enumerate(batch)}
-    reqs = [e.request for e in batch]
-    if num_decode == B:
-        token_ids = np.fromiter((e.tokens[0] for e in batch), dtype=np.int32, count=B)
-        positions = np.asarray(ctx_lens, dtype=np.int32)
-        token_seq = np.arange(B, dtype=np.int32)
-    else:
-        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in batch])
-        positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(ctx_lens, q_lens)])
-        token_seq = np.repeat(np.arange(B, dtype=np.int32), q_lens)
-    logit_rows = np.asarray([start_of[e.request] + w for e in entries for w in e.want], dtype=np.int32)
-    state_slots = np.asarray([cache.state_slot(r) for r in reqs], dtype=np.int32)
-    tiles = [(s, r) for s in range(num_decode, B) for r in range(0, q_lens[s], PREFILL_TILE_ROWS)]
-    tiles_np = np.asarray(tiles, dtype=np.int32).reshape(-1)
-    segs: List[np.ndarray] = [token_ids, positions, token_seq, starts, np.asarray(ctx_lens, dtype=np.int32),
-                              state_slots, logit_rows, tiles_np]
-    bt_shapes = []
-    for g in cache.groups:
-        bt = cache.block_table_rows(g.index, reqs, bt_width)
-        bt_shapes.append(bt.shape)
-        segs.append(np.concatenate([cache.token_slots(g.index, r, c, q) for r, c, q in zip(reqs, ctx_lens, q_lens)]))
-        segs.append(bt.reshape(-1))
-    offsets, total = [], 0
-    for s in segs:
-        offsets.append(total)
-        total += _align4(max(s.size, 1))
-    host = np.zeros(total, dtype=np.int32)
-    for o, s in zip(offsets, segs):
-        host[o:o + s.size] = s
-    return PackedStep(host, offsets, [s.size for s in segs], bt_shapes, batch, q_lens, ctx_lens, num_decode,
-                      len(tiles), int(logit_rows.size))
+    return PackedStep(host, offsets, sizes, [(n, c) for c in cols], batch, [q_lens_in[i] for i in order], ctx_lens,
+                      num_decode, num_tiles, num_rows)

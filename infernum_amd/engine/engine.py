@@ -21,7 +21,7 @@ from ..cache import CacheConfig, CacheManager
 from ..models.model import DecoderModel
 from ..parts.base import Runtime
 
-from .batch import StepEntry, StepError, check_entries, pack_step  # noqa: F401  (StepError is part of this module's face)
+from .batch import POW2_WIDTH, StepEntry, StepError, check_entries, pack_step  # noqa: F401  (StepError is part of this module's face)
 
 
 class OutOfPages(RuntimeError):
@@ -108,15 +108,8 @@ class Engine:
 
     # ---- the step ------------------------------------------------------------------
     def pages_short(self, entries: Sequence[StepEntry]) -> bool:
-        """True when the pool cannot hold this step's new tokens."""
-        need = [0] * len(self.cache.groups)
-        for e in entries:
-            for i, n in enumerate(self.cache.pages_needed(e.request, len(e.tokens))):
-                need[i] += n
-        if any(n > g.allocator.num_free for n, g in zip(need, self.cache.groups)):
-            return True
-        new = sum(1 for e in entries if not self.cache.has(e.request))
-        return new > self.cache.slots.num_free
+        """True when the pools or the state slots cannot hold this step's new tokens."""
+        return not self.cache.step_fits([e.request for e in entries], [len(e.tokens) for e in entries])
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one batch; returns logits [sum(len(want)), vocab] fp32 in the order of entries and of ``want``."""
@@ -129,19 +122,19 @@ class Engine:
             total = sum(len(e.tokens) for e in entries)
             raise OutOfPages(f"not enough free pages or state slots for a step of {total} tokens")
         cache = self.cache
-        for e in entries:
-            if not cache.has(e.request):
-                cache.admit(e.request)
-            ok = cache.reserve(e.request, len(e.tokens))
-            assert ok
+        reqs, q_lens = [e.request for e in entries], [len(e.tokens) for e in entries]
+        for r in reqs:
+            if not cache.has(r):
+                cache.admit(r)
+        ok = cache.reserve_step(reqs, q_lens)
+        assert ok
         if all(len(e.tokens) == 1 for e in entries):
             logits = self._decode_step(entries)
         else:
             packed = pack_step(cache, entries)
             ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
             logits = self.model.forward(ctx, self.views)
-        for e in entries:
-            cache.commit(e.request, len(e.tokens))
+        cache.commit_step(reqs, q_lens)
         self.steps_run += 1
         return logits
 
@@ -150,15 +143,8 @@ class Engine:
         kernels are told that width as the longest length, so that a shape's launches are the same from
         step to step, recorded or not."""
         cache = self.cache
-        widths = []
-        for g in cache.groups:
-            need = max(len(g.tables[e.request].pages) for e in entries)
-            w = 8
-            while w < need:
-                w *= 2
-            widths.append(w)
-        width = max(widths) if widths else None
-        packed = pack_step(cache, entries, bt_width=width)
+        packed = pack_step(cache, entries, bt_width=POW2_WIDTH)
+        width = packed.bt_shapes[0][1] if packed.bt_shapes else None
         limit = (width or 0) * cache.page_size
         key = (len(entries), width, packed.num_logit_rows)
         g = self._graphs.get(key)
