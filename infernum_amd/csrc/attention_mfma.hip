@@ -359,9 +359,14 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
   constexpr int PF_THREADS = 4 * HGW * 64;
   const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, qd = lane >> 4;
   const int wave = (tid >> 6) & 3, hgw = tid >> 8;      // group of 16 rows, group of CT heads
-  const int sidx = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
+  // Workgroups start in the order of their number: all heads of the first tile, then of the next (the
+  // host lists the tiles with the most keys first, so that the long ones do not start last), and the
+  // key/value heads of one tile go to different dies, each of which then keeps its head's keys in its L2.
+  const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+  const int tile = lin / gridDim.y, by = lin - tile * gridDim.y;
+  const int sidx = tiles[2 * tile], row0 = tiles[2 * tile + 1];
   const int G = nh / nkv, HC = (G + CT * HGW - 1) / (CT * HGW);
-  const int g = blockIdx.y / HC, hc = blockIdx.y - g * HC;
+  const int g = by / HC, hc = by - g * HC;
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
   const int rows_here = (qlen - row0) < 64 ? (qlen - row0) : 64;      // rows of this workgroup (>= 1)
   const int rb = row0 + wave * 16;                                     // first row of this wave

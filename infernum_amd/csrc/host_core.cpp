@@ -18,6 +18,7 @@
 #include <cstring>
 #include <string>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -435,7 +436,8 @@ int ia_cache_token_slots(void* h, int g, int64_t req, int64_t start, int n, int3
 //
 // Segments of the buffer, each aligned to 4 values: 0 token ids, 1 positions, 2 row of each token,
 // 3 first token of each row (n + 1), 4 tokens stored before the step per row, 5 state slots, 6 rows of the
-// wanted logits, 7 prefill tiles (row, first query) pairs of tile_rows queries, then per group:
+// wanted logits, 7 prefill tiles (row, first query) pairs of tile_rows queries, the ones with the most
+// keys before them first, then per group:
 // 8 + 2 g slots of the tokens in the pages, 9 + 2 g block tables [n, columns].
 //
 // meta (int32): [0] buffer length, [1] single-token rows, [2] tiles, [3] wanted rows, [4] longest portion,
@@ -534,11 +536,6 @@ int ia_cache_pack_step(void* h, int n, const int64_t* reqs, const int* q_lens, c
     starts[r] = (int32_t)at;
     ctxs[r] = (int32_t)ctx[(size_t)r];
     slots[r] = c->slot_of[reqs[e]];
-    if (r >= num_decode)
-      for (int64_t q0 = 0; q0 < q; q0 += tile_rows) {
-        tile[t_at++] = r;
-        tile[t_at++] = (int32_t)q0;
-      }
     for (int g = 0; g < G; ++g) {
       Group& grp = c->groups[(size_t)g];
       const std::vector<int>& pages = grp.tables[reqs[e]].pages;
@@ -554,6 +551,20 @@ int ia_cache_pack_step(void* h, int n, const int64_t* reqs, const int* q_lens, c
     }
   }
   starts[n] = (int32_t)N;
+  // tiles with the most keys before them first: workgroups start in this order, and the long ones
+  // must not start last
+  {
+    std::vector<std::pair<int64_t, std::pair<int, int>>> list;   // (keys before the tile, (row, first query))
+    for (int r = num_decode; r < n; ++r)
+      for (int64_t q0 = 0; q0 < q_lens[order[(size_t)r]]; q0 += tile_rows)
+        list.push_back({ctx[(size_t)r] + q0, {r, (int)q0}});
+    std::stable_sort(list.begin(), list.end(),
+                     [](const auto& a, const auto& b) { return a.first > b.first; });
+    for (const auto& t : list) {
+      tile[t_at++] = t.second.first;
+      tile[t_at++] = t.second.second;
+    }
+  }
   // wanted rows in the order of the entries as given and of their places
   int64_t w_at = 0;
   for (int e = 0; e < n; ++e)

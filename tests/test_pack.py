@@ -30,8 +30,11 @@ def plain_pack(cache, entries, bt_width=None):
         "seq_starts": starts, "seq_ctx": ctx,
         "state_slots": [cache.state_slot(e.request) for e in batch],
         "logit_rows": [starts[row[e.request]] + w for e in entries for w in e.want],
-        "tiles": [v for r, n in enumerate(q) if n != 1 for q0 in range(0, n, PREFILL_TILE_ROWS) for v in (r, q0)],
     }
+    # tiles of 64 queries of the portions, the ones with the most keys before them first
+    tiles = [(r, q0) for r, n in enumerate(q) if n != 1 for q0 in range(0, n, PREFILL_TILE_ROWS)]
+    tiles.sort(key=lambda t: -(ctx[t[0]] + t[1]))
+    out["tiles"] = [v for t in tiles for v in t]
     ps = cache.page_size
     for g in range(len(cache.groups)):
         tables = [cache.block_table(g, e.request).pages for e in batch]
