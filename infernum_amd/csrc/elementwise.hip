@@ -241,6 +241,13 @@ __device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t 
   return v;
 }
 
+// The rotation of one pair, in one fixed order of roundings (a product, then a fused multiply-add), so that
+// every kernel that rotates gives the same bits.
+__device__ __forceinline__ void rope_pair(float a, float b, float cs, float sn, float& lo, float& hi) {
+  lo = __builtin_fmaf(a, cs, -(b * sn));
+  hi = __builtin_fmaf(a, sn, b * cs);
+}
+
 // grid (N, ceil(heads / 4)), 256 threads: one wave per (token, head), so that a handful of decoded tokens
 // still spread over the GPU; heads are nh queries, then nkv keys, then nkv values.
 template <typename TS, typename T>
@@ -278,11 +285,75 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restric
     sincosf(pos * inv_freq[i], &sn, &cs);
     const float a = load_split_sum(x + i, splits, split_stride);
     const float b = load_split_sum(x + i + half, splits, split_stride);
-    dst[i] = from_float<T>(a * cs - b * sn);
-    dst[i + half] = from_float<T>(a * sn + b * cs);
+    float lo, hi;
+    rope_pair(a, b, cs, sn, lo, hi);
+    dst[i] = from_float<T>(lo);
+    dst[i + half] = from_float<T>(hi);
   }
   if (!is_q || copy_q_tail)           // values beyond the rotated part are plain copies
     for (int i = rot + lane; i < d; i += 64) dst[i] = from_float<T>(load_split_sum(x + i, splits, split_stride));
+}
+
+// Many tokens (a prompt's portion): one workgroup per token takes all its heads with 8- or 16-byte loads
+// and stores, and the angles of the token are worked out once for all heads.  One part only (splits == 1),
+// rot a multiple of 8, d, row_stride and q_stride multiples of 4, d <= 256.  Same arithmetic as the kernel
+// above: a token's values do not depend on which of the two ran.
+template <typename TS, typename T>
+__global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(
+    const TS* __restrict__ src, T* __restrict__ q_out, int q_stride, const int* __restrict__ positions,
+    const int* __restrict__ slots, const float* __restrict__ inv_freq, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int row_stride, int nh, int nkv, int d, int rot, int page_size, int num_pages,
+    int write_kv, int copy_q_tail) {
+  __shared__ __attribute__((aligned(16))) float cs_[128], sn_[128];
+  const int n = blockIdx.x, tid = threadIdx.x;
+  const int half = rot >> 1;
+  const float pos = (float)positions[n];
+  for (int i = tid; i < half; i += 256) {
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    sn_[i] = sn;
+    cs_[i] = cs;
+  }
+  __syncthreads();
+  const int slot = (write_kv && slots) ? slots[n] : -1;
+  const bool do_write = slot >= 0 && slot < num_pages * page_size;
+  const int page = do_write ? slot / page_size : 0;
+  const int off = do_write ? slot % page_size : 0;
+  const TS* row = src + (size_t)n * row_stride;
+  const int heads = nh + (do_write ? nkv : 0);
+  const int per_head = half >> 2;
+  for (int it = tid; it < heads * per_head; it += 256) {
+    const int head = it / per_head, i = (it - head * per_head) << 2;
+    const TS* x = row + (size_t)head * d;
+    T* dst = head < nh ? q_out + (size_t)n * q_stride + (size_t)head * d
+                       : k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
+    const float4 a = load4(x + i), b = load4(x + i + half);
+    const float4 c = *reinterpret_cast<const float4*>(cs_ + i), sn = *reinterpret_cast<const float4*>(sn_ + i);
+    float4 lo, hi;
+    rope_pair(a.x, b.x, c.x, sn.x, lo.x, hi.x);
+    rope_pair(a.y, b.y, c.y, sn.y, lo.y, hi.y);
+    rope_pair(a.z, b.z, c.z, sn.z, lo.z, hi.z);
+    rope_pair(a.w, b.w, c.w, sn.w, lo.w, hi.w);
+    store4(dst + i, lo);
+    store4(dst + i + half, hi);
+  }
+  if (rot < d) {                       // values beyond the rotated part are plain copies
+    const int tail4 = (d - rot) >> 2;
+    for (int it = tid; it < heads * tail4; it += 256) {
+      const int head = it / tail4, i = rot + ((it - head * tail4) << 2);
+      if (head < nh && !copy_q_tail) continue;
+      T* dst = head < nh ? q_out + (size_t)n * q_stride + (size_t)head * d
+                         : k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
+      store4(dst + i, load4(row + (size_t)head * d + i));
+    }
+  }
+  if (do_write) {                      // values: plain copies into the transposed pages
+    const TS* v = row + (size_t)(nh + nkv) * d;
+    for (int it = tid; it < nkv * d; it += 256) {
+      const int g = it / d, i = it - g * d;
+      v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] = from_float<T>(to_float(v[it]));
+    }
+  }
 }
 
 // src: [splits, src_rows, row_stride] of src_dtype; q_out, pages: act_dtype.
@@ -301,6 +372,21 @@ extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int
   const int heads = nh + (write_kv ? 2 * nkv : 0);
   if ((heads + 3) / 4 > 65535) return IA_ERR_UNSUPPORTED;
   const dim3 grid(N, (heads + 3) / 4);
+  const bool aligned = (((uintptr_t)src | (uintptr_t)q_out | (uintptr_t)k_pages) & 15) == 0;
+  if (N >= 32 && splits == 1 && (rot & 7) == 0 && (d & 3) == 0 && d <= 256 && (row_stride & 3) == 0 &&
+      (q_stride & 3) == 0 && aligned) {
+#define ROPE_ROWS_LAUNCH(TS, T)                                                                                    \
+  rope_kv_append_rows_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, (T*)q_out, q_stride, positions, slots,  \
+                                                           inv_freq, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
+                                                           d, rot, page_size, num_pages, write_kv, copy_q_tail)
+    if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_ROWS_LAUNCH(float, float);
+    else if (act_dtype == IA_BF16 && src_dtype == IA_BF16) ROPE_ROWS_LAUNCH(bf16_t, bf16_t);
+    else if (act_dtype == IA_BF16 && src_dtype == IA_F32) ROPE_ROWS_LAUNCH(float, bf16_t);
+    else return IA_ERR_BAD_ARG;
+#undef ROPE_ROWS_LAUNCH
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
 #define ROPE_LAUNCH(TS, T)                                                                                         \
   rope_kv_append_kernel<TS, T><<<grid, 256, 0, stream>>>((const TS*)src, splits, stride, (T*)q_out, q_stride,      \
                                                          positions, slots, inv_freq, (T*)k_pages, (T*)v_pages,     \

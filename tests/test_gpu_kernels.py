@@ -157,6 +157,42 @@ def test_rope_kv_append(dtype, nh, nkv, d, rot, ps):
     assert torch.allclose(q2.double().reshape(N, nh, d), roted[:, :nh], atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,rot,ps", [(6, 2, 48, 48, 5), (32, 8, 128, 128, 16), (5, 1, 128, 64, 7), (3, 3, 20, 8, 4)])
+def test_rope_of_many_tokens_equals_rope_of_few(dtype, nh, nkv, d, rot, ps):
+    """A portion of a prompt takes another kernel (one workgroup per token) than a few decoded tokens (one wave
+    per token and head): the same tokens in one call of 70 and in calls of 10 leave the same bits."""
+    N, pages = 70, 20
+    qkv = _rand(N, (nh + 2 * nkv) * d, dtype=dtype, seed=11)
+    pos = (torch.arange(N, dtype=torch.int32) * 37 % 2000).to(DEV)
+    inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV)
+    slots = torch.randperm(pages * ps)[:N].to(torch.int32).to(DEV)
+    many, few = qkv.clone(), qkv.clone()
+    kp1, vp1 = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV), torch.zeros(pages, nkv, d, ps, dtype=dtype, device=DEV)
+    kp2, vp2 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    K().rope_kv_append(many, pos, inv, nh, nkv, d, rot, slots, kp1, vp1)
+    for n0 in range(0, N, 10):
+        part = few[n0:n0 + 10]
+        K().rope_kv_append(part, pos[n0:n0 + 10].contiguous(), inv, nh, nkv, d, rot, slots[n0:n0 + 10].contiguous(), kp2, vp2)
+    assert torch.equal(many, few) and torch.equal(kp1, kp2) and torch.equal(vp1, vp2)
+    # and both are the rotation: against fp64 at a few places
+    x = qkv.double().reshape(N, nh + 2 * nkv, d)
+    ang = (pos.float()[:, None] * inv[None, :]).double()
+    c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[:, :nh, :rot // 2], x[:, :nh, rot // 2:rot]
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    got = many[:, :nh * d].double().reshape(N, nh, d)
+    assert torch.allclose(got[..., :rot // 2], a * c - b * s_, atol=tol, rtol=tol)
+    assert torch.allclose(got[..., rot // 2:rot], a * s_ + b * c, atol=tol, rtol=tol)
+    assert torch.equal(got[..., rot:], x[:, :nh, rot:])
+    # a separate output for the queries (the source stays as it is)
+    src = qkv.clone()
+    q_out = torch.full((N, nh * d), float("nan"), dtype=dtype, device=DEV)
+    kp3, vp3 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    K().rope_kv_append(src, pos, inv, nh, nkv, d, rot, slots, kp3, vp3, q_out=q_out)
+    assert torch.equal(q_out, many[:, :nh * d]) and torch.equal(src, qkv) and torch.equal(kp3, kp1)
+
+
 # -------------------------------------------------------------- matrix products
 @pytest.mark.parametrize("M,N,K_", [(1, 250, 96), (7, 384, 176), (70, 129, 1000), (300, 64, 33)])
 def test_gemm_generic(M, N, K_):
