@@ -30,7 +30,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef const __attribute__((address_space(1))) void* gm_global_ptr;
 typedef __attribute__((address_space(3))) void* gm_lds_ptr;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X,
                                                                            const uint16_t* __restrict__ W,
                                                                            uint16_t* __restrict__ C, int M, int N,
@@ -139,9 +139,13 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
                   *reinterpret_cast<const bf16x8*>(xa + (r - TN) * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
           }
         }
+        // the loads of the later stage, spread over the first FILL_STEPS matrix-core steps
+        if (s < FILL_STEPS) {
+          constexpr int SLOTS = FILL_STEPS * MF;
 #pragma unroll
-        for (int f = (g * FPW) / MF; f < ((g + 1) * FPW) / MF; ++f)
-          if (s == 0) GM_FILL(f, kt_fill, fill_buf);   // all of them early
+          for (int f = ((s * MF + g) * FPW) / SLOTS; f < ((s * MF + g + 1) * FPW) / SLOTS; ++f)
+            GM_FILL(f, kt_fill, fill_buf);
+        }
         acc[g / TM][g % TM] =
             __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][g / TM], xf[s & 1][g % TM], acc[g / TM][g % TM], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -180,21 +184,21 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS>
 static int launch_gemm_mfma(const uint16_t* x, const uint16_t* w, uint16_t* c, int M, int N, int K,
                             hipStream_t stream) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds_bytes = (size_t)STAGES * (BM + BN) * GM_ROW_BYTES;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
-  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES><<<tiles_m * tiles_n, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
+  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS><<<tiles_m * tiles_n, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
       x, w, c, M, N, K, tiles_m, tiles_n);
   IA_LAUNCH_CHECK();
   return IA_OK;
@@ -217,8 +221,10 @@ extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     const long long t128 = (long long)((M + 127) / 128) * ((N + 255) / 256);
     tile = t256 >= 512 ? 1 : (t128 >= 128 ? 2 : 3);
   }
-  if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2>(x, w, c, M, N, K, stream);
-  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3>(x, w, c, M, N, K, stream);
-  if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4>(x, w, c, M, N, K, stream);
+  // the later stage's loads go out during the first two quarters of a step for the large tile (measured
+  // best: later ones are waited for at the step's end), during the first for the others
+  if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2, 2>(x, w, c, M, N, K, stream);
+  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3, 1>(x, w, c, M, N, K, stream);
+  if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4, 1>(x, w, c, M, N, K, stream);
   return IA_ERR_BAD_ARG;
 }
