@@ -47,8 +47,9 @@ class CacheGroup:
 class StateSlotPool:
     """Indices of per-request state records of fixed size (alone, or the slots of a cache manager)."""
 
-    def __init__(self, num_slots: int, _view: Optional[ctypes.c_void_p] = None):
+    def __init__(self, num_slots: int, _view: Optional[ctypes.c_void_p] = None, _owner: object = None):
         self._lib = native.lib()
+        self._owner = _owner                 # the cache manager whose slots these are, kept alive
         self.num_slots = int(num_slots)
         if _view is not None:
             self._h, self._owned = _view, False
@@ -128,8 +129,8 @@ class CacheManager:
         if not self._h:
             raise ValueError("the cache could not be created: page_size, num_pages must be positive, slots not negative")
         for g in self.groups:
-            g.allocator = PageAllocator(0, _view=self._lib.ia_cache_group_pool(self._h, g.index))
-        self.slots = StateSlotPool(config.num_state_slots, _view=self._h)
+            g.allocator = PageAllocator(0, _view=self._lib.ia_cache_group_pool(self._h, g.index), _owner=self)
+        self.slots = StateSlotPool(config.num_state_slots, _view=self._h, _owner=self)
         self._ids: Dict[Hashable, int] = {}          # request -> its number in the native bookkeeping
         self._names: Dict[int, Hashable] = {}
         self._next_id = 0

@@ -24,10 +24,12 @@ class PageError(RuntimeError):
 
 
 class PageAllocator:
-    """A pool of ``num_pages`` pages; ``_view`` wraps a pool that a cache manager owns."""
+    """A pool of ``num_pages`` pages; ``_view`` wraps a pool that a cache manager (``_owner``, kept alive by
+    this object) owns."""
 
-    def __init__(self, num_pages: int, _view: Optional[int] = None):
+    def __init__(self, num_pages: int, _view: Optional[int] = None, _owner: object = None):
         self._lib = native.lib()
+        self._owner = _owner
         if _view is not None:
             self._h, self._owned = ctypes.c_void_p(_view), False
         else:
