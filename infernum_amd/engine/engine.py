@@ -126,8 +126,8 @@ class Engine:
         for r in reqs:
             if not cache.has(r):
                 cache.admit(r)
-        ok = cache.reserve_step(reqs, q_lens)
-        assert ok
+        if not cache.reserve_step(reqs, q_lens):
+            raise OutOfPages("the pages this step was checked for are gone")   # step_fits said they were there
         if all(len(e.tokens) == 1 for e in entries):
             logits = self._decode_step(entries)
         else:
