@@ -270,6 +270,19 @@ class CacheManager:
         del self._names[rid]
         self._poison()
 
+    def forget(self, req: Hashable) -> None:
+        """The native side has released the request already (while scheduling): drop its name here."""
+        rid = self._ids.pop(req, None)
+        if rid is not None:
+            del self._names[rid]
+            if self._lib.ia_cache_has(self._h, rid):
+                raise PageError(f"request {req!r} is forgotten but still holds pages")
+
+    def poison_freed(self) -> None:
+        """After native calls that released requests themselves: what they gave back is filled with NaN
+        (when ``poison_freed_pages`` is set)."""
+        self._poison()
+
     def _poison(self) -> None:
         """Fill the pages that the last commit or release gave back with NaN (when asked to)."""
         if not self.config.poison_freed_pages or self.device is None:

@@ -589,6 +589,177 @@ int ia_cache_pack_step(void* h, int n, const int64_t* reqs, const int* q_lens, c
   return 0;
 }
 
+// ------------------------------------------------------------------------------------- scheduling
+// The decisions of one scheduling step over the cache's counts (infernum-runtime/src/scheduler.rs:289-352 is
+// the reference's step: decode every running request, admit first come first served without skipping).
+// In this order: one token for every decoding request; the next portion of every running prompt; then
+// admissions from the head of the queue while it fits (its first portion and one spare page per running
+// request), all under one budget of tokens.  When a decoding request cannot get its page, or no request can
+// move at all, the request admitted last is set back: it gives back what it holds (released here) and
+// returns to the front of the queue; a request that is alone and still does not fit fails.
+//
+// Running requests come in the order of admission: rid (their number in the cache, -1 when they hold
+// nothing yet), phase (1 = prompt, 2 = decoding) and tokens (prompt and generated).  The queue comes head
+// first.  Actions are records of four ints (kind, index, a, b):
+//   1 decode   index = running request
+//   2 portion  index = running request, a = tokens already stored, b = tokens of the portion
+//   3 set back index = running request (everything it held is released)
+//   4 fail     index = running request (released), or queue position when a == 3;
+//              a: 1 = too large while decoding, 2 = too large for its prompt, 3 = no free page with nothing running
+//   5 admit    index = queue position, b = tokens of the first portion
+// Portions and decodes of a request that is set back later in the step are taken out again.
+// Returns the number of actions, or IA_HOST_ERROR.
+int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run_phase, const int64_t* run_tokens,
+                  int n_waiting, const int64_t* wait_tokens, int max_batch, int max_prefill, int max_step_tokens,
+                  int* actions, int cap) {
+  Cache* c = static_cast<Cache*>(h);
+  const size_t G = c->groups.size();
+  struct Act { int kind, index, a, b; };
+  std::vector<Act> acts;
+  std::vector<int> live;                       // running requests still running, in the order of admission
+  for (int i = 0; i < n_running; ++i) live.push_back(i);
+  std::vector<int64_t> rid(run_rid, run_rid + n_running);
+  std::vector<int64_t> promised(G, 0);
+  std::vector<int> need(G, 0), prom32(G, 0);
+  int64_t budget = max_step_tokens;
+  int new_slots = 0, admitted_now = 0;
+  bool any_set_back = false;
+
+  auto pages_needed = [&](int64_t r, int64_t n) {
+    ia_cache_pages_needed(h, r >= 0 ? 1 : 0, r >= 0 ? r : 0, n, need.data());
+  };
+  auto fits = [&](int64_t spare) {
+    for (size_t g = 0; g < G; ++g)
+      if (need[g] + spare + promised[g] > c->groups[g].pool.num_free()) return false;
+    return true;
+  };
+  auto take = [&]() {
+    for (size_t g = 0; g < G; ++g) promised[g] += need[g];
+  };
+  auto tokens_that_fit = [&](int64_t r) {
+    for (size_t g = 0; g < G; ++g) prom32[g] = (int)promised[g];
+    return ia_cache_tokens_that_fit(h, r >= 0 ? 1 : 0, r >= 0 ? r : 0, prom32.data());
+  };
+  auto planned = [&]() {
+    for (const Act& a : acts)
+      if (a.kind == 1 || a.kind == 2 || a.kind == 5) return true;
+    return false;
+  };
+  auto drop_from_live = [&](int s) { live.erase(std::find(live.begin(), live.end(), s)); };
+  std::vector<int> freed;                      // (group, page) pairs of everything released in this step
+  auto release = [&](int s) {
+    if (rid[(size_t)s] >= 0 && c->admitted(rid[(size_t)s])) {
+      ia_cache_release(h, rid[(size_t)s]);
+      freed.insert(freed.end(), c->last_freed.begin(), c->last_freed.end());
+    }
+    rid[(size_t)s] = -1;
+  };
+  auto set_back = [&](int victim) {
+    drop_from_live(victim);
+    release(victim);
+    acts.erase(std::remove_if(acts.begin(), acts.end(),
+                              [&](const Act& a) { return (a.kind == 1 || a.kind == 2) && a.index == victim; }),
+               acts.end());
+    acts.push_back({3, victim, 0, 0});
+    any_set_back = true;
+  };
+
+  // one token for every decoding request
+  for (size_t i = 0; i < live.size();) {
+    const int s = live[i];
+    if (run_phase[s] != 2) { ++i; continue; }
+    if (rid[(size_t)s] < 0) return c->fail("a decoding request holds nothing in the cache");
+    pages_needed(rid[(size_t)s], 1);
+    if (fits(0)) {
+      take();
+      --budget;
+      acts.push_back({1, s, 0, 0});
+      ++i;
+      continue;
+    }
+    const int victim = live.back();
+    if (victim == s && live.size() == 1) {
+      acts.push_back({4, s, 1, 0});
+      drop_from_live(s);
+      release(s);
+      continue;
+    }
+    set_back(victim);     // the victim stood at or after i: position i now holds the next request (or none)
+  }
+
+  // next portions of running prompts
+  bool blocked = false;
+  for (size_t i = 0; i < live.size();) {
+    const int s = live[i];
+    if (run_phase[s] != 1) { ++i; continue; }
+    if (budget <= 0) break;
+    const int64_t r = (rid[(size_t)s] >= 0 && c->admitted(rid[(size_t)s])) ? rid[(size_t)s] : -1;
+    const int64_t cached = r >= 0 ? c->tokens[r] : 0;
+    int64_t n = std::min<int64_t>(std::min<int64_t>(run_tokens[s] - cached, max_prefill), budget);
+    n = std::min<int64_t>(n, tokens_that_fit(r));
+    if (n <= 0) {
+      if (!planned()) {
+        const int victim = live.back();           // nobody can move: the last admitted request makes room
+        if (victim == s && live.size() == 1) {
+          acts.push_back({4, s, 2, 0});
+          drop_from_live(s);
+          release(s);
+          continue;
+        }
+        set_back(victim);
+        continue;
+      }
+      blocked = true;
+      break;
+    }
+    if (r < 0) ++new_slots;
+    pages_needed(r, n);
+    take();
+    budget -= n;
+    acts.push_back({2, s, (int)cached, (int)n});
+    ++i;
+  }
+
+  // admissions, first come first served, while the head of the queue fits
+  int w = 0;
+  while (w < n_waiting && !blocked && !any_set_back && budget > 0 &&
+         (int)live.size() + admitted_now < max_batch && (int)c->free_slots.size() - new_slots > 0) {
+    const int64_t running_now = (int64_t)live.size() + admitted_now;
+    int64_t n = std::min<int64_t>(std::min<int64_t>(wait_tokens[w], max_prefill), budget);
+    pages_needed(-1, n);
+    // one page in hand for every running request, so that a newcomer is not set back at once
+    if (!fits(running_now)) {
+      if (running_now == 0 && !planned()) {
+        // alone and still too large for one portion: shrink the portion to the pool
+        n = std::min<int64_t>(n, tokens_that_fit(-1));
+        if (n <= 0) {
+          acts.push_back({4, w, 3, 0});
+          ++w;
+          continue;
+        }
+        pages_needed(-1, n);
+      } else {
+        break;
+      }
+    }
+    acts.push_back({5, w, 0, (int)n});
+    ++admitted_now;
+    ++new_slots;
+    take();
+    budget -= n;
+    ++w;
+  }
+  c->last_freed.swap(freed);                   // ia_cache_last_freed: all pages given back while deciding
+  if ((int)acts.size() > cap) return c->fail("the action buffer is too small");
+  for (size_t i = 0; i < acts.size(); ++i) {
+    actions[4 * i] = acts[i].kind;
+    actions[4 * i + 1] = acts[i].index;
+    actions[4 * i + 2] = acts[i].a;
+    actions[4 * i + 3] = acts[i].b;
+  }
+  return (int)acts.size();
+}
+
 // the buffer of the last packed step (valid until the next ia_cache_pack_step on this cache)
 const int32_t* ia_cache_packed(void* h) { return static_cast<Cache*>(h)->packed.data(); }
 

@@ -27,17 +27,22 @@ and ignores a failed allocation while decoding, engine.rs:476-480.)
 
 The scheduler only decides; it keeps no tensors and calls no kernels.  It reads
 the cache manager's counts, and gives back what finished or set-back requests
-hold.
+hold.  The decisions of a step are taken natively (``ia_sched_step`` in
+csrc/host_core.cpp, beside the cache's bookkeeping); this module keeps the
+requests themselves, their tokens, phases and events, and applies the decisions.
 """
 from __future__ import annotations
 
+import ctypes
 import enum
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Hashable, List, Optional, Sequence
 
-from ..cache import CacheManager
+from ..cache import CacheManager, native
 from ..sampling.params import GenerateOptions
+
+_ACT_DECODE, _ACT_PORTION, _ACT_SET_BACK, _ACT_FAIL, _ACT_ADMIT = 1, 2, 3, 4, 5     # kinds of ia_sched_step's actions
 
 
 class FinishReason(enum.Enum):
@@ -186,110 +191,61 @@ class Scheduler:
 
     # ---- one step -----------------------------------------------------------------
     def step(self, cache: CacheManager) -> SchedulerOutput:
+        """The decisions themselves are taken natively (``ia_sched_step`` in csrc/host_core.cpp) over the
+        cache's counts; here they are applied to the requests."""
         cfg = self.config
         out = SchedulerOutput()
-        # 1. finished requests give back what they hold (scheduler.rs:289-305)
+        # finished requests give back what they hold (scheduler.rs:289-305)
         out.finished.extend(self.reap(cache))
-
-        budget = cfg.max_tokens_per_step
-        promised = [0] * len(cache.groups)        # pages this step's earlier entries will take
-        new_slots = 0
-
-        def fits(need: List[int]) -> bool:
-            return all(n + p <= g.allocator.num_free for n, p, g in zip(need, promised, cache.groups))
-
-        def take(need: List[int]) -> None:
-            for i, n in enumerate(need):
-                promised[i] += n
-
-        # 2. one token for every decoding request
-        i = 0
-        while i < len(self.running):
-            seq = self.running[i]
-            if seq.phase != SequencePhase.DECODE:
-                i += 1
-                continue
-            need = cache.pages_needed(seq.id, 1)
-            if fits(need):
-                take(need)
-                budget -= 1
-                out.decode.append(DecodeTask(seq))
-                i += 1
-                continue
-            victim = self.running[-1]
-            if victim is seq and len(self.running) == 1:
-                self._fail(seq, f"the page pool is too small for a request of {seq.num_tokens + 1} tokens")
+        running, waiting = list(self.running), list(self.waiting)
+        if not running and not waiting:
+            return out
+        nr, nw = len(running), len(waiting)
+        rid = (ctypes.c_int64 * max(nr, 1))(*[cache.request_id(s.id) if cache.has(s.id) else -1 for s in running])
+        phase = (ctypes.c_int * max(nr, 1))(*[2 if s.phase == SequencePhase.DECODE else 1 for s in running])
+        tokens = (ctypes.c_int64 * max(nr, 1))(*[s.num_tokens for s in running])
+        wait_tokens = (ctypes.c_int64 * max(nw, 1))(*[s.num_tokens for s in waiting])
+        cap = 3 * nr + 2 * nw + 4
+        actions = (ctypes.c_int * (4 * cap))()
+        n = native.lib().ia_sched_step(cache.native_handle(), nr, rid, phase, tokens, nw, wait_tokens,
+                                       cfg.max_batch_size, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
+                                       actions, cap)
+        if n < 0:
+            cache._fail()
+        cache.poison_freed()
+        for i in range(n):
+            kind, index, a, b = actions[4 * i:4 * i + 4]
+            if kind == _ACT_DECODE:
+                out.decode.append(DecodeTask(running[index]))
+            elif kind == _ACT_PORTION:
+                seq = running[index]
+                out.prefill.append(PrefillTask(seq, seq.all_tokens()[a:a + b], a + b == seq.num_tokens))
+            elif kind == _ACT_SET_BACK:
+                seq = running[index]
                 self.running.remove(seq)
-                cache.release(seq.id)
+                cache.forget(seq.id)                       # released natively while deciding
+                seq.phase = SequencePhase.WAITING
+                seq.times_set_back += 1
+                self.waiting.appendleft(seq)
+                out.set_back.append(seq)
+            elif kind == _ACT_FAIL and a == 3:
+                seq = self._pop_waiting(waiting[index])
+                self._fail(seq, "the page pool has no free page although nothing is running")
                 out.finished.append(seq)
-                continue
-            self._set_back(victim, cache, out)
-            # the victim stood at or after i: position i now holds the next request (or none)
-
-        # 3. next portions of running prompts, in the order of admission
-        blocked = False
-        i = 0
-        while i < len(self.running):
-            seq = self.running[i]
-            if seq.phase != SequencePhase.PREFILL:
-                i += 1
-                continue
-            if budget <= 0:
-                break
-            cached = cache.num_tokens(seq.id) if cache.has(seq.id) else 0
-            n = min(seq.num_tokens - cached, cfg.max_prefill_tokens, budget)
-            n = min(n, cache.tokens_that_fit(seq.id, promised) if cache.has(seq.id)
-                    else cache.tokens_that_fit(None, promised))
-            if n <= 0:
-                if out.is_empty():
-                    # nobody can move: the last admitted request makes room
-                    victim = self.running[-1]
-                    if victim is seq and len(self.running) == 1:
-                        self._fail(seq, f"the page pool is too small for a request of {seq.num_tokens} tokens")
-                        self.running.remove(seq)
-                        if cache.has(seq.id):
-                            cache.release(seq.id)
-                        out.finished.append(seq)
-                        continue
-                    self._set_back(victim, cache, out)
-                    continue
-                blocked = True
-                break
-            if not cache.has(seq.id):
-                new_slots += 1
-            take(cache.pages_needed(seq.id, n))
-            budget -= n
-            tokens = seq.all_tokens()[cached:cached + n]
-            out.prefill.append(PrefillTask(seq, tokens, cached + n == seq.num_tokens))
-            i += 1
-
-        # 4. admissions, first come first served, while the head of the queue fits
-        while (self.waiting and not blocked and not out.set_back and budget > 0
-               and len(self.running) < cfg.max_batch_size and cache.slots.num_free - new_slots > 0):
-            seq = self.waiting[0]
-            n = min(seq.num_tokens, cfg.max_prefill_tokens, budget)
-            need = cache.pages_needed(seq.id, n)
-            # keep one page in hand for every running request, so that a newcomer is not set back at once
-            spare = [len(self.running)] * len(need) if self.running else [0] * len(need)
-            if not fits([a + b for a, b in zip(need, spare)]):
-                if not self.running and out.is_empty():
-                    # alone and still too large for one portion: shrink the portion to the pool
-                    n = min(n, cache.tokens_that_fit(None, promised))
-                    if n <= 0:
-                        self.waiting.popleft()
-                        self._fail(seq, "the page pool has no free page although nothing is running")
-                        out.finished.append(seq)
-                        continue
-                    need = cache.pages_needed(seq.id, n)
-                else:
-                    break
-            self.waiting.popleft()
-            seq.phase = SequencePhase.PREFILL
-            self.running.append(seq)
-            new_slots += 1
-            take(need)
-            budget -= n
-            out.prefill.append(PrefillTask(seq, seq.all_tokens()[:n], n == seq.num_tokens))
+            elif kind == _ACT_FAIL:
+                seq = running[index]
+                size = seq.num_tokens + 1 if a == 1 else seq.num_tokens
+                self._fail(seq, f"the page pool is too small for a request of {size} tokens")
+                self.running.remove(seq)
+                cache.forget(seq.id)
+                out.finished.append(seq)
+            elif kind == _ACT_ADMIT:
+                seq = self._pop_waiting(waiting[index])
+                seq.phase = SequencePhase.PREFILL
+                self.running.append(seq)
+                out.prefill.append(PrefillTask(seq, seq.all_tokens()[:b], b == seq.num_tokens))
+            else:
+                raise RuntimeError(f"unknown scheduling action {kind}")
         return out
 
     # ---- after the model has run ------------------------------------------------------
@@ -334,6 +290,12 @@ class Scheduler:
         seq.finish_reason = FinishReason.CANCELLED
 
     # ---- helpers ------------------------------------------------------------------------
+    def _pop_waiting(self, expected: SequenceState) -> SequenceState:
+        seq = self.waiting.popleft()
+        if seq is not expected:
+            raise RuntimeError("the queue changed while a step was decided")
+        return seq
+
     def _finish(self, seq: SequenceState, reason: FinishReason) -> None:
         seq.phase = SequencePhase.FINISHED
         seq.finish_reason = reason
@@ -343,15 +305,3 @@ class Scheduler:
         seq.phase = SequencePhase.FINISHED
         seq.error = message
         seq.send(GenerationEvent("error", error=message))
-
-    def _set_back(self, victim: SequenceState, cache: CacheManager, out: SchedulerOutput) -> None:
-        self.running.remove(victim)
-        if cache.has(victim.id):
-            cache.release(victim.id)
-        # drop what this step had planned for it
-        out.decode = [t for t in out.decode if t.seq is not victim]
-        out.prefill = [t for t in out.prefill if t.seq is not victim]
-        victim.phase = SequencePhase.WAITING
-        victim.times_set_back += 1
-        self.waiting.appendleft(victim)
-        out.set_back.append(victim)
