@@ -153,7 +153,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
     }
     // the next step's loads must have landed; the ones issued since may still be on their way
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * FPW) : "memory");
-    __syncthreads();
+    // A bare barrier: __syncthreads() brings a fence with it that waits for every load in flight, the ones
+    // of the stages after the next included, which is the very wait that more than two stages are there to
+    // avoid.  The wait above covers what the next step reads (LDS writes of these loads are counted by
+    // vmcnt); this wave's own LDS reads have been waited for by the matrix instructions that used them.
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     buf = (buf + 1 == STAGES) ? 0 : buf + 1;
     fill_buf = (fill_buf + 1 == STAGES) ? 0 : fill_buf + 1;
   }
