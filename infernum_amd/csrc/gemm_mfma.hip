@@ -109,37 +109,49 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
 #pragma unroll
   for (int s = 0; s < KS; ++s) swz[s] = ((2 * s + lh) ^ (li & 7)) * 16;
 
+  // The operands of a step's first matrix instructions are read during the last quarter of the step before,
+  // and the barrier stands before that quarter, so that no wave waits at a step's start:
+  //   quarters 0 .. KS-2: reads of the next quarter's operands; the loads of step kt + STAGES - 1 (into the
+  //                       stage that step kt - 1 has left: the barrier of step kt - 1 lies behind);
+  //   end of quarter KS-2: wait for the loads of step kt + 1 (the ones issued since may stay in flight) and
+  //                       for this wave's own LDS reads, then a bare barrier (__syncthreads() would bring a
+  //                       fence that waits for every load in flight): stage kt + 1 is complete for all waves,
+  //                       and every wave has the last operands of stage kt in registers;
+  //   quarter KS-1:       reads of the first operands of step kt + 1.
+  static_assert(FILL_STEPS <= KS - 1, "a step's loads must be out before its barrier");
+  bf16x8 wf[2][TN], xf[2][TM];
+#pragma unroll
+  for (int a = 0; a < TN; ++a) wf[0][a] = *reinterpret_cast<const bf16x8*>(lds + wrow + a * 32 * GM_ROW_BYTES + swz[0]);
+#pragma unroll
+  for (int b = 0; b < TM; ++b) xf[0][b] = *reinterpret_cast<const bf16x8*>(lds + xrow + b * 32 * GM_ROW_BYTES + swz[0]);
   int buf = 0, fill_buf = STAGES - 1;
   for (int kt = 0; kt < ksteps; ++kt) {
+    const int next_buf = (buf + 1 == STAGES) ? 0 : buf + 1;
     const char* xa = lds + buf * STAGE_BYTES + xrow;
     const char* wb = lds + buf * STAGE_BYTES + wrow;
+    const char* xa_next = lds + next_buf * STAGE_BYTES + xrow;
+    const char* wb_next = lds + next_buf * STAGE_BYTES + wrow;
     // past the end the last step is fetched again, into a stage that is not read any more
     const int kt_fill = min(kt + STAGES - 1, ksteps - 1);
-    bf16x8 wf[2][TN], xf[2][TM];
-#pragma unroll
-    for (int a = 0; a < TN; ++a) wf[0][a] = *reinterpret_cast<const bf16x8*>(wb + a * 32 * GM_ROW_BYTES + swz[0]);
-#pragma unroll
-    for (int b = 0; b < TM; ++b) xf[0][b] = *reinterpret_cast<const bf16x8*>(xa + b * 32 * GM_ROW_BYTES + swz[0]);
     __builtin_amdgcn_sched_barrier(0);
-    // The order below is kept as written (nothing moves across a sched_barrier): the reads of the next
-    // operands and the loads of the next step go between the matrix instructions of this one, so that
-    // none of them is waited for with the matrix cores idle.
+    // The order below is kept as written (nothing moves across a sched_barrier): LDS reads and loads go
+    // between the matrix instructions, so that none of them is waited for with the matrix cores idle.
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       constexpr int MF = TN * TM, RD = TN + TM;
+      const char* wsrc = (s + 1 < KS) ? wb : wb_next;
+      const char* xsrc = (s + 1 < KS) ? xa : xa_next;
 #pragma unroll
       for (int g = 0; g < MF; ++g) {
-        if (s + 1 < KS) {
 #pragma unroll
-          for (int r = (g * RD) / MF; r < ((g + 1) * RD) / MF; ++r) {
-            if (r < TN)
-              wf[(s + 1) & 1][r] = *reinterpret_cast<const bf16x8*>(wb + r * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
-            else
-              xf[(s + 1) & 1][r - TN] =
-                  *reinterpret_cast<const bf16x8*>(xa + (r - TN) * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
-          }
+        for (int r = (g * RD) / MF; r < ((g + 1) * RD) / MF; ++r) {
+          if (r < TN)
+            wf[(s + 1) & 1][r] = *reinterpret_cast<const bf16x8*>(wsrc + r * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
+          else
+            xf[(s + 1) & 1][r - TN] =
+                *reinterpret_cast<const bf16x8*>(xsrc + (r - TN) * 32 * GM_ROW_BYTES + swz[(s + 1) % KS]);
         }
-        // the loads of the later stage, spread over the first FILL_STEPS matrix-core steps
+        // the loads of the later stage, spread over the first FILL_STEPS quarters
         if (s < FILL_STEPS) {
           constexpr int SLOTS = FILL_STEPS * MF;
 #pragma unroll
@@ -150,16 +162,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
             __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][g / TM], xf[s & 1][g % TM], acc[g / TM][g % TM], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if (s == KS - 2) {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * FPW) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    // the next step's loads must have landed; the ones issued since may still be on their way
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * FPW) : "memory");
-    // A bare barrier: __syncthreads() brings a fence with it that waits for every load in flight, the ones
-    // of the stages after the next included, which is the very wait that more than two stages are there to
-    // avoid.  The wait above covers what the next step reads (LDS writes of these loads are counted by
-    // vmcnt); this wave's own LDS reads have been waited for by the matrix instructions that used them.
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    buf = (buf + 1 == STAGES) ? 0 : buf + 1;
+    buf = next_buf;
     fill_buf = (fill_buf + 1 == STAGES) ? 0 : fill_buf + 1;
   }
 
@@ -221,15 +231,16 @@ extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
   const uint16_t* w = (const uint16_t*)W;
   uint16_t* c = (uint16_t*)C;
   if (tile == 0) {
-    // the largest tile that still gives every compute unit about two workgroups
+    // the large tile when it gives at least three quarters of a round of workgroups (it runs fastest per
+    // workgroup), else the middle one while that fills half the compute units, else the small one
     const long long t256 = (long long)((M + 255) / 256) * ((N + 255) / 256);
     const long long t128 = (long long)((M + 127) / 128) * ((N + 255) / 256);
-    tile = t256 >= 512 ? 1 : (t128 >= 128 ? 2 : 3);
+    tile = t256 >= 192 ? 1 : (t128 >= 128 ? 2 : 3);
   }
-  // the later stage's loads go out during the first two quarters of a step for the large tile (measured
-  // best: later ones are waited for at the step's end), during the first for the others
+  // the later stage's loads go out during the first two quarters of a step where the tile is large
+  // (measured best), during the first for the small tile
   if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2, 2>(x, w, c, M, N, K, stream);
-  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3, 1>(x, w, c, M, N, K, stream);
+  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3, 2>(x, w, c, M, N, K, stream);
   if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4, 1>(x, w, c, M, N, K, stream);
   return IA_ERR_BAD_ARG;
 }
