@@ -305,9 +305,6 @@ class CacheManager:
     def free_pages(self, group: int = 0) -> int:
         return self.groups[group].allocator.num_free
 
-    def min_free_pages(self) -> int:
-        return min((g.allocator.num_free for g in self.groups), default=1 << 30)
-
     def block_table(self, group: int, req: Hashable) -> BlockTable:
         """A copy of the request's block table in the group."""
         rid = self._id(req)
@@ -318,24 +315,6 @@ class CacheManager:
         pages = (ctypes.c_int * max(n, 1))()
         self._lib.ia_cache_table(self._h, int(group), rid, pages, n, None, None)
         return BlockTable(list(pages[:n]), tokens.value, first.value)
-
-    def num_pages_held(self, group: int, req: Hashable) -> int:
-        """Length of the request's block table in the group (pages given back by a window count)."""
-        n = int(self._lib.ia_cache_table(self._h, int(group), self._id(req), None, 0, None, None))
-        if n == native.HOST_ERROR:
-            self._fail()
-        return n
-
-    def block_table_rows(self, group: int, reqs: Sequence[Hashable], width: Optional[int] = None) -> np.ndarray:
-        """int32 [len(reqs), width], NO_PAGE where a request holds no page."""
-        tables = [self.block_table(group, r).pages for r in reqs]
-        if width is None:
-            width = max((len(t) for t in tables), default=1)
-        width = max(width, 1)
-        out = np.full((len(reqs), width), NO_PAGE, dtype=np.int32)
-        for i, p in enumerate(tables):
-            out[i, :len(p)] = p
-        return out
 
     def token_slots(self, group: int, req: Hashable, start: int, n: int) -> np.ndarray:
         """page * page_size + offset of positions start .. start+n-1 (pages must be reserved)."""
