@@ -89,6 +89,28 @@ def test_add_rmsnorm_joins_partial_sums(H, S):
     assert torch.equal(out2, out[rows.long()])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H", [2048, 3000, 4096, 5120, 1000])
+def test_add_rmsnorm_of_many_rows_equals_that_of_few(dtype, H):
+    """Many rows take a kernel with fewer threads per row than a few rows do: the same rows in one call of
+    300 and in calls of 20 leave the same bits (the sums of squares are taken in one order)."""
+    N, eps = 300, 1e-5
+    h = _rand(N, H, seed=4)
+    delta = _rand(N, H, dtype=dtype, seed=5)
+    w = (_rand(H, seed=6).abs() + 0.5).to(dtype)
+    h_many, h_few = h.clone(), h.clone()
+    out_many = torch.empty(N, H, dtype=dtype, device=DEV)
+    out_few = torch.empty(N, H, dtype=dtype, device=DEV)
+    K().add_rmsnorm(h_many, delta, w, eps, out_many)
+    for n0 in range(0, N, 20):
+        K().add_rmsnorm(h_few[n0:n0 + 20], delta[n0:n0 + 20], w, eps, out_few[n0:n0 + 20])
+    assert torch.equal(h_many, h_few) and torch.equal(out_many, out_few)
+    s = h.double() + delta.double()
+    want = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert torch.allclose(out_many.double(), want, atol=tol, rtol=tol)
+
+
 def test_rmsnorm_reference_vector():
     # infernum-cuda/src/inner/cuda/ops/rmsnorm.rs:171-203
     h = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)
