@@ -13,7 +13,21 @@ __global__ __launch_bounds__(SNT) void argmax_kernel(const float* __restrict__ l
   const float* x = logits + (size_t)blockIdx.x * ld;
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += SNT) {
+  // 16-byte loads where the row allows it (four at a time in flight), single values for the rest
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  const int V4 = vec ? (V >> 2) : 0;
+#pragma unroll 4
+  for (int i4 = threadIdx.x; i4 < V4; i4 += SNT) {
+    const float4 q = *reinterpret_cast<const float4*>(x + 4 * i4);
+    const float qs[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v = qs[e];
+      const int i = 4 * i4 + e;
+      if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    }
+  }
+  for (int i = 4 * V4 + threadIdx.x; i < V; i += SNT) {
     const float v = x[i];
     if (v > best || (v == best && i < idx)) { best = v; idx = i; }
   }
