@@ -353,11 +353,14 @@ def _attn(d: int) -> ctypes.CDLL:
 
 
 def decode_splits(batch: int, nh: int, nkv: int, max_len: int) -> int:
-    """Parts the keys of a request are cut into, so that a small batch still fills the GPU: about 512
-    workgroups (of four waves, each wave one tile of 16 keys at a time), at least 4 tiles a workgroup."""
+    """Parts the keys of a request are cut into, so that a small batch still fills the GPU (workgroups of
+    four waves, each wave one tile of 16 keys at a time): about 256 workgroups while the batch alone gives at
+    most 64, about 512 above that, and at least 8 tiles a workgroup (measured: more and shorter parts cost
+    more in the join than they gain)."""
     groups = batch * nkv * ((nh // nkv + 15) // 16)
     tiles = max(1, (max_len + 15) // 16)
-    return max(1, min((512 + groups - 1) // groups, (tiles + 3) // 4, 64))
+    wanted = 256 // groups if groups <= 64 else (512 + groups - 1) // groups
+    return max(1, min(wanted, tiles // 8, 64))
 
 
 def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
