@@ -68,3 +68,36 @@ def test_first_tokens(models, name, dtype):
     # a token's logits at position 0 are those of a sequence of that token alone
     alone = P.forward(cfg, w, toks[:1])[0]
     assert (one[0].double().cpu() - alone).abs().max().item() <= TOL[dtype] * rms
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_many_requests_decoded_together(models, name, dtype):
+    """150 requests in one decode step: more rows than the decode GEMM kernel takes (64), so the products go
+    the way of many rows while attention and the rest stay on the decode kernels."""
+    import random
+    from infernum_amd import CacheConfig, Engine
+    from infernum_amd.engine import StepEntry
+    d, cfg, w = models[(name, dtype)]
+    rng = random.Random(1)
+    n = 150
+    reqs = {f"r{i}": [rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(3, 20))] for i in range(n)}
+    ref = {r: P.forward(cfg, w, t) for r, t in reqs.items()}
+    eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=8, num_pages=n * 4,
+                                                                          num_state_slots=n + 2))
+    names = list(reqs)
+    fed = {r: max(1, len(reqs[r]) - 4) for r in names}
+    for i in range(0, n, 30):
+        eng.step([StepEntry(r, reqs[r][:fed[r]], []) for r in names[i:i + 30]])
+    worst = 0.0
+    while any(fed[r] < len(reqs[r]) for r in names):
+        live = [r for r in names if fed[r] < len(reqs[r])]
+        logits = eng.step([StepEntry(r, [reqs[r][fed[r]]], [0]) for r in live]).double().cpu()
+        for k, r in enumerate(live):
+            want = ref[r][fed[r]].double()
+            worst = max(worst, float((logits[k] - want).abs().max() / want.pow(2).mean().sqrt()))
+            fed[r] += 1
+    assert worst <= TOL[dtype], f"worst |diff| / rms {worst:.2e}"
+    for r in names:
+        eng.end(r)
+    assert eng.cache.free_pages() == n * 4
