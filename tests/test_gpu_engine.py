@@ -71,6 +71,26 @@ def test_whole(models, name, dtype):
     assert eng.cache.free_pages(0) == 64
 
 
+def test_whole_with_the_hand_written_prefill_gemm(models):
+    """Configuration B (width 128) with the many-row products on the hand-written LDS-tiled MFMA kernel where it
+    takes the size (K in steps of 64: QKV, output projection, gate and up; the down projection's K of 352
+    stays with the library): prompts of 97 and 64 tokens bring more than 64 rows."""
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    d, cfg, reqs, ref = models[("B", "bfloat16")]
+    previous = L.set_prefill_gemm("mfma")
+    try:
+        eng = _engine(d, "bfloat16", PAGE["B"], 64)
+        got = TT.run_steps(eng, TT.trace_whole(reqs))
+    finally:
+        L.set_prefill_gemm(previous)
+    _check(got, ref, "bfloat16", "B bfloat16 whole, own prefill GEMM")
+    # and the same logits as with the library's product: both accumulate in fp32 and round once
+    lib = TT.run_steps(_engine(d, "bfloat16", PAGE["B"], 64), TT.trace_whole(reqs))
+    worst, rms, where = TT.error_against(got, {r: torch.stack([lib[(r, i)] for i in range(len(t))]) for r, t in reqs.items()})
+    assert worst <= 2e-2 * rms, f"own and library products differ by {worst:.3e} at {where}"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_tail_one_by_one(models, name, dtype):
