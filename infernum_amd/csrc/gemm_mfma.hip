@@ -173,7 +173,44 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
     fill_buf = (fill_buf + 1 == STAGES) ? 0 : fill_buf + 1;
   }
 
-  // ---- C
+  // ---- C.  A whole tile with rows of N that 16-byte stores can take goes through LDS, so that a row of the
+  // wave's part leaves as consecutive 16-byte pieces (the accumulators hold 4 values of a row per lane, 32
+  // rows apart from lane to lane).  Every wave has a region of its own, WM rows of WN values; the 16-byte
+  // piece c of row m lies at position c ^ (m % CP): the lanes of a store instruction write 32 different rows.
+  constexpr int CP = WN / 8;                        // 16-byte pieces per row of a wave's part
+  static_assert(STAGES * STAGE_BYTES >= WAVES * WM * WN * 2, "the stages must hold the tile of C");
+  if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the loads asked for past the end write LDS too
+    __syncthreads();
+    char* region = lds + wave * (WM * WN * 2);
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+      for (int b = 0; b < TM; ++b) {
+        const int m = b * 32 + li;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = a * 32 + 8 * g + 4 * lh;                      // 4 values from here on
+          uint2 v;
+          v.x = (uint32_t)float_to_bf16_bits(acc[a][b][4 * g]) | ((uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 1]) << 16);
+          v.y = (uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 2]) | ((uint32_t)float_to_bf16_bits(acc[a][b][4 * g + 3]) << 16);
+          const int piece = (n >> 3) ^ (m & (CP - 1));
+          *reinterpret_cast<uint2*>(region + (m * CP + piece) * 16 + (n & 4) * 2) = v;
+        }
+      }
+    // a wave reads back what it wrote itself: no barrier, only the wait for its LDS writes
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    constexpr int RPI = 64 / CP;                      // rows per store instruction of the wave
+    uint16_t* cbase = C + (size_t)(m0 + wm * WM) * N + n0 + wn * WN;
+#pragma unroll 4
+    for (int r0 = 0; r0 < WM; r0 += RPI) {
+      const int m = r0 + lane / CP, c = lane % CP;
+      const uint4 v = *reinterpret_cast<const uint4*>(region + (m * CP + (c ^ (m & (CP - 1)))) * 16);
+      *reinterpret_cast<uint4*>(cbase + (size_t)m * N + c * 8) = v;
+    }
+    return;
+  }
+  // a tile at the edge of C, or rows that are no multiple of 16 bytes: straight from the accumulators
   const bool vec_ok = (N & 3) == 0;
 #pragma unroll
   for (int a = 0; a < TN; ++a)
