@@ -47,6 +47,8 @@ HEADERS = ["common.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
 HOST_SOURCES = ["host_core.cpp"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
+# The binding of the vendor's GEMM library (hipBLASLt): host code too, against ROCm's headers and libraries.
+BLASLT_SOURCES = ["gemm_library.cpp"]
 
 # Head sizes whose attention library `build_all` compiles ahead of time.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)
@@ -66,6 +68,19 @@ def find_hipcc() -> Optional[str]:
         if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
             return cand
     return None
+
+
+def rocm_root() -> str:
+    """Where ROCm's include/ and lib/ are: $ROCM_PATH, beside hipcc, or /opt/rocm."""
+    cands = [os.environ.get("ROCM_PATH")]
+    hipcc = find_hipcc()
+    if hipcc:
+        cands.append(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))))
+    cands.append("/opt/rocm")
+    for c in cands:
+        if c and os.path.isfile(os.path.join(c, "include", "hipblaslt", "hipblaslt.h")):
+            return c
+    return "/opt/rocm"
 
 
 def find_cxx() -> Optional[str]:
@@ -114,9 +129,15 @@ def _fingerprint(sources: Sequence[str], defines: Sequence[str], host: bool = Fa
 
 
 def library_plan(name: str) -> Dict:
-    """Sources and defines of a library by its name ('core', 'attn_d<D>' or 'host')."""
+    """Sources and defines of a library by its name ('core', 'attn_d<D>', 'host' or 'blaslt')."""
     if name == "host":
         return {"sources": _existing(HOST_SOURCES), "defines": [], "host": True}
+    if name == "blaslt":
+        root = rocm_root()
+        return {"sources": _existing(BLASLT_SOURCES), "host": True,
+                "defines": ["-D__HIP_PLATFORM_AMD__", f"-I{os.path.join(root, 'include')}"],
+                "link": [f"-L{os.path.join(root, 'lib')}", "-lhipblaslt", "-lamdhip64",
+                         f"-Wl,-rpath,{os.path.join(root, 'lib')}"]}
     if name == "core":
         return {"sources": _existing(CORE_SOURCES), "defines": []}
     if name.startswith("attn_d"):
@@ -153,13 +174,15 @@ def _compile_host_library(name: str, plan: Dict) -> str:
     t0 = time.time()
     try:
         tmp_out = os.path.join(tmp_dir, "lib.so")
-        cmd = [cxx] + CXX_FLAGS + ["-shared", "-o", tmp_out] + [os.path.join(CSRC_DIR, f) for f in plan["sources"]]
+        cmd = [cxx] + CXX_FLAGS + list(plan["defines"]) + ["-shared", "-o", tmp_out] + \
+            [os.path.join(CSRC_DIR, f) for f in plan["sources"]] + list(plan.get("link", []))
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, cwd=tmp_dir)
         if r.returncode != 0:
             raise BuildError(f"{os.path.basename(cxx)} failed on {', '.join(plan['sources'])}:\n{r.stderr[-6000:]}")
         os.replace(tmp_out, out)
         with open(_stamp_path(name), "w") as f:
-            json.dump({"fingerprint": _fingerprint(plan["sources"], plan["defines"], host=True)}, f)
+            json.dump({"fingerprint": _fingerprint(plan["sources"], list(plan["defines"]) + list(plan.get("link", [])),
+                                                   host=True)}, f)
     finally:
         shutil.rmtree(tmp_dir, ignore_errors=True)
     _say(f"built {os.path.basename(out)} in {time.time() - t0:.1f} s")
@@ -215,8 +238,8 @@ def ensure(name: str) -> str:
     if os.path.isfile(out):
         try:
             with open(_stamp_path(name)) as f:
-                if json.load(f).get("fingerprint") == _fingerprint(plan["sources"], plan["defines"],
-                                                                   host=bool(plan.get("host"))):
+                if json.load(f).get("fingerprint") == _fingerprint(
+                        plan["sources"], list(plan["defines"]) + list(plan.get("link", [])), host=bool(plan.get("host"))):
                     return out
         except (OSError, ValueError):
             pass
@@ -228,7 +251,7 @@ def ensure(name: str) -> str:
 
 def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> List[str]:
     """Compile every library (the core one, and attention for the given head sizes)."""
-    names = ["host", "core"]
+    names = ["host", "blaslt", "core"]
     if os.path.isfile(os.path.join(CSRC_DIR, "attention_mfma.hip")):
         names += [f"attn_d{d}" for d in head_dims]
     workers = max(1, min(4, int(os.environ.get("MAX_JOBS", "8"))))

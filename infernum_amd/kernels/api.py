@@ -20,10 +20,15 @@ class KernelError(RuntimeError):
     pass
 
 
+class KernelUnsupported(KernelError):
+    """The kernel (or the library) does not take this size; nothing was launched."""
+
+
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 _libs: Dict[str, ctypes.CDLL] = {}
 
-_ERRORS = {10001: "bad argument", 10002: "size not supported by this kernel"}
+_ERRORS = {10001: "bad argument", 10002: "size not supported by this kernel",
+           10003: "a call into the GEMM library failed"}
 
 
 def load_library(name: str) -> ctypes.CDLL:
@@ -77,7 +82,7 @@ class on_current_stream:
 def _ok(code: int, what: str) -> None:
     if code != 0:
         why = _ERRORS.get(code, f"HIP error {code}")
-        raise KernelError(f"{what}: {why}")
+        raise (KernelUnsupported if code == 10002 else KernelError)(f"{what}: {why}")
 
 
 def _need(cond: bool, msg: str) -> None:
@@ -263,6 +268,37 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     _need(out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N),
           f"gemm_mfma: out must be contiguous bf16 [{M}, {N}]")
     _ok(_core().ia_gemm_mfma(_p(a), _p(w), _p(out), M, N, K, MFMA_GEMM_TILES[tile], _stream()), "gemm_mfma")
+    return out
+
+
+LIBRARY_WORKSPACE_BYTES = 128 << 20
+_library_workspace: Dict[torch.device, torch.Tensor] = {}
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T by the vendor's library (hipBLASLt), called directly: bf16 with fp32
+    accumulation, or fp32 throughout.  The library's choice of an algorithm is asked once per shape and kept,
+    so a later product of the same shape costs one call on the host.  All products share one workspace per
+    device: they must be on one stream, or ordered otherwise."""
+    _dev(a, w, out)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_library: shapes")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == w.dtype and a.dtype in DTYPE_CODE, "gemm_library: bf16 or fp32 operands of one dtype")
+    _need(M >= 1 and N >= 1 and K >= 1, "gemm_library: empty operand")
+    if out is None:
+        out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    _need(out.dtype == a.dtype and tuple(out.shape) == (M, N), f"gemm_library: out must be {a.dtype} [{M}, {N}]")
+    ws = _library_workspace.get(a.device)
+    if ws is None:
+        ws = _library_workspace[a.device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+    lib = load_library("blaslt")
+    code = lib.ia_gemm_lt(_p(a), _p(w), _p(out), M, N, K, DTYPE_CODE[a.dtype], _p(ws), ctypes.c_size_t(ws.numel()),
+                          _stream())
+    if code == 10003:
+        raise KernelError(f"gemm_library: hipBLASLt failed with status {lib.ia_gemm_lt_last_status()} "
+                          f"(M={M} N={N} K={K} {a.dtype})")
+    _ok(code, f"gemm_library (M={M} N={N} K={K})")
     return out
 
 

@@ -7,12 +7,14 @@ and calls cuBLAS (infernum-cuda/src/inner/cuda/ops/matmul.rs:68-117).
 
 fp32: the hand-written fp32 kernel, always (no reduced-precision matrix mode).
 bf16: up to 64 rows the hand-written MFMA kernel that streams the weight once;
-above that the library product (hipBLASLt through torch), as the reference uses
-its library there; an fp32 result of many rows comes 64 rows at a time from the
-hand-written kernel.  ``set_prefill_gemm("mfma")`` (or INFERNUM_PREFILL_GEMM=mfma
-in the environment) sends the many-row bf16 products to the hand-written
-LDS-tiled MFMA kernel instead, where it takes the size (K in steps of 64); it is
-correct at every size but slower than the library so far, hence not the default.
+above that the library product (hipBLASLt, called directly with its choice of
+an algorithm kept per shape), as the reference uses its library there; an fp32
+result of many rows comes 64 rows at a time from the hand-written kernel.
+``set_prefill_gemm("mfma")`` (or INFERNUM_PREFILL_GEMM=mfma in the environment)
+sends the many-row bf16 products to the hand-written LDS-tiled MFMA kernel
+instead, where it takes the size (K in steps of 64); it is correct at every size
+but slower than the library so far, hence not the default.  ``"torch"`` sends
+them to the same library through ``torch.mm``, which costs more on the host.
 
 ``epilogue="swiglu"`` returns silu(y[:, :N/2]) * y[:, N/2:]; the decode kernel
 does it while it joins its partial sums, the other paths in a kernel of its own.
@@ -30,7 +32,7 @@ from ..kernels import api as K
 from ..kernels.api import SplitSum
 
 
-PREFILL_GEMMS = ("library", "mfma")
+PREFILL_GEMMS = ("library", "mfma", "torch")
 _prefill_gemm = os.environ.get("INFERNUM_PREFILL_GEMM", "library")
 if _prefill_gemm not in PREFILL_GEMMS:
     raise ValueError(f"INFERNUM_PREFILL_GEMM={_prefill_gemm!r}: one of {PREFILL_GEMMS}")
@@ -66,8 +68,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     elif out_dtype == torch.bfloat16:
         if _prefill_gemm == "mfma" and x.is_contiguous() and K.gemm_mfma_supported(M, N, Kdim):
             y = K.gemm_mfma(x, w)
-        else:
+        elif _prefill_gemm == "torch" or not x.is_contiguous():
             y = torch.mm(x, w.t())                  # library product, fp32 accumulation
+        else:
+            try:
+                y = K.gemm_library(x, w)
+            except K.KernelUnsupported:             # the library has no algorithm for this shape
+                y = K.gemm_mfma(x, w) if K.gemm_mfma_supported(M, N, Kdim) else \
+                    K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
     elif K.gemm_skinny_supported(1, N, Kdim) and x.is_contiguous():
         # fp32 result from bf16 operands, many rows: 64 rows at a time through the skinny kernel
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)

@@ -356,6 +356,54 @@ def test_linear_with_the_hand_written_prefill_gemm():
     assert tuple(odd.shape) == (200, 330)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K_", [(65, 100, 72), (67, 31, 9), (300, 1003, 192), (1, 7, 128), (640, 384, 320)])
+def test_gemm_library(dtype, M, N, K_):
+    """The vendor library's product, called directly: sizes that fill no tile and that are no multiple of
+    anything; the second call of a shape takes the kept plan and gives the same bits."""
+    api = K()
+    a, w = _rand(M, K_, dtype=dtype, seed=8), _rand(N, K_, dtype=dtype, scale=0.1, seed=9)
+    want = a.double() @ w.double().t()
+    out = torch.full((M, N), float("nan"), dtype=dtype, device=DEV)
+    api.gemm_library(a, w, out)
+    if dtype == torch.bfloat16:
+        bound = 2e-5 * math.sqrt(K_) * 0.1 + 2.0 ** -8 * want.abs()
+    else:
+        # fp32 throughout: the worst case of K roundings of 2^-24 each on the sum of the products' magnitudes,
+        # far below what a reduced-precision matrix mode (2^-11 per product) would leave
+        bound = K_ * 2.0 ** -24 * (a.abs().double() @ w.abs().double().t())
+    assert bool(((out.double() - want).abs() <= bound).all())
+    plans = api.load_library("blaslt").ia_gemm_lt_plans()
+    assert torch.equal(api.gemm_library(a, w), out)
+    assert api.load_library("blaslt").ia_gemm_lt_plans() == plans
+
+
+def test_gemm_library_refuses_what_it_cannot_do():
+    api = K()
+    with pytest.raises(api.KernelError):
+        api.gemm_library(_rand(80, 96, dtype=torch.bfloat16), _rand(32, 96))                       # two dtypes
+    with pytest.raises(api.KernelError):
+        api.gemm_library(_rand(80, 96), _rand(32, 64))                                             # inner sizes
+    with pytest.raises(api.KernelError):
+        api.gemm_library(_rand(80, 128)[:, :64], _rand(32, 64))                                    # not contiguous
+
+
+def test_linear_by_the_library_directly_and_through_torch():
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    x, w = _rand(200, 256, dtype=torch.bfloat16, seed=3), _rand(330, 256, dtype=torch.bfloat16, scale=0.1, seed=4)
+    assert L.prefill_gemm() == "library"
+    direct = L.linear(x, w)
+    previous = L.set_prefill_gemm("torch")
+    try:
+        through = L.linear(x, w)
+    finally:
+        L.set_prefill_gemm(previous)
+    want = x.double() @ w.double().t()
+    bound = 2e-5 * 16 * 0.1 + 2.0 ** -8 * want.abs()
+    assert bool(((direct.double() - want).abs() <= bound).all()) and bool(((through.double() - want).abs() <= bound).all())
+
+
 def test_rope_from_partial_sums():
     """The rotary kernel joins a split product itself: same pages and queries as from the joined tensor."""
     api = K()
