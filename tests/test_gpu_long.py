@@ -101,3 +101,35 @@ def test_many_requests_decoded_together(models, name, dtype):
     for r in names:
         eng.end(r)
     assert eng.cache.free_pages() == n * 4
+
+
+def test_recorded_decode_step_of_many_requests_equals_the_eager_one():
+    """100 requests a step at layer sizes where the library's large GEMM kernels run: the step is recorded
+    with the library's launches inside and replayed six times, with other work of the program between the
+    replays; every replay gives the bits of the same step run launch by launch."""
+    from infernum_amd import CacheConfig, Engine
+    from infernum_amd.config import LlamaConfig
+    from infernum_amd.engine import StepEntry
+    cfg = LlamaConfig.from_dict({"model_type": "llama", "vocab_size": 32000, "hidden_size": 2048,
+                                 "intermediate_size": 8192, "num_hidden_layers": 2, "num_attention_heads": 16,
+                                 "num_key_value_heads": 4, "rope_theta": 500000.0, "max_position_embeddings": 4096,
+                                 "rms_norm_eps": 1e-5})
+    B, steps = 100, 8
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine.from_config(cfg, seed=3, dtype="bfloat16", use_graphs=graphs,
+                                 cache_config=CacheConfig(page_size=16, num_pages=B * 8 + 8, num_state_slots=B + 1))
+        g = torch.Generator().manual_seed(0)
+        prompts = [torch.randint(0, cfg.vocab_size, (40 + (i % 7),), generator=g).tolist() for i in range(B)]
+        for i in range(0, B, 25):
+            eng.step([StepEntry(j, prompts[j], []) for j in range(i, min(B, i + 25))])
+        toks, res = [1 + j for j in range(B)], []
+        for _ in range(steps):
+            logits = eng.step([StepEntry(j, [toks[j]], [0]) for j in range(B)])
+            assert bool(torch.isfinite((logits * 2).sum()))           # eager work and a synchronisation between replays
+            res.append(logits.cpu())
+            toks = logits.argmax(-1).tolist()
+        outs[graphs] = res
+        assert eng.graph_replays == (steps - 1 if graphs else 0)
+    for s in range(steps):
+        assert torch.equal(outs[False][s], outs[True][s]), f"step {s}"
