@@ -2,9 +2,11 @@
 // multiply-add only: the matrix product of the true 32-bit path, and the plain
 // twin that the MFMA kernels are checked against.
 //
-// Every output element is one chain of fused multiply-adds over k = 0 .. K-1 in
-// this order, whatever M, N and the tile it falls into: results do not depend on
-// how many rows a step brings.
+// Every output element is summed in one fixed order, whatever M, N and the tile
+// it falls into: results do not depend on how many rows a step brings.  The order
+// is in three levels, so that rounding grows with the square root of K / 256 and
+// not of K: a chain of 16 fused multiply-adds from zero (one LDS stage), 16 such
+// chains added up (256 values of k), and those sums added in the order of k.
 #include "common.h"
 
 #define GT 64   // tile of C: GT x GT
@@ -21,11 +23,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
   const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
   const int lr = tid >> 2;          // row of the tile this thread loads: 0..63
   const int lk = (tid & 3) * 4;     // first of its 4 consecutive k
-  float acc[4][4];
+  float acc[4][4], mid[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = mid[i][j] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += GK) {
     {
@@ -38,6 +40,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
       }
     }
     __syncthreads();
+    float part[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
       float a[4], b[4];
@@ -48,8 +55,19 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+    const bool close = ((k0 / GK) & 15) == 15 || k0 + GK >= K;      // 256 values of k are in, or the last stage
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mid[i][j] += part[i][j];
+        if (close) {
+          acc[i][j] += mid[i][j];
+          mid[i][j] = 0.f;
+        }
+      }
     __syncthreads();
   }
 #pragma unroll
