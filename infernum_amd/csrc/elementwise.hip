@@ -101,11 +101,16 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
 // registers (16-byte loads, all issued before the first use), so the row is read once and no load waits for
 // another.  Sums are taken in the same order whatever the batch: a row's result depends on the row alone.
 #define RN_MAXV 4
+// x^2 + y^2 + z^2 + w^2 with its roundings written out (two products, two fused multiply-adds, one addition), so
+// that every instantiation of the kernel below gives the same bits for the same row.
+__device__ __forceinline__ float sum_of_squares4(const float4 v) {
+  return __builtin_fmaf(v.x, v.x, v.y * v.y) + __builtin_fmaf(v.z, v.z, v.w * v.w);
+}
 // AS_WIDE (NT = 256, H <= 4096): the sum of squares is taken in the very order of the kernel of 1024 threads
 // (piece c of this thread is the piece of thread threadIdx.x + 256 c there: 16 sums over 64 lanes, added in the
 // order of their index), so that a row's result has the same bits from either; with many rows 256 threads
 // per row keep more rows on a compute unit and are a sixth faster.
-template <typename TD, typename TO, int NT, bool AS_WIDE = false>
+template <typename TD, typename TO, int NT, bool AS_WIDE = false, int MAXV = RN_MAXV>
 __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                              int splits, size_t split_stride,
                                                              const void* __restrict__ w, int w_dtype,
@@ -117,20 +122,21 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
   float* hr = h + (size_t)src * H;
   const TD* dr = delta ? delta + (size_t)src * H : nullptr;
   const bool store = (rows == nullptr) && (delta != nullptr);
-  float4 v[RN_MAXV];
+  float4 v[MAXV];
 #pragma unroll
-  for (int c = 0; c < RN_MAXV; ++c) {
+  for (int c = 0; c < MAXV; ++c) {
     const int i = (threadIdx.x + c * NT) * 4;
     v[c] = (i < H) ? load4(hr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
   if (dr) {
-    float4 ds[RN_MAXV];
+    float4 ds[MAXV];
+    constexpr int UNROLL_PARTS = MAXV == 1 ? 8 : 4;
 #pragma unroll
-    for (int c = 0; c < RN_MAXV; ++c) ds[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 4
+    for (int c = 0; c < MAXV; ++c) ds[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma clang loop unroll_count(UNROLL_PARTS)
     for (int k = 0; k < splits; ++k) {           // unrolled: the loads of several parts are in flight together
 #pragma unroll
-      for (int c = 0; c < RN_MAXV; ++c) {
+      for (int c = 0; c < MAXV; ++c) {
         const int i = (threadIdx.x + c * NT) * 4;
         if (i < H) {
           const float4 d = load4(dr + k * split_stride + i);
@@ -139,38 +145,38 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
       }
     }
 #pragma unroll
-    for (int c = 0; c < RN_MAXV; ++c) { v[c].x += ds[c].x; v[c].y += ds[c].y; v[c].z += ds[c].z; v[c].w += ds[c].w; }
+    for (int c = 0; c < MAXV; ++c) { v[c].x += ds[c].x; v[c].y += ds[c].y; v[c].z += ds[c].z; v[c].w += ds[c].w; }
   }
   float ss = 0.f;
   if (AS_WIDE) {
-    static_assert(!AS_WIDE || (NT == 256 && RN_MAXV == 4), "256 threads stand for 1024");
+    static_assert(!AS_WIDE || (NT == 256 && MAXV == 4), "256 threads stand for 1024");
     __shared__ float red_wide[16];
-    float part[RN_MAXV];
+    float part[MAXV];
 #pragma unroll
-    for (int c = 0; c < RN_MAXV; ++c) {
+    for (int c = 0; c < MAXV; ++c) {
       const int i = (threadIdx.x + c * NT) * 4;
       part[c] = 0.f;
       if (i < H) {
         if (store) store4(hr + i, v[c]);
-        part[c] += (v[c].x * v[c].x + v[c].y * v[c].y) + (v[c].z * v[c].z + v[c].w * v[c].w);
+        part[c] += sum_of_squares4(v[c]);
       }
       part[c] = wave_sum(part[c]);
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (lane == 0) {
 #pragma unroll
-      for (int c = 0; c < RN_MAXV; ++c) red_wide[wave + 4 * c] = part[c];
+      for (int c = 0; c < MAXV; ++c) red_wide[wave + 4 * c] = part[c];
     }
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < 16; ++k) ss += red_wide[k];
   } else {
 #pragma unroll
-    for (int c = 0; c < RN_MAXV; ++c) {
+    for (int c = 0; c < MAXV; ++c) {
       const int i = (threadIdx.x + c * NT) * 4;
       if (i < H) {
         if (store) store4(hr + i, v[c]);
-        ss += (v[c].x * v[c].x + v[c].y * v[c].y) + (v[c].z * v[c].z + v[c].w * v[c].w);
+        ss += sum_of_squares4(v[c]);
       }
     }
     ss = block_sum<NT>(ss, red);
@@ -178,7 +184,7 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
   TO* o = out + (size_t)row * H;
 #pragma unroll
-  for (int c = 0; c < RN_MAXV; ++c) {
+  for (int c = 0; c < MAXV; ++c) {
     const int i = (threadIdx.x + c * NT) * 4;
     if (i < H) {
       const float4 g = load4_any(w, w_dtype, i);
@@ -198,6 +204,11 @@ static int launch_add_rmsnorm(float* h, const void* delta, int splits, size_t sp
     if (H >= 2048 && H <= 4096 && N >= 1024)   // measured: from about 1,000 rows on the narrow workgroups win
       add_rmsnorm_vec_kernel<TD, TO, 256, true><<<N, 256, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o,
                                                                         rows, H, eps);
+    else if (H >= 2048 && H <= 4096)
+      // one piece a thread: few registers, so the loads of up to eight partial sums are in flight together
+      // (the sums are the same: the pieces beyond the first are empty at this width)
+      add_rmsnorm_vec_kernel<TD, TO, 1024, false, 1><<<N, 1024, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o,
+                                                                              rows, H, eps);
     else if (H >= 2048)
       add_rmsnorm_vec_kernel<TD, TO, 1024><<<N, 1024, 0, stream>>>(h, d, splits, split_stride, w, w_dtype, o, rows,
                                                                     H, eps);
