@@ -1,7 +1,7 @@
-// bf16 attention over the paged cache on the matrix cores (v_mfma_f32_16x16x16_bf16),
-// compiled for one head size, IA_HEAD_DIM (a multiple of 16, at most 256).
+// bf16 attention over the paged cache on the matrix cores (v_mfma_f32_16x16x16_bf16 and
+// v_mfma_f32_16x16x32_bf16), compiled for one head size, IA_HEAD_DIM (a multiple of 16, at most 256).
 //
-// Both kernels work on the transposed problem, one wave per workgroup and no LDS:
+// Both kernels work on the transposed problem:
 //   S^T[key, col] = K[key, :] . Q[col, :]      A operand = 16 keys of K, B operand = 16 columns of Q
 //   O^T[dim, col] += V^T[dim, key] P^T[key, col]
 // A column is one (token, query head).  The accumulator of S^T leaves lane l with
@@ -16,9 +16,9 @@
 // token, so a page is read once for its whole group of heads; the keys of a
 // request are split over blockIdx.z, each part leaves (max, sum, unnormalised
 // output) and a second kernel joins the parts in a fixed order.
-// Prefill: a wave takes CT column tiles that share their keys: GH heads of one
-// key/value head times CT/GH blocks of 16 consecutive tokens; K and V^T registers
-// are loaded once per 16 keys and used for all CT tiles.
+// Prefill: a wave takes 16 consecutive tokens of one query head; the waves of a
+// workgroup (64 tokens of up to four query heads of one key/value head) share the
+// tiles of keys and values, which go through LDS.
 //
 // Key pages are [num_pages, nkv, page_size, d]; page_size must be a multiple of 4.
 // Keys outside [first key any column may see, last key of the request] are
@@ -32,7 +32,6 @@
 #define HD IA_HEAD_DIM
 #define NS (HD / 16)
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
-#define PREFILL_CT (HD <= 128 ? 4 : 2)
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -327,11 +326,13 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 }
 
 // ----------------------------------------------------------------------- prefill
-// grid (num_tiles, nkv * ceil(G / CT)), 256 threads.
+// grid (num_tiles, nkv * ceil(G / (CT * HGW))), HGW * 256 threads.
 // tiles[i] = (request, first row of a block of 64 rows among the request's new tokens).
-// A workgroup takes 64 rows x CT query heads of one key/value head: wave w takes rows 16 w .. 16 w + 15 for
-// all CT heads.  Keys and values go through LDS in tiles of 32 keys, loaded once per workgroup and read by
-// its four waves; the loads of the next tile are in flight while the matrix cores work on this one.
+// A workgroup takes 64 rows x CT * HGW query heads of one key/value head: it has HGW groups of four waves,
+// wave w of a group takes rows 16 w .. 16 w + 15 for the group's CT heads (CT = 1 in every launch: see
+// ia_attn_prefill).  Keys and values go through LDS in tiles of 64 keys (32 above a head size of 128), loaded
+// once per workgroup and read by all its waves; the loads of the next tile are in flight while the matrix
+// cores work on this one.
 //   S^T[key, col] = K[key, :] . Q[col, :]       v_mfma_f32_16x16x32_bf16 over 32 head dims a step
 //   O^T[dim, col] += V^T[dim, key] P^T[key, col] one v_mfma_f32_16x16x32_bf16 over the 32 keys of a tile
 // The accumulators of the two S^T tiles of 16 keys leave lane (col, qd) with the keys 4 qd .. 4 qd + 3 and
@@ -343,7 +344,6 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 #define PF_QPT (PF_KT / 4)             // quads of 4 keys per round
 #define PF_KROW (HD + 8)        // bf16 per key row in LDS: 16 bytes of padding spread the banks
 #define PF_VROW 40              // bf16 per dim row of V^T in LDS (32 keys + 8 of padding)
-#define PF_CT_MAX (HD <= 128 ? 4 : 2)
 #define PF_LAZY 6.0f            // log2 of how far the running maximum may run ahead of the reference point
 
 template <int CT, int HGW>
@@ -664,23 +664,32 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
   return IA_OK;
 }
 
+// heads_per_workgroup: 0 lets this function choose; 1, 2 or 4 (4 up to a head size of 160) asks for that many
+// groups of four waves, one query head each, that share the tiles of keys and values a workgroup brings in.
 extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
                                int out_row_stride, const int* seq_starts, const int* seq_ctx, const int* block_tables,
                                int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
-                               float scale, int window, hipStream_t stream) {
+                               float scale, int window, int heads_per_workgroup, hipStream_t stream) {
   if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
       bt_stride <= 0 || !(scale > 0.f))
     return IA_ERR_BAD_ARG;
   if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
   if (num_tiles == 0) return IA_OK;
   const int G = nh / nkv;
-  // A wave takes 16 rows of CT query heads of one key/value head; two heads keep its accumulators within 256
-  // vector registers, so that two waves share a SIMD and one's softmax overlaps the other's products.  With
-  // four or more heads to a key/value head a workgroup has a second set of four waves for the next CT heads:
-  // twice the rows of Q per tile of keys that is brought in.
-  int CT = G >= 2 ? 2 : 1;
-  int HGW = G >= 2 * CT ? 2 : 1;
-  const int HC = (G + CT * HGW - 1) / (CT * HGW);
+  // A wave takes 16 rows of one query head (more heads a wave need more registers than leave room for a second
+  // wave on the SIMD, or spill at large head sizes: measured 3 to 4 % slower at head size 128, 3 times slower
+  // at 256).  A workgroup has one, two or four groups of four waves, one head of the same key/value head each:
+  // that many times the rows of Q per tile of keys brought into LDS.  Four groups are 1024 threads, which
+  // leaves 128 registers a wave: enough up to a head size of 160.  At head sizes up to 64 two groups measure
+  // faster than four (the small tiles let several workgroups share a compute unit).
+  const int widest = (IA_HEAD_DIM >= 80 && IA_HEAD_DIM <= 160) ? 4 : 2;
+  int HGW = G >= 3 ? widest : (G == 2 ? 2 : 1);
+  if (heads_per_workgroup != 0) {
+    if (heads_per_workgroup != 1 && heads_per_workgroup != 2 && heads_per_workgroup != 4) return IA_ERR_BAD_ARG;
+    if (heads_per_workgroup == 4 && IA_HEAD_DIM > 160) return IA_ERR_UNSUPPORTED;
+    HGW = heads_per_workgroup;
+  }
+  const int HC = (G + HGW - 1) / HGW;
   if ((long long)nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(num_tiles, nkv * HC);
@@ -688,13 +697,11 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   attn_prefill_kernel<C, W><<<grid, 4 * W * 64, 0, stream>>>(                                                     \
       (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
       out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window)
-  if (CT == 1 && HGW == 1) PF_LAUNCH(1, 1);
-  else if (CT == 1) PF_LAUNCH(1, 2);
-  else if (CT == 2 && HGW == 1) PF_LAUNCH(2, 1);
-  else if (CT == 2) PF_LAUNCH(2, 2);
+  if (HGW == 1) PF_LAUNCH(1, 1);
+  else if (HGW == 2) PF_LAUNCH(1, 2);
   else {
-#if IA_HEAD_DIM <= 128
-    if (HGW == 1) PF_LAUNCH(4, 1); else PF_LAUNCH(4, 2);
+#if IA_HEAD_DIM <= 160
+    PF_LAUNCH(1, 4);
 #else
     return IA_ERR_UNSUPPORTED;
 #endif
