@@ -5,9 +5,12 @@ ties open, infernum-cuda/kernels/argmax.cu:14-86).  Sampled rows go through the
 repetition penalty, temperature, softmax, nucleus and inverse CDF of
 infernum-cuda/src/inner/cuda/ops/sample.rs:94-159, which the reference runs on the
 host over a downloaded row; here the row stays on the device and one int32 per row
-comes back.  Two stated differences: the nucleus takes every token that ties with
-the one that crosses ``top_p``, and the CDF walks the nucleus in the order of the
-vocabulary rather than by falling probability (no sort of the vocabulary).
+comes back.  Three stated differences: the nucleus takes every token that ties with
+the one that crosses ``top_p``; the CDF walks the nucleus in the order of the
+vocabulary rather than by falling probability (no sort of the vocabulary); and
+masses are added as integers, exp((x - max) / T) * 2^31 rounded down, so that sums
+do not depend on their order: a token whose probability is below 5e-10 of the
+likeliest one's is never drawn.
 """
 from __future__ import annotations
 

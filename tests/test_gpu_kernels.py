@@ -700,6 +700,32 @@ def test_sample_matches_host_rule(V):
     assert bad <= 1
 
 
+@pytest.mark.parametrize("V", [50000, 50001, 128256])
+def test_sample_of_a_row_alone_and_again(V):
+    """A row's token does not depend on the rows beside it nor on the run: masses are integers, their sums exact.
+    V = 50001 takes the path of single loads, the others that of 16-byte loads."""
+    R = 6
+    x = _rand(R, V, scale=3.0, seed=21)
+    g = torch.Generator().manual_seed(2)
+    T = (torch.rand(R, generator=g) + 0.3).to(DEV)
+    tp = torch.tensor([1.0, 0.95, 0.9, 0.5, 0.1, 0.999], device=DEV)
+    u = torch.rand(R, generator=g).to(DEV)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    K().sample(x, torch.empty(R, V, device=DEV), T, tp, u, out)
+    again = torch.empty_like(out)
+    K().sample(x, torch.empty(R, V, device=DEV), T, tp, u, again)
+    assert torch.equal(out, again)
+    for r in range(R):
+        one = torch.empty(1, dtype=torch.int32, device=DEV)
+        K().sample(x[r:r + 1].contiguous(), torch.empty(1, V, device=DEV), T[r:r + 1].contiguous(),
+                   tp[r:r + 1].contiguous(), u[r:r + 1].contiguous(), one)
+        assert int(one[0]) == int(out[r]), r
+    # against the rule worked out on the host in float64: only a draw within 1e-4 of a boundary of the running
+    # mass may differ (masses are cut off at 2^-31 of the largest one)
+    differ = sum(int(out[r]) != _host_sample(x[r], float(T[r]), float(tp[r]), float(u[r])) for r in range(R))
+    assert differ <= 1, differ
+
+
 def test_sample_limits_and_frequencies():
     V = 50
     x = _rand(1, V, scale=1.5, seed=3)
