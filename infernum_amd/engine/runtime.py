@@ -119,7 +119,13 @@ class Runtime:
         sp = s.options.sampling
         if sp is None:
             return RowRequest(None)
-        hist = s.all_tokens() if abs(sp.repetition_penalty - 1.0) > 1.1920929e-07 else ()
+        hist: Sequence[int] = ()
+        if abs(sp.repetition_penalty - 1.0) > 1.1920929e-07 and sp.repetition_penalty_window > 0:
+            # the last tokens of prompt and generation that the penalty looks at, not the whole sequence
+            n = sp.repetition_penalty_window
+            hist = s.generated_ids[-n:]
+            if len(hist) < n:
+                hist = s.prompt_ids[len(s.prompt_ids) - min(n - len(hist), len(s.prompt_ids)):] + hist
         return RowRequest(sp, len(s.generated_ids), hist)
 
     def run(self, until: Optional[Callable[[], bool]] = None) -> None:

@@ -17,6 +17,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import api as K
@@ -50,27 +51,38 @@ class Sampler:
             K.argmax(logits, out)
         if not sampled:
             return out.tolist()
-        # sampled rows are worked on in a copy: the penalty changes logits in place
-        idx = torch.tensor(sampled, dtype=torch.long, device=logits.device)
-        work_logits = logits.index_select(0, idx).contiguous()
         S = len(sampled)
         params = [rows[i].sampling for i in sampled]
-        if any(abs(p.repetition_penalty - 1.0) > 1.1920929e-07 for p in params):
-            W = max(1, max(min(p.repetition_penalty_window, len(rows[i].history)) for p, i in zip(params, sampled)))
-            recent = torch.zeros((S, W), dtype=torch.int32)
-            counts = torch.zeros(S, dtype=torch.int32)
-            for s, (p, i) in enumerate(zip(params, sampled)):
-                n = min(p.repetition_penalty_window, len(rows[i].history))
-                if n:
-                    recent[s, :n] = torch.tensor(list(rows[i].history[-n:]), dtype=torch.int32)
-                counts[s] = n
-            pen = torch.tensor([p.repetition_penalty for p in params], dtype=torch.float32)
-            K.repetition_penalty(work_logits, recent.to(logits.device), counts.to(logits.device),
-                                 pen.to(logits.device))
-        host = torch.tensor([[p.temperature for p in params], [p.top_p for p in params],
-                             [token_uniform(p.seed, rows[i].generated_before) for p, i in zip(params, sampled)]],
-                            dtype=torch.float32).to(logits.device)
-        picked = torch.empty(S, dtype=torch.int32, device=logits.device)
-        K.sample(work_logits, torch.empty_like(work_logits), host[0], host[1], host[2], picked)
-        out.index_copy_(0, idx, picked)
+        penalised = any(abs(p.repetition_penalty - 1.0) > 1.1920929e-07 for p in params)
+        # one block of host numbers for all rows, one copy: temperature, top_p, draw, penalty
+        nums = np.empty((4, S), dtype=np.float32)
+        for s, (p, i) in enumerate(zip(params, sampled)):
+            nums[0, s], nums[1, s] = p.temperature, p.top_p
+            nums[2, s] = token_uniform(p.seed, rows[i].generated_before)
+            nums[3, s] = p.repetition_penalty
+        dev_nums = torch.from_numpy(nums).to(logits.device)
+        if S == R and not penalised and logits.is_contiguous():
+            work_logits = logits                     # nothing changes the logits: no copy
+            idx = None
+        else:
+            # sampled rows are worked on in a copy: the penalty changes logits in place
+            idx = torch.tensor(sampled, dtype=torch.long, device=logits.device) if S < R else None
+            work_logits = (logits.index_select(0, idx) if idx is not None else logits.clone()).contiguous()
+        if penalised:
+            tails = []
+            for p, i in zip(params, sampled):
+                h = rows[i].history
+                n = min(p.repetition_penalty_window, len(h))
+                tails.append(list(h[len(h) - n:]) if n else [])
+            W = max(1, max(len(t) for t in tails))
+            ints = np.zeros(S * W + S, dtype=np.int32)           # the rows' tokens, then how many of each row count
+            for s, t in enumerate(tails):
+                ints[s * W:s * W + len(t)] = t
+                ints[S * W + s] = len(t)
+            dev_ints = torch.from_numpy(ints).to(logits.device)
+            K.repetition_penalty(work_logits, dev_ints[:S * W].view(S, W), dev_ints[S * W:], dev_nums[3])
+        picked = out if idx is None else torch.empty(S, dtype=torch.int32, device=logits.device)
+        K.sample(work_logits, torch.empty_like(work_logits), dev_nums[0], dev_nums[1], dev_nums[2], picked)
+        if idx is not None:
+            out.index_copy_(0, idx, picked)
         return out.tolist()
