@@ -55,6 +55,8 @@ std::mutex g_mu;
 hipblasLtHandle_t g_handle = nullptr;
 std::unordered_map<Key, Plan, KeyHash> g_plans;
 int g_last_status = 0;          // the library's last status that was not a success
+int g_in_flight = 0;            // calls between their lookup of a plan and the end of their hipblasLtMatmul
+constexpr size_t kMaxPlans = 4096;
 
 bool ok(hipblasStatus_t s) {
   if (s == HIPBLAS_STATUS_SUCCESS) return true;
@@ -125,18 +127,26 @@ extern "C" int ia_gemm_lt(const void* X, const void* W, void* C, int M, int N, i
     const Key key{M, N, K, dtype, workspace_bytes};
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
+      // portions of prompts come in any length: the table is emptied when it has grown large, so that it stays
+      // bounded; only while no call is between its lookup of a plan and the end of its hipblasLtMatmul
+      if (g_plans.size() >= kMaxPlans && g_in_flight == 0) {
+        for (auto& kv : g_plans) drop(kv.second);
+        g_plans.clear();
+      }
       Plan fresh;
       const int rc = make_plan(key, fresh);
       if (rc != IA_OK) return rc;
       it = g_plans.emplace(key, fresh).first;
     }
-    plan = it->second;      // descriptors are never destroyed while the process lives
+    plan = it->second;
+    ++g_in_flight;          // the plan's descriptors stay alive until this call has used them
   }
   const float alpha = 1.0f, beta = 0.0f;
   const hipblasStatus_t s = hipblasLtMatmul(g_handle, plan.desc, &alpha, W, plan.a, X, plan.b, &beta, C, plan.c, C,
                                             plan.c, &plan.algo, workspace, workspace_bytes, stream);
+  std::lock_guard<std::mutex> lock(g_mu);
+  --g_in_flight;
   if (s != HIPBLAS_STATUS_SUCCESS) {
-    std::lock_guard<std::mutex> lock(g_mu);
     g_last_status = (int)s;
     return IA_ERR_LIBRARY;
   }
