@@ -56,7 +56,6 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
                                                                     TO* __restrict__ C, float* __restrict__ part,
                                                                     int M, int N, int K, int chunks_per_split) {
   constexpr int XROW = SK_KC + SK_XPAD;
-  constexpr int TPW = 1;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][XROW];
   __shared__ f32x4 glu_up[GLU ? 2 : 1][GLU ? MT : 1][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -70,14 +69,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   const int NO = GLU ? N / 2 : N;                      // columns of the result
 
   const int n_row = (n_base + r < NO) ? n_base + r : NO - 1;
-  const uint16_t* wrow[TPW];
+  const uint16_t* wrow = W + ((size_t)n_row + (size_t)half * NO) * K;
+  f32x4 acc[MT];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t) wrow[t] = W + ((size_t)n_row + (size_t)half * NO) * K;
-  f32x4 acc[TPW][MT];
-#pragma unroll
-  for (int t = 0; t < TPW; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   // the chunk of X is MT*16 rows of 256 values = MT*512 pieces of 16 bytes, spread over the 256 threads
   constexpr int XPIECES = MT * 16 * (SK_KC / 8);
@@ -102,15 +97,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
       *reinterpret_cast<uint4*>(&xs[buf][row][kk]) = xreg[i];
     }
   };
-  uint4 wcur[TPW][SK_NLD], wnext[TPW][SK_NLD];
-  auto load_w = [&](int c, uint4 (&dst)[TPW][SK_NLD]) {
+  uint4 wcur[SK_NLD], wnext[SK_NLD];
+  auto load_w = [&](int c, uint4 (&dst)[SK_NLD]) {
 #pragma unroll
-    for (int t = 0; t < TPW; ++t)
-#pragma unroll
-      for (int i = 0; i < SK_NLD; ++i) {
-        const int k = c * SK_KC + (i * 4 + q) * 8;
-        dst[t][i] = (k < K) ? load_stream_16(wrow[t] + k) : make_uint4(0u, 0u, 0u, 0u);
-      }
+    for (int i = 0; i < SK_NLD; ++i) {
+      const int k = c * SK_KC + (i * 4 + q) * 8;
+      dst[i] = (k < K) ? load_stream_16(wrow + k) : make_uint4(0u, 0u, 0u, 0u);
+    }
   };
 
   if (c0 < c1) {
@@ -132,18 +125,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const uint4 xv = *reinterpret_cast<const uint4*>(&xs[buf][mt * 16 + r][(i * 4 + q) * 8]);
-#pragma unroll
-        for (int t = 0; t < TPW; ++t)
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wcur[t][i]),
-                                                               __builtin_bit_cast(bf16x8, xv), acc[t][mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wcur[i]),
+                                                          __builtin_bit_cast(bf16x8, xv), acc[mt], 0, 0, 0);
       }
     }
     if (more) {
       store_x(buf ^ 1);
 #pragma unroll
-      for (int t = 0; t < TPW; ++t)
-#pragma unroll
-        for (int i = 0; i < SK_NLD; ++i) wcur[t][i] = wnext[t][i];
+      for (int i = 0; i < SK_NLD; ++i) wcur[i] = wnext[i];
     }
     __syncthreads();
   }
@@ -152,7 +141,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   if (GLU) {
     if (half == 1) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) glu_up[wave & 1][mt][lane] = acc[0][mt];
+      for (int mt = 0; mt < MT; ++mt) glu_up[wave & 1][mt][lane] = acc[mt];
     }
     __syncthreads();
     if (half == 1) return;
@@ -166,23 +155,23 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
       TO* o = C + (size_t)m * NO + n;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float gt = acc[0][mt][e];
+        const float gt = acc[mt][e];
         if (n + e < NO) store_out<TO>(o + e, gt / (1.0f + expf(-gt)) * up[e]);
       }
     } else if (part) {
       float* o = part + ((size_t)split * M + m) * N + n;
       if (n + 3 < N && (N & 3) == 0) {
-        *reinterpret_cast<f32x4*>(o) = acc[0][mt];
+        *reinterpret_cast<f32x4*>(o) = acc[mt];
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (n + e < N) o[e] = acc[0][mt][e];
+          if (n + e < N) o[e] = acc[mt][e];
       }
     } else {
       TO* o = C + (size_t)m * N + n;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (n + e < N) store_out<TO>(o + e, acc[0][mt][e]);
+        if (n + e < N) store_out<TO>(o + e, acc[mt][e]);
     }
   }
 }
