@@ -1,10 +1,11 @@
-// C[M, N] = X[M, K] * W[N, K]^T in bf16 with fp32 accumulation, for M <= 64: the
+// C[M, N] = X[M, K] * W[N, K]^T in bf16 with fp32 accumulation, for M <= 128: the
 // matrix product of a decode step.  The weight is read once from HBM, which is
 // what bounds the step.
 //
 // A workgroup of 4 waves owns 64 rows of W (16 per wave) and a range of K.  K is
 // walked in chunks of 256.  The chunk of X (all M rows) is staged in LDS once per
-// workgroup and shared by its waves; every wave reads its own 16 rows of W
+// workgroup and shared by its waves (above 64 rows of X the chunks are 128 long, so that
+// two stages of X still leave room for two workgroups on a compute unit); every wave reads its own 16 rows of W
 // straight from global memory into registers (each byte of W is used by one wave
 // only, so LDS would gain nothing), one chunk ahead of the matrix cores, with
 // plain 16-byte loads.  Products run on v_mfma_f32_16x16x32_bf16 with W as the A
@@ -31,7 +32,6 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #define SK_WAVES 4
 #define SK_KC 256               // k per chunk
-#define SK_NLD (SK_KC / 32)     // 16-byte loads per lane and chunk
 #define SK_XPAD 8               // bf16 elements of padding per LDS row (spreads the banks)
 #define SK_BN (SK_WAVES * 16)   // rows of W per workgroup
 #define SK_TARGET_BLOCKS 512    // K is split until the grid has about this many workgroups ...
@@ -50,22 +50,29 @@ template <> __device__ __forceinline__ void store_out<uint16_t>(uint16_t* p, flo
 // GLU (one split only): a workgroup takes 32 columns n of the result; waves 0 and 1 multiply with the rows n
 // of the first half of W, waves 2 and 3 with the rows N/2 + n of the second half; the halves meet in LDS and
 // silu(first) * second goes to C[m, n], n < N/2.
-template <int MT, bool GLU, typename TO>
+template <int MT, bool GLU, typename TO, int KC>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ X,
                                                                     const uint16_t* __restrict__ W,
                                                                     TO* __restrict__ C, float* __restrict__ part,
                                                                     int M, int N, int K, int chunks_per_split) {
-  constexpr int XROW = SK_KC + SK_XPAD;
-  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][XROW];
-  __shared__ f32x4 glu_up[GLU ? 2 : 1][GLU ? MT : 1][64];
+  // chunks_per_split counts chunks of SK_KC; the kernel walks them in pieces of KC (the sums are the same in
+  // the same order either way: a piece is a run of the chunk's matrix instructions)
+  constexpr int XROW = KC + SK_XPAD;
+  constexpr int NLD = KC / 32;                         // 16-byte loads of W per lane and piece
+  constexpr int PER_CHUNK = SK_KC / KC;
+  extern __shared__ __attribute__((aligned(16))) char skinny_lds[];
+  uint16_t (*xs)[MT * 16][XROW] = reinterpret_cast<uint16_t (*)[MT * 16][XROW]>(skinny_lds);      // two stages
+  // the second halves' sums meet the first halves' in the same memory, once the last stage has been read
+  f32x4 (*glu_up)[MT][64] = reinterpret_cast<f32x4 (*)[MT][64]>(skinny_lds);
+  static_assert(2 * MT * 16 * XROW * 2 >= 2 * MT * 64 * 16, "the stages of X hold the halves' sums");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
   const int half = GLU ? wave >> 1 : 0;                // which half of W this wave multiplies with
   const int n_base = GLU ? blockIdx.x * (SK_BN / 2) + (wave & 1) * 16 : blockIdx.x * SK_BN + wave * 16;
   const int split = blockIdx.y;
-  const int nchunks = (K + SK_KC - 1) / SK_KC;
-  const int c0 = split * chunks_per_split;
-  const int c1 = min(nchunks, c0 + chunks_per_split);
+  const int nchunks = (K + KC - 1) / KC;
+  const int c0 = split * chunks_per_split * PER_CHUNK;
+  const int c1 = min(nchunks, c0 + chunks_per_split * PER_CHUNK);
   const int NO = GLU ? N / 2 : N;                      // columns of the result
 
   const int n_row = (n_base + r < NO) ? n_base + r : NO - 1;
@@ -74,8 +81,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  // the chunk of X is MT*16 rows of 256 values = MT*512 pieces of 16 bytes, spread over the 256 threads
-  constexpr int XPIECES = MT * 16 * (SK_KC / 8);
+  // the chunk of X is MT*16 rows of KC values = MT*2*KC/16 pieces of 16 bytes, spread over the 256 threads
+  constexpr int XPIECES = MT * 16 * (KC / 8);
   constexpr int XPT = XPIECES / (SK_WAVES * 64);
   static_assert(XPIECES % (SK_WAVES * 64) == 0, "pieces of X must divide over the threads");
   uint4 xreg[XPT];
@@ -83,8 +90,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
       const int pc = tid + i * SK_WAVES * 64;
-      const int row = pc / (SK_KC / 8), kk = (pc % (SK_KC / 8)) * 8;
-      const int k = c * SK_KC + kk;
+      const int row = pc / (KC / 8), kk = (pc % (KC / 8)) * 8;
+      const int k = c * KC + kk;
       const int m = row < M ? row : M - 1;
       xreg[i] = (k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k) : make_uint4(0u, 0u, 0u, 0u);
     }
@@ -93,15 +100,15 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
       const int pc = tid + i * SK_WAVES * 64;
-      const int row = pc / (SK_KC / 8), kk = (pc % (SK_KC / 8)) * 8;
+      const int row = pc / (KC / 8), kk = (pc % (KC / 8)) * 8;
       *reinterpret_cast<uint4*>(&xs[buf][row][kk]) = xreg[i];
     }
   };
-  uint4 wcur[SK_NLD], wnext[SK_NLD];
-  auto load_w = [&](int c, uint4 (&dst)[SK_NLD]) {
+  uint4 wcur[NLD], wnext[NLD];
+  auto load_w = [&](int c, uint4 (&dst)[NLD]) {
 #pragma unroll
-    for (int i = 0; i < SK_NLD; ++i) {
-      const int k = c * SK_KC + (i * 4 + q) * 8;
+    for (int i = 0; i < NLD; ++i) {
+      const int k = c * KC + (i * 4 + q) * 8;
       dst[i] = (k < K) ? load_stream_16(wrow + k) : make_uint4(0u, 0u, 0u, 0u);
     }
   };
@@ -121,7 +128,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
       load_w(c + 1, wnext);
     }
 #pragma unroll
-    for (int i = 0; i < SK_NLD; ++i) {
+    for (int i = 0; i < NLD; ++i) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const uint4 xv = *reinterpret_cast<const uint4*>(&xs[buf][mt * 16 + r][(i * 4 + q) * 8]);
@@ -132,7 +139,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
     if (more) {
       store_x(buf ^ 1);
 #pragma unroll
-      for (int i = 0; i < SK_NLD; ++i) wcur[i] = wnext[i];
+      for (int i = 0; i < NLD; ++i) wcur[i] = wnext[i];
     }
     __syncthreads();
   }
@@ -209,6 +216,22 @@ static int skinny_splits(int N, int K) {
 // Number of K splits the kernel uses for a weight [N, K] (a function of N and K only).
 extern "C" int ia_gemm_skinny_splits(int N, int K) { return (N > 0 && K > 0) ? skinny_splits(N, K) : 0; }
 
+template <int MT, bool GLU, typename TO, int KC>
+static int launch_skinny_one(dim3 grid, const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K,
+                             int cps, hipStream_t stream) {
+  constexpr size_t lds = (size_t)2 * MT * 16 * (KC + SK_XPAD) * sizeof(uint16_t);
+  static bool allowed = false;      // more than 64 KB of LDS has to be asked for, once per kernel
+  if (lds > 65536 && !allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, GLU, TO, KC>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    allowed = true;
+  }
+  gemm_skinny_kernel<MT, GLU, TO, KC><<<grid, SK_WAVES * 64, lds, stream>>>(x, w, c, part, M, N, K, cps);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 template <bool GLU, typename TO>
 static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K, int splits,
                          hipStream_t stream) {
@@ -218,14 +241,17 @@ static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* par
   const int cols = GLU ? SK_BN / 2 : SK_BN;           // columns of the result per workgroup
   dim3 grid((NO + cols - 1) / cols, splits);
   switch ((M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 2: gemm_skinny_kernel<2, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 3: gemm_skinny_kernel<3, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
-    case 4: gemm_skinny_kernel<4, GLU, TO><<<grid, SK_WAVES * 64, 0, stream>>>(x, w, c, part, M, N, K, cps); break;
+    case 1: return launch_skinny_one<1, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 2: return launch_skinny_one<2, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 3: return launch_skinny_one<3, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 4: return launch_skinny_one<4, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
+    // above 64 rows: pieces of 128, so that the two stages of X of two workgroups fit a compute unit's LDS
+    case 5: return launch_skinny_one<5, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 6: return launch_skinny_one<6, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 7: return launch_skinny_one<7, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 8: return launch_skinny_one<8, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
     default: return IA_ERR_UNSUPPORTED;
   }
-  IA_LAUNCH_CHECK();
-  return IA_OK;
 }
 
 template <typename TO>
@@ -246,7 +272,7 @@ static int launch_join(const float* part, TO* c, int M, int N, int splits, int e
 // as [splits, M, N] for a later kernel to join.
 extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
                               int epilogue, float* workspace, size_t workspace_floats, hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
+  if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
   if (epilogue != SK_EPI_NONE && epilogue != SK_EPI_SWIGLU) return IA_ERR_BAD_ARG;
   if (epilogue == SK_EPI_SWIGLU && (N & 1)) return IA_ERR_BAD_ARG;
   if (out_dtype != IA_F32 && out_dtype != IA_BF16) return IA_ERR_BAD_ARG;

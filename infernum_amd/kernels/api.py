@@ -302,7 +302,7 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] =
     return out
 
 
-SKINNY_MAX_M = 64
+SKINNY_MAX_M = 128
 EPILOGUE = {None: 0, "swiglu": 1}
 
 
@@ -328,7 +328,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     N = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bf16 operands")
     _need(w.dim() == 2 and w.shape[1] == K, "gemm_skinny: shapes")
-    _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 64, K % 8 == 0)")
+    _need(gemm_skinny_supported(M, N, K), f"gemm_skinny: M={M} N={N} K={K} not supported (M <= 128, K % 8 == 0)")
     _need(epilogue in EPILOGUE, f"gemm_skinny: unknown epilogue {epilogue!r}")
     _need(epilogue is None or N % 2 == 0, "gemm_skinny: the swiglu epilogue needs an even N")
     splits = gemm_skinny_splits(N, K)

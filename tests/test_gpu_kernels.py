@@ -237,7 +237,7 @@ def test_gemm_generic(M, N, K_):
     assert torch.allclose(outf.double(), wantb, atol=1e-3, rtol=1e-4)
 
 
-@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64, 65, 81, 100, 128])
 @pytest.mark.parametrize("N,K_", [(250, 96), (384, 176), (4096, 4096), (1000, 14336), (16, 8), (129, 1000)])
 def test_gemm_skinny(M, N, K_):
     api = K()
@@ -256,7 +256,7 @@ def test_gemm_skinny(M, N, K_):
     assert torch.equal(one[0], outf[M - 1])
 
 
-@pytest.mark.parametrize("M", [1, 8, 40, 64])
+@pytest.mark.parametrize("M", [1, 8, 40, 64, 72, 128])
 @pytest.mark.parametrize("N,K_", [(352, 128), (4096, 4096), (1000, 14336), (28672, 4096), (130, 1000)])
 def test_gemm_skinny_partial_sums_and_swiglu(M, N, K_):
     api = K()
@@ -284,7 +284,7 @@ def test_gemm_skinny_partial_sums_and_swiglu(M, N, K_):
 
 def test_gemm_skinny_refuses_what_it_cannot_do():
     api = K()
-    a, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
+    a, w = _rand(129, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
     with pytest.raises(api.KernelError):
         api.gemm_skinny(a, w)
     with pytest.raises(api.KernelError):
