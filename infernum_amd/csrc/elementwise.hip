@@ -269,7 +269,10 @@ extern "C" int ia_residual_add(float* h, const void* delta, int act_dtype, int N
 // the q heads are read.  src is [splits, N, row_stride]: one tensor in the activations' dtype, or a stack
 // of fp32 partial sums of a split matrix product (added in the order of their index).
 // The first `rot` values of every q and k head are rotated in half-split pairs (x[i], x[i + rot/2]) by the
-// angle pos * inv_freq[i], computed in fp32 (one sincos per thread, used for all its heads).
+// angle pos * inv_freq[i] (one sincos per thread, used for all its heads).  With a table of float64
+// frequencies the product is formed in float64 and brought into [-pi, pi] there before the fp32 sine and
+// cosine, so that the angle is good to 3e-7 rad at any position; with a table of fp32 frequencies the
+// product is the fp32 one (off by up to pos * 2^-24 rad).
 // Rotated q goes to q_out (row stride q_stride; it may be src itself: rotation in place); rotated k and raw
 // v go to the page slot of the token: key pages are [num_pages, nkv, page_size, d]; value pages are stored
 // transposed, [num_pages, nkv, d, page_size], the layout the matrix cores want for the product of
@@ -281,6 +284,20 @@ __device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t 
 #pragma unroll 4
   for (int k = 1; k < splits; ++k) v += to_float(p[k * split_stride]);
   return v;
+}
+
+// Sine and cosine of position * frequency i (see above), the same arithmetic in every kernel that rotates.
+__device__ __forceinline__ void rope_sincos(int position, const void* __restrict__ table, int table_f64, int i,
+                                            float& sn, float& cs) {
+  if (table_f64) {
+    const double a = (double)position * reinterpret_cast<const double*>(table)[i];
+    const double turns = rint(a * 0.15915494309189535);                 // a / (2 pi)
+    // 2 pi as a double is off by 2.4e-16: times a million turns still far below the fp32 sine's own error
+    const double r = __builtin_fma(-turns, 6.283185307179586, a);
+    sincosf((float)r, &sn, &cs);
+  } else {
+    sincosf((float)position * reinterpret_cast<const float*>(table)[i], &sn, &cs);
+  }
 }
 
 // The rotation of one pair, in one fixed order of roundings (a product, then a fused multiply-add), so that
@@ -297,7 +314,7 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restric
                                                              size_t split_stride, T* __restrict__ q_out,
                                                              int q_stride, const int* __restrict__ positions,
                                                              const int* __restrict__ slots,
-                                                             const float* __restrict__ inv_freq,
+                                                             const void* __restrict__ inv_freq, int freq_f64,
                                                              T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                              int row_stride, int nh, int nkv, int d, int rot,
                                                              int page_size, int num_pages, int write_kv,
@@ -321,10 +338,10 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restric
   T* dst = is_q ? q_out + (size_t)n * q_stride + (size_t)head * d
                 : k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d;
   const int half = rot >> 1;
-  const float pos = (float)positions[n];
+  const int pos = positions[n];
   for (int i = lane; i < half; i += 64) {
     float sn, cs;
-    sincosf(pos * inv_freq[i], &sn, &cs);
+    rope_sincos(pos, inv_freq, freq_f64, i, sn, cs);
     const float a = load_split_sum(x + i, splits, split_stride);
     const float b = load_split_sum(x + i + half, splits, split_stride);
     float lo, hi;
@@ -343,16 +360,16 @@ __global__ __launch_bounds__(256) void rope_kv_append_kernel(const TS* __restric
 template <typename TS, typename T>
 __global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(
     const TS* __restrict__ src, T* __restrict__ q_out, int q_stride, const int* __restrict__ positions,
-    const int* __restrict__ slots, const float* __restrict__ inv_freq, T* __restrict__ k_pages,
+    const int* __restrict__ slots, const void* __restrict__ inv_freq, int freq_f64, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int row_stride, int nh, int nkv, int d, int rot, int page_size, int num_pages,
     int write_kv, int copy_q_tail) {
   __shared__ __attribute__((aligned(16))) float cs_[128], sn_[128];
   const int n = blockIdx.x, tid = threadIdx.x;
   const int half = rot >> 1;
-  const float pos = (float)positions[n];
+  const int pos = positions[n];
   for (int i = tid; i < half; i += 256) {
     float sn, cs;
-    sincosf(pos * inv_freq[i], &sn, &cs);
+    rope_sincos(pos, inv_freq, freq_f64, i, sn, cs);
     sn_[i] = sn;
     cs_[i] = cs;
   }
@@ -398,10 +415,11 @@ __global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(
   }
 }
 
-// src: [splits, src_rows, row_stride] of src_dtype; q_out, pages: act_dtype.
+// src: [splits, src_rows, row_stride] of src_dtype; q_out, pages: act_dtype; inv_freq: rot/2 values, float64
+// when freq_f64 is set, fp32 otherwise.
 extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int src_rows, void* q_out, int q_stride,
-                                 int act_dtype, const int* positions, const int* slots, const float* inv_freq,
-                                 void* k_pages, void* v_pages, int N, int row_stride, int nh, int nkv, int d, int rot,
+                                 int act_dtype, const int* positions, const int* slots, const void* inv_freq,
+                                 int freq_f64, void* k_pages, void* v_pages, int N, int row_stride, int nh, int nkv, int d, int rot,
                                  int page_size, int num_pages, int write_kv, hipStream_t stream) {
   if (N < 0 || nh <= 0 || nkv <= 0 || d <= 0 || rot < 0 || rot > d || (rot & 1)) return IA_ERR_BAD_ARG;
   if (row_stride < (nh + (write_kv ? 2 * nkv : 0)) * d || q_stride < nh * d || splits < 1 || src_rows < N)
@@ -419,7 +437,7 @@ extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int
       (q_stride & 3) == 0 && aligned) {
 #define ROPE_ROWS_LAUNCH(TS, T)                                                                                    \
   rope_kv_append_rows_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, (T*)q_out, q_stride, positions, slots,  \
-                                                           inv_freq, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
+                                                           inv_freq, freq_f64, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
                                                            d, rot, page_size, num_pages, write_kv, copy_q_tail)
     if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_ROWS_LAUNCH(float, float);
     else if (act_dtype == IA_BF16 && src_dtype == IA_BF16) ROPE_ROWS_LAUNCH(bf16_t, bf16_t);
@@ -431,7 +449,7 @@ extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int
   }
 #define ROPE_LAUNCH(TS, T)                                                                                         \
   rope_kv_append_kernel<TS, T><<<grid, 256, 0, stream>>>((const TS*)src, splits, stride, (T*)q_out, q_stride,      \
-                                                         positions, slots, inv_freq, (T*)k_pages, (T*)v_pages,     \
+                                                         positions, slots, inv_freq, freq_f64, (T*)k_pages, (T*)v_pages, \
                                                          row_stride, nh, nkv, d, rot, page_size, num_pages,        \
                                                          write_kv, copy_q_tail)
   if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_LAUNCH(float, float);

@@ -199,8 +199,8 @@ def rope_kv_append(qkv, positions: torch.Tensor, inv_freq: Optional[torch.Tensor
     _need(row >= (nh + (2 * nkv if write else 0)) * d, "rope: row of qkv is too short for its heads")
     _i32(positions, N, "rope positions")
     if inv_freq is not None:
-        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2 and rot % 2 == 0 and 0 < rot <= d,
-              "rope: inv_freq must hold rot/2 fp32 values, rot even and at most the head size")
+        _need(inv_freq.dtype in (torch.float32, torch.float64) and inv_freq.numel() == rot // 2 and rot % 2 == 0
+              and 0 < rot <= d, "rope: inv_freq must hold rot/2 fp32 or float64 values, rot even and at most the head size")
     page_size = num_pages = 0
     if write:
         _need(v_pages is not None and slots is not None, "rope: k_pages, v_pages and slots go together")
@@ -212,6 +212,7 @@ def rope_kv_append(qkv, positions: torch.Tensor, inv_freq: Optional[torch.Tensor
         _i32(slots, N, "rope slots")
     _ok(_core().ia_rope_kv_append(_p(src), DTYPE_CODE[src.dtype], src.shape[0] if split else 1, N, _p(q_out),
                                   q_out.stride(0), DTYPE_CODE[act], _p(positions), _p(slots), _p(inv_freq),
+                                  1 if (inv_freq is not None and inv_freq.dtype == torch.float64) else 0,
                                   _p(k_pages), _p(v_pages), N, row, nh, nkv, d, rot if inv_freq is not None else 0,
                                   page_size, num_pages, 1 if write else 0, _stream()), "rope_kv_append")
     return q_out

@@ -13,8 +13,11 @@ context n, L < n/high keeps f, L > n/low gives f/factor, and between them
 f' = (1-r) f/factor + r f with r = (n/L - low) / (high - low).  There is no
 magnitude correction.
 
-Frequencies are formed in float64 and rounded once to fp32; angles are the
-fp32 product of the fp32 position and the fp32 frequency.
+Frequencies are formed and kept in float64; the rotation kernel forms the angle
+position * frequency in float64 too and brings it into [-pi, pi] before it takes
+the fp32 sine and cosine, so that the angle is as good at position 100,000 as at
+position 1 (a table of fp32 frequencies, which a position encoding may also give,
+is multiplied in fp32: off by up to position * 2^-24 rad).
 """
 from __future__ import annotations
 
@@ -27,7 +30,7 @@ from .base import PositionEncoding, Runtime, register_part
 
 
 def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Mapping[str, Any]] = None) -> torch.Tensor:
-    """fp32 [rotary_dim / 2] on the CPU."""
+    """float64 [rotary_dim / 2] on the CPU."""
     if rotary_dim <= 0 or rotary_dim % 2:
         raise ValueError(f"rotary size must be even and positive, got {rotary_dim}")
     half = rotary_dim // 2
@@ -51,7 +54,7 @@ def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Ma
                 r = (n / wavelen - low) / (high - low)
                 f = (1.0 - r) * f / factor + r * f
         freqs.append(f)
-    return torch.tensor(freqs, dtype=torch.float64).to(torch.float32)
+    return torch.tensor(freqs, dtype=torch.float64)
 
 
 class RotaryEmbedding(PositionEncoding):

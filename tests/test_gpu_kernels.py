@@ -179,6 +179,31 @@ def test_rope_kv_append(dtype, nh, nkv, d, rot, ps):
     assert torch.allclose(q2.double().reshape(N, nh, d), roted[:, :nh], atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("N", [6, 40])
+def test_rope_angles_at_far_positions(N):
+    """With a table of float64 frequencies the angle is formed in float64: positions of a million are rotated as
+    exactly as position 1 (an fp32 product would be off by 0.06 rad there); both kernels (few tokens, many)."""
+    nh, nkv, d, rot, ps = 2, 1, 64, 64, 8
+    qkv = _rand(N, (nh + 2 * nkv) * d, seed=5)
+    pos = torch.tensor([1, 1000, 65537, 999983, 1000000, 16777215] * (N // 6 + 1), dtype=torch.int32, device=DEV)[:N].contiguous()
+    inv64 = 500000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)
+    slots = torch.arange(N, dtype=torch.int32, device=DEV)
+    kp, vp = torch.zeros(N // ps + 1, nkv, ps, d, device=DEV), torch.zeros(N // ps + 1, nkv, d, ps, device=DEV)
+    got = qkv.clone()
+    K().rope_kv_append(got, pos, inv64.to(DEV), nh, nkv, d, rot, slots, kp, vp)
+    x = qkv.double().cpu().reshape(N, nh + 2 * nkv, d)
+    ang = pos.cpu().double()[:, None] * inv64[None, :]
+    c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[:, :nh, :rot // 2], x[:, :nh, rot // 2:]
+    g = got[:, :nh * d].double().cpu().reshape(N, nh, d)
+    assert (g[..., :rot // 2] - (a * c - b * s_)).abs().max() <= 3e-6
+    assert (g[..., rot // 2:] - (a * s_ + b * c)).abs().max() <= 3e-6
+    # the same positions with the table rounded to fp32 are visibly off: the test can tell the two apart
+    off = qkv.clone()
+    K().rope_kv_append(off, pos, inv64.float().to(DEV), nh, nkv, d, rot)
+    assert (off[:, :nh * d].double().cpu().reshape(N, nh, d)[..., :rot // 2] - (a * c - b * s_)).abs().max() > 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,d,rot,ps", [(6, 2, 48, 48, 5), (32, 8, 128, 128, 16), (5, 1, 128, 64, 7), (3, 3, 20, 8, 4)])
 def test_rope_of_many_tokens_equals_rope_of_few(dtype, nh, nkv, d, rot, ps):

@@ -59,8 +59,8 @@ def test_position_frequencies(name):
     rope = make_part("position", PartSpec("rope", {"head_dim": cfg.head_dim, "theta": cfg.rope_theta,
                                                    "scaling": scaling}), rt)
     want = P.rope_frequencies(cfg.head_dim, cfg.rope_theta, scaling)
-    assert rope.inv_freq.dtype == torch.float32 and rope.rotary_dim == cfg.head_dim
-    assert torch.allclose(rope.inv_freq.cpu().double(), want, rtol=1e-7, atol=0)
+    assert rope.inv_freq.dtype == torch.float64 and rope.rotary_dim == cfg.head_dim
+    assert torch.allclose(rope.inv_freq.cpu(), want, rtol=1e-15, atol=0)
     if name == "B":      # the three bands: kept, blended, divided by the factor
         plain = P.rope_frequencies(cfg.head_dim, cfg.rope_theta, None)
         r = (rope.inv_freq.cpu().double() / plain)
