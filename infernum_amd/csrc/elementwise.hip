@@ -17,6 +17,35 @@ __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table,
     return;
   }
   const T* r = table + (size_t)id * H;
+  // 16 bytes of the table at a time where rows allow it, all of a thread's loads issued before its first store
+  constexpr int PER = 16 / (int)sizeof(T);              // values in 16 bytes
+  if (H % PER == 0 && (reinterpret_cast<uintptr_t>(table) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+      H <= 256 * PER * 4) {
+    uint4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = (threadIdx.x + k * 256) * PER;
+      v[k] = i < H ? *reinterpret_cast<const uint4*>(r + i) : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = (threadIdx.x + k * 256) * PER;
+      if (i >= H) continue;
+      if (sizeof(T) == 4) {
+        *reinterpret_cast<uint4*>(o + i) = v[k];
+      } else {
+        const uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        float4 lo, hi;
+        lo.x = __uint_as_float(w[0] << 16); lo.y = __uint_as_float(w[0] & 0xffff0000u);
+        lo.z = __uint_as_float(w[1] << 16); lo.w = __uint_as_float(w[1] & 0xffff0000u);
+        hi.x = __uint_as_float(w[2] << 16); hi.y = __uint_as_float(w[2] & 0xffff0000u);
+        hi.z = __uint_as_float(w[3] << 16); hi.w = __uint_as_float(w[3] & 0xffff0000u);
+        *reinterpret_cast<float4*>(o + i) = lo;
+        *reinterpret_cast<float4*>(o + i + 4) = hi;
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H; i += 256) o[i] = to_float(r[i]);
 }
 

@@ -23,7 +23,7 @@ def _rand(*shape, dtype=torch.float32, scale=1.0, seed=0):
 
 # ------------------------------------------------------------------------ rows
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,V", [(100, 77), (4096, 1000), (1536, 333)])
+@pytest.mark.parametrize("H,V", [(100, 77), (4096, 1000), (1536, 333), (5120, 50), (8200, 9)])
 def test_embed(dtype, H, V):
     table = _rand(V, H, dtype=dtype)
     ids = torch.tensor([0, V - 1, 5, 5, V // 2], dtype=torch.int32, device=DEV)
