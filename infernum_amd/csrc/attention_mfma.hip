@@ -74,11 +74,12 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 // loads of keys and values wait for no other global load, and a wave's next tile is in flight while it
 // works on this one.
 #define DEC_WAVES 4
-#define DEC_BT_LDS 4096          // block-table entries kept in LDS (a longer slice is read from global memory)
+#define DEC_BT_LDS 2048          // block-table entries kept in LDS (a longer slice is read from global memory)
 
 struct DecTile {                 // 16 keys as they come from memory: operands of the two products
   s16x4 k[NS];
   uint2 v[NS];
+  uint32_t mlo, mhi;             // which of the lane's four values are of keys in range (16 bits each)
   bool bad;                      // a key that is needed has no page
 };
 
@@ -90,6 +91,11 @@ struct DecGeom {                 // what does not change from tile to tile
   int bt_first, bt_count;        // the slice [bt_first, bt_first + bt_count) of the table lies in bt_lds
   size_t page_elems;
   int ps, ps_shift, num_pages, key_lo, key_hi;
+  // the token's own key and value, when the kernel made them itself: they replace what the loads of the
+  // tile of key patch_key bring for that key (patch_key < 0: nothing to replace)
+  int patch_key;
+  const uint16_t* new_k;         // [HD] in LDS
+  const uint16_t* new_v;         // [HD] in LDS
 };
 
 __device__ __forceinline__ int dec_page(const DecGeom& G, int key) {
@@ -119,12 +125,35 @@ __device__ __forceinline__ void dec_load(const DecGeom& G, int t0, int j, int qd
     mhi = ((kg + 2 >= G.key_lo && kg + 2 <= G.key_hi) ? 0x0000ffffu : 0u) | ((kg + 3 >= G.key_lo && kg + 3 <= G.key_hi) ? 0xffff0000u : 0u);
   }
 #pragma unroll
-  for (int n = 0; n < NS; ++n) {
-    const uint2 v = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
-    T.v[n] = make_uint2(v.x & mlo, v.y & mhi);
-  }
+  for (int n = 0; n < NS; ++n) T.v[n] = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
+  T.mlo = mlo;
+  T.mhi = mhi;
   const bool k_needed = key == keyc, v_needed = kg + 3 >= G.key_lo && kg <= G.key_hi;
   T.bad = (k_needed && !page_ok) || (v_needed && !pagev_ok);
+}
+
+// What is done to a tile once its loads have come: values of keys out of range become zero, and the token's
+// own key and value take the place of what the page held.  Called right before the tile is used, so that the
+// loads stay in flight until then.
+__device__ __forceinline__ void dec_finish(const DecGeom& G, int t0, int j, int qd, DecTile& T) {
+#pragma unroll
+  for (int n = 0; n < NS; ++n) T.v[n] = make_uint2(T.v[n].x & T.mlo, T.v[n].y & T.mhi);
+  if (G.patch_key >= 0 && t0 == (G.patch_key & ~15)) {       // the same for all lanes of the wave
+    if (j == (G.patch_key & 15)) load_row_operand(G.new_k, qd, T.k);
+    const int e = G.patch_key - (t0 + 4 * qd);               // which of this lane's four keys, if any
+    if (e >= 0 && e < 4) {
+#pragma unroll
+      for (int n = 0; n < NS; ++n) {
+        const uint32_t nv = G.new_v[n * 16 + j];
+        uint32_t lo = T.v[n].x, hi = T.v[n].y;
+        if (e == 0) lo = (lo & 0xffff0000u) | nv;
+        else if (e == 1) lo = (lo & 0x0000ffffu) | (nv << 16);
+        else if (e == 2) hi = (hi & 0xffff0000u) | nv;
+        else hi = (hi & 0x0000ffffu) | (nv << 16);
+        T.v[n] = make_uint2(lo, hi);
+      }
+    }
+  }
 }
 
 // One tile of 16 keys, t0 .. t0+15, against the 16 columns (heads) of this wave.
@@ -171,23 +200,65 @@ __device__ __forceinline__ void dec_compute(int t0, const DecTile& T, const s16x
   }
 }
 
-extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
-    const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o,
-    float* __restrict__ part_ml, const int* __restrict__ positions, const int* __restrict__ block_tables,
-    int bt_stride, int nh, int nkv, int ps, int num_pages, float scale_log2, int window, int num_splits) {
+// What the kernel needs to make the token's query, key and value itself (FUSED): the row of the QKV product
+// [nh q heads | nkv k heads | nkv v heads], possibly as a stack of partial sums, and what the rotation needs.
+// The arithmetic is that of rope_kv_append_kernel, so the bits are the same as with that kernel in front.
+struct DecFused {
+  const void* src;               // [gsplits, rows, row_stride] in TS
+  size_t split_stride;
+  const int* slots;              // page * page_size + offset of every token's key; nullptr: no key and value are made
+  const void* inv_freq;          // rot/2 frequencies; nullptr with rot == 0
+  int gsplits, row_stride, freq_f64, rot;
+};
+
+// FUSED: q is not read; every workgroup rotates the queries of its heads into LDS, the workgroups whose keys
+// include the token's own also make its key and value, use them from LDS (the loads from the page are replaced
+// in registers) and one of them (the first tile of heads) writes them to the page.
+template <bool FUSED, typename TS>
+__global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_decode_kernel(
+    const uint16_t* __restrict__ q, int q_row_stride, uint16_t* k_pages, uint16_t* v_pages,
+    uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ positions, const int* __restrict__ block_tables, int bt_stride, int nh, int nkv, int ps,
+    int num_pages, float scale_log2, int window, int num_splits, DecFused F) {
   __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
   __shared__ f32x4 s_o[DEC_WAVES][NS][64];
   __shared__ int s_bt[DEC_BT_LDS];
+  __shared__ __attribute__((aligned(16))) uint16_t s_q[FUSED ? 16 : 1][HD];
+  __shared__ __attribute__((aligned(16))) uint16_t s_newk[HD], s_newv[HD];
+  __shared__ float s_cos[HD / 2], s_sin[HD / 2];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, qd = lane >> 4;
   const int G = nh / nkv, HT = (G + 15) / 16;
   const int g = blockIdx.y / HT, ht = blockIdx.y - g * HT;
   const int split = blockIdx.z;
-  const int p = positions[b];
-  const int lo0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  constexpr int NT = DEC_WAVES * 64;
+  const int tid = threadIdx.x;
   const int hj = ht * 16 + j;
   const bool col_ok = hj < G;
   const int h = g * G + hj;
+  const int heads_here = (G - ht * 16) < 16 ? (G - ht * 16) : 16;
+
+  // FUSED: the sums of the queries' pairs are asked for first of all (they need nothing but the token's row),
+  // so that they come in while the position, the block table and the angles are worked out
+  constexpr int QPT = (16 * (HD / 2) + NT - 1) / NT;        // pairs of query values a thread may have to rotate
+  float qa[FUSED ? QPT : 1], qb[FUSED ? QPT : 1];
+  const int half = FUSED ? F.rot >> 1 : 0;
+  const TS* row = reinterpret_cast<const TS*>(F.src) + (size_t)b * F.row_stride;
+  if (FUSED) {
+#pragma unroll
+    for (int u = 0; u < QPT; ++u) {
+      const int idx = tid + u * NT;
+      qa[u] = qb[u] = 0.f;
+      if (idx < heads_here * half) {
+        const int c = idx / half, i = idx - c * half;
+        const TS* x = row + (size_t)(g * G + ht * 16 + c) * HD + i;
+        qa[u] = load_split_sum(x, F.gsplits, F.split_stride);
+        qb[u] = load_split_sum(x + half, F.gsplits, F.split_stride);
+      }
+    }
+  }
+
+  const int p = positions[b];
+  const int lo0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int t_first = lo0 / 16, t_last = p / 16;
   const int per = (t_last - t_first + 1 + num_splits - 1) / num_splits;
   const int ta = t_first + split * per;
@@ -205,6 +276,9 @@ extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
   geo.v_base = v_pages + (size_t)g * HD * ps;
   geo.bt_global = bt;
   geo.bt_lds = s_bt;
+  geo.patch_key = -1;
+  geo.new_k = s_newk;
+  geo.new_v = s_newv;
   // the slice of the block table that this workgroup's keys need
   {
     const int k_from = ta * 16 < lo0 ? lo0 : ta * 16, k_to = tb * 16 - 1 > p ? p : tb * 16 - 1;
@@ -214,32 +288,100 @@ extern "C" __global__ __launch_bounds__(DEC_WAVES * 64) void attn_decode_kernel(
     if (count > DEC_BT_LDS) count = DEC_BT_LDS;
     geo.bt_first = first;
     geo.bt_count = count;
-    for (int i = threadIdx.x; i < count; i += DEC_WAVES * 64) s_bt[i] = bt[first + i];
+    for (int i = tid; i < count; i += NT) s_bt[i] = bt[first + i];
   }
-  s16x4 qreg[NS];
-  if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg);
-  else zero_row_operand(qreg);
   const int pos = col_ok ? p : -1;
   f32x4 o[NS];
 #pragma unroll
   for (int n = 0; n < NS; ++n) o[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  __syncthreads();
-  // two tiles in flight: the loads of the next tile of this wave are issued before this one is worked on
+  s16x4 qreg[NS];
   DecTile A, B;
   int t = ta + wave;
-  if (t < tb) dec_load(geo, t * 16, j, qd, A);
+  // this workgroup's keys end with the token's own, which it makes itself
+  const bool own_key = FUSED && F.slots != nullptr && ta < tb && t_last < tb;
+  if (FUSED) {
+    // the key's pair and the value of this thread, and the angles (one a thread)
+    float ka = 0.f, kb = 0.f, vv = 0.f;
+    if (own_key) {
+      if (tid < half) {
+        const TS* x = row + (size_t)(nh + g) * HD + tid;
+        ka = load_split_sum(x, F.gsplits, F.split_stride);
+        kb = load_split_sum(x + half, F.gsplits, F.split_stride);
+      }
+      if (tid < HD) vv = load_split_sum(row + (size_t)(nh + nkv + g) * HD + tid, F.gsplits, F.split_stride);
+    }
+    for (int i = tid; i < half; i += NT) rope_sincos(p, F.inv_freq, F.freq_f64, i, s_sin[i], s_cos[i]);
+    // barriers without the fence of __syncthreads(), which would wait for every load in flight: only LDS
+    // traffic has to be through
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    if (t < tb) dec_load(geo, t * 16, j, qd, A);             // the first tile's loads fly during the rotation
+#pragma unroll
+    for (int u = 0; u < QPT; ++u) {
+      const int idx = tid + u * NT;
+      if (idx < heads_here * half) {
+        const int c = idx / half, i = idx - c * half;
+        float lo, hi;
+        rope_pair(qa[u], qb[u], s_cos[i], s_sin[i], lo, hi);
+        s_q[c][i] = float_to_bf16_bits(lo);
+        s_q[c][i + half] = float_to_bf16_bits(hi);
+      }
+    }
+    const int tail = HD - F.rot;                             // values beyond the rotated part: copies
+    for (int idx = tid; idx < heads_here * tail; idx += NT) {
+      const int c = idx / tail, i = F.rot + (idx - c * tail);
+      s_q[c][i] = float_to_bf16_bits(
+          load_split_sum(row + (size_t)(g * G + ht * 16 + c) * HD + i, F.gsplits, F.split_stride));
+    }
+    if (own_key) {
+      if (tid < half) {
+        float lo, hi;
+        rope_pair(ka, kb, s_cos[tid], s_sin[tid], lo, hi);
+        s_newk[tid] = float_to_bf16_bits(lo);
+        s_newk[tid + half] = float_to_bf16_bits(hi);
+      }
+      for (int i = F.rot + tid; i < HD; i += NT)
+        s_newk[i] = float_to_bf16_bits(load_split_sum(row + (size_t)(nh + g) * HD + i, F.gsplits, F.split_stride));
+      if (tid < HD) s_newv[tid] = float_to_bf16_bits(vv);
+      geo.patch_key = p;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    if (col_ok) load_row_operand(s_q[j], qd, qreg);
+    else zero_row_operand(qreg);
+  } else {
+    if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg);
+    else zero_row_operand(qreg);
+    __syncthreads();
+    if (t < tb) dec_load(geo, t * 16, j, qd, A);
+  }
+  // two tiles in flight: the loads of the next tile of this wave are issued before this one is worked on
   while (t < tb) {
     const bool more1 = t + DEC_WAVES < tb;
     if (more1) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, B);
+    dec_finish(geo, t * 16, j, qd, A);
     dec_compute(t * 16, A, qreg, pos, lo0, qd, scale_log2, o, m, l);
     t += DEC_WAVES;
     if (!more1) break;
     const bool more2 = t + DEC_WAVES < tb;
     if (more2) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, A);
+    dec_finish(geo, t * 16, j, qd, B);
     dec_compute(t * 16, B, qreg, pos, lo0, qd, scale_log2, o, m, l);
     t += DEC_WAVES;
     if (!more2) break;
+  }
+  if (FUSED && own_key && ht == 0) {                         // to the page, for the steps to come
+    const int slot = F.slots[b];
+    if (slot >= 0 && slot < num_pages * ps) {
+      const int page = slot / ps, off = slot - page * ps;
+      uint16_t* kd = k_pages + (((size_t)page * nkv + g) * ps + off) * HD;
+      uint16_t* vd = v_pages + ((size_t)page * nkv + g) * HD * ps + off;
+      for (int i = tid; i < HD; i += NT) {
+        kd[i] = s_newk[i];
+        vd[(size_t)i * ps] = s_newv[i];
+      }
+    }
   }
   // ---- join the waves: common maximum, rescale, add in the order of the waves
   if (qd == 0) { s_m[wave][j] = m; s_l[wave][j] = l; }
@@ -637,24 +779,78 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
 // ------------------------------------------------------------------ C interface
 extern "C" int ia_attn_head_dim() { return HD; }
 
-extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
-                              int out_row_stride, float* part_o, float* part_ml, const int* positions,
-                              const int* block_tables, int bt_stride, int B, int nh, int nkv, int ps, int num_pages,
-                              float scale, int window, int num_splits, hipStream_t stream) {
+static int dec_check(int B, int nh, int nkv, int ps, int num_pages, int bt_stride, int num_splits,
+                     const float* part_o, const float* part_ml, int out_row_stride) {
   if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 || bt_stride <= 0 ||
       num_splits < 1 || num_splits > 65535)
     return IA_ERR_BAD_ARG;
   if (num_splits > 1 && (!part_o || !part_ml)) return IA_ERR_BAD_ARG;
-  if ((q_row_stride & 7) || (out_row_stride & 3)) return IA_ERR_UNSUPPORTED;
-  if (B == 0) return IA_OK;
+  if (out_row_stride & 3) return IA_ERR_UNSUPPORTED;
   const int G = nh / nkv, HT = (G + 15) / 16;
   if (nkv * HT > 65535) return IA_ERR_UNSUPPORTED;
+  return IA_OK;
+}
+
+extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
+                              int out_row_stride, float* part_o, float* part_ml, const int* positions,
+                              const int* block_tables, int bt_stride, int B, int nh, int nkv, int ps, int num_pages,
+                              float scale, int window, int num_splits, hipStream_t stream) {
+  const int rc = dec_check(B, nh, nkv, ps, num_pages, bt_stride, num_splits, part_o, part_ml, out_row_stride);
+  if (rc != IA_OK) return rc;
+  if (q_row_stride & 7) return IA_ERR_UNSUPPORTED;
+  if (B == 0) return IA_OK;
+  const int G = nh / nkv, HT = (G + 15) / 16;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(B, nkv * HT, num_splits);
-  attn_decode_kernel<<<grid, DEC_WAVES * 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
-                                              (const uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o,
-                                              part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages,
-                                              scale_log2, window, num_splits);
+  attn_decode_kernel<false, bf16_t><<<grid, DEC_WAVES * 64, 0, stream>>>(
+      (const uint16_t*)q, q_row_stride, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o,
+      part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{});
+  IA_LAUNCH_CHECK();
+  if (num_splits > 1) {
+    attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,
+                                                         num_splits);
+    IA_LAUNCH_CHECK();
+  }
+  return IA_OK;
+}
+
+// The same with the rotation in front: row b of src is the QKV product of token b, [nh q heads | nkv k heads |
+// nkv v heads] (the k and v heads only with slots), in bf16 (src_dtype IA_BF16, src_splits 1) or as src_splits
+// partial sums in fp32, part s at src + s * src_rows * row_stride.  The first `rot` values of every q and k head
+// are rotated by position * inv_freq (rot/2 values, float64 with freq_f64); inv_freq == nullptr: no rotation.
+// With slots, the token's key and value go to slot slots[b] of the pages and take part in the attention.
+extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_splits, int src_rows, int row_stride,
+                                    const int* slots, const void* inv_freq, int freq_f64, int rot, void* k_pages,
+                                    void* v_pages, void* out, int out_row_stride, float* part_o, float* part_ml,
+                                    const int* positions, const int* block_tables, int bt_stride, int B, int nh,
+                                    int nkv, int ps, int num_pages, float scale, int window, int num_splits,
+                                    hipStream_t stream) {
+  const int rc = dec_check(B, nh, nkv, ps, num_pages, bt_stride, num_splits, part_o, part_ml, out_row_stride);
+  if (rc != IA_OK) return rc;
+  if (!src || src_splits < 1 || src_rows < B || rot < 0 || rot > HD || (rot & 1)) return IA_ERR_BAD_ARG;
+  if (row_stride < (nh + (slots ? 2 * nkv : 0)) * HD) return IA_ERR_BAD_ARG;
+  if (!(src_dtype == IA_F32 || (src_dtype == IA_BF16 && src_splits == 1))) return IA_ERR_BAD_ARG;
+  if (B == 0) return IA_OK;
+  if (!inv_freq) rot = 0;
+  const int G = nh / nkv, HT = (G + 15) / 16;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  DecFused F;
+  F.src = src;
+  F.split_stride = (size_t)src_rows * row_stride;
+  F.slots = slots;
+  F.inv_freq = inv_freq;
+  F.gsplits = src_splits;
+  F.row_stride = row_stride;
+  F.freq_f64 = freq_f64;
+  F.rot = rot;
+  dim3 grid(B, nkv * HT, num_splits);
+#define DEC_FUSED_LAUNCH(TS)                                                                                        \
+  attn_decode_kernel<true, TS><<<grid, DEC_WAVES * 64, 0, stream>>>(                                                \
+      nullptr, 0, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, part_ml, positions, \
+      block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, F)
+  if (src_dtype == IA_F32) DEC_FUSED_LAUNCH(float);
+  else DEC_FUSED_LAUNCH(bf16_t);
+#undef DEC_FUSED_LAUNCH
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
     attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,

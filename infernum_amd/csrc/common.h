@@ -76,6 +76,39 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
+// ---- rotation of queries and keys: one arithmetic for every kernel that rotates
+// A value that may be a stack of partial sums of a split matrix product: added in the order of their index.
+template <typename TS>
+__device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t split_stride) {
+  float v = to_float(p[0]);
+#pragma unroll 4
+  for (int k = 1; k < splits; ++k) v += to_float(p[k * split_stride]);
+  return v;
+}
+
+// Sine and cosine of position * frequency i.  With a table of float64 frequencies the product is formed in
+// float64 and brought into [-pi, pi] there before the fp32 sine and cosine, so that the angle is good to
+// 3e-7 rad at any position; with a table of fp32 frequencies the product is the fp32 one.
+__device__ __forceinline__ void rope_sincos(int position, const void* __restrict__ table, int table_f64, int i,
+                                            float& sn, float& cs) {
+  if (table_f64) {
+    const double a = (double)position * reinterpret_cast<const double*>(table)[i];
+    const double turns = rint(a * 0.15915494309189535);                 // a / (2 pi)
+    // 2 pi as a double is off by 2.4e-16: times a million turns still far below the fp32 sine's own error
+    const double r = __builtin_fma(-turns, 6.283185307179586, a);
+    sincosf((float)r, &sn, &cs);
+  } else {
+    sincosf((float)position * reinterpret_cast<const float*>(table)[i], &sn, &cs);
+  }
+}
+
+// The rotation of one pair, in one fixed order of roundings (a product, then a fused multiply-add), so that
+// every kernel that rotates gives the same bits.
+__device__ __forceinline__ void rope_pair(float a, float b, float cs, float sn, float& lo, float& hi) {
+  lo = __builtin_fmaf(a, cs, -(b * sn));
+  hi = __builtin_fmaf(a, sn, b * cs);
+}
+
 #define IA_LAUNCH_CHECK()                          \
   do {                                             \
     hipError_t e__ = hipGetLastError();            \

@@ -307,34 +307,7 @@ extern "C" int ia_residual_add(float* h, const void* delta, int act_dtype, int N
 // transposed, [num_pages, nkv, d, page_size], the layout the matrix cores want for the product of
 // probabilities and values; slot = page * page_size + offset.
 // inv_freq == nullptr: no rotation.  slot < 0 or write_kv == 0: nothing is written to pages.
-template <typename TS>
-__device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t split_stride) {
-  float v = to_float(p[0]);
-#pragma unroll 4
-  for (int k = 1; k < splits; ++k) v += to_float(p[k * split_stride]);
-  return v;
-}
-
-// Sine and cosine of position * frequency i (see above), the same arithmetic in every kernel that rotates.
-__device__ __forceinline__ void rope_sincos(int position, const void* __restrict__ table, int table_f64, int i,
-                                            float& sn, float& cs) {
-  if (table_f64) {
-    const double a = (double)position * reinterpret_cast<const double*>(table)[i];
-    const double turns = rint(a * 0.15915494309189535);                 // a / (2 pi)
-    // 2 pi as a double is off by 2.4e-16: times a million turns still far below the fp32 sine's own error
-    const double r = __builtin_fma(-turns, 6.283185307179586, a);
-    sincosf((float)r, &sn, &cs);
-  } else {
-    sincosf((float)position * reinterpret_cast<const float*>(table)[i], &sn, &cs);
-  }
-}
-
-// The rotation of one pair, in one fixed order of roundings (a product, then a fused multiply-add), so that
-// every kernel that rotates gives the same bits.
-__device__ __forceinline__ void rope_pair(float a, float b, float cs, float sn, float& lo, float& hi) {
-  lo = __builtin_fmaf(a, cs, -(b * sn));
-  hi = __builtin_fmaf(a, sn, b * cs);
-}
+// (load_split_sum, rope_sincos and rope_pair are in common.h: the decode attention rotates with them too.)
 
 // grid (N, ceil(heads / 4)), 256 threads: one wave per (token, head), so that a handful of decoded tokens
 // still spread over the GPU; heads are nh queries, then nkv keys, then nkv values.

@@ -426,6 +426,58 @@ def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Te
         "attention_decode")
 
 
+def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot: int,
+                              slots: Optional[torch.Tensor], k_pages: torch.Tensor, v_pages: torch.Tensor,
+                              out: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                              window: int, max_len: int, num_splits: Optional[int] = None) -> None:
+    """:func:`rope_kv_append` and :func:`attention_decode` of B single tokens in one launch (the same bits).
+
+    ``qkv`` is the QKV product of the tokens, [B, (nh + 2 nkv) d] in bf16 or a :class:`SplitSum` of it (with
+    ``slots`` None only the nh query heads are read and no key or value is made: the pages belong to another
+    run of a layer).  Rotated queries stay inside the kernel; the token's key and value go to their slot of the
+    pages and take part in the attention.
+    """
+    split = isinstance(qkv, SplitSum)
+    src = qkv.parts if split else qkv
+    B = out.shape[0]
+    rows, row = (src.shape[1], src.shape[2]) if split else tuple(src.shape)
+    _need(src.is_cuda and src.is_contiguous(), "attention_decode_rotating: qkv must be contiguous on the GPU")
+    _need(src.dtype == (torch.float32 if split else torch.bfloat16),
+          "attention_decode_rotating: bf16 rows or fp32 partial sums")
+    _need(rows >= B and row >= (nh + (2 * nkv if slots is not None else 0)) * d,
+          "attention_decode_rotating: rows of qkv are too few or too short for their heads")
+    _need(k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+          and k_pages.dim() == 4 and k_pages.shape[1] == nkv and k_pages.shape[3] == d and out.is_cuda
+          and tuple(v_pages.shape) == (k_pages.shape[0], nkv, d, k_pages.shape[2]) and tuple(out.shape) == (B, nh * d)
+          and out.is_contiguous() and k_pages.is_contiguous() and v_pages.is_contiguous(),
+          "attention_decode_rotating: bf16 key pages [num_pages, nkv, page_size, d], value pages "
+          "[num_pages, nkv, d, page_size], out [B, nh d]")
+    _dev(src, positions, inv_freq, slots, k_pages, v_pages, out, block_tables)
+    _i32(positions, B, "attention_decode_rotating positions")
+    if slots is not None:
+        _i32(slots, B, "attention_decode_rotating slots")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+          and block_tables.shape[0] >= B, "attention_decode_rotating: one int32 row of block_tables per token")
+    if inv_freq is not None:
+        _need(inv_freq.dtype in (torch.float32, torch.float64) and inv_freq.numel() == rot // 2 and rot % 2 == 0
+              and 0 < rot <= d and inv_freq.is_contiguous(),
+              "attention_decode_rotating: inv_freq must hold rot/2 fp32 or float64 values, rot even and at most d")
+    ps = k_pages.shape[2]
+    _need(ps % 4 == 0, f"attention_decode_rotating: page size {ps} is not a multiple of 4")
+    _need(block_tables.shape[1] * ps >= max_len, "attention_decode_rotating: block_tables are narrower than max_len")
+    splits = num_splits or decode_splits(B, nh, nkv, max_len)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)
+        part_ml = torch.empty(B * nh * splits * 2, dtype=torch.float32, device=out.device)
+    _ok(_attn(d).ia_attn_decode_fused(
+        _p(src), DTYPE_CODE[src.dtype], src.shape[0] if split else 1, rows, row, _p(slots), _p(inv_freq),
+        1 if (inv_freq is not None and inv_freq.dtype == torch.float64) else 0, rot if inv_freq is not None else 0,
+        _p(k_pages), _p(v_pages), _p(out), nh * d, _p(part_o), _p(part_ml), _p(positions), _p(block_tables),
+        block_tables.shape[1], B, nh, nkv, ps, k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _stream()),
+        "attention_decode_rotating")
+
+
 def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
                       tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, d: int, scale: float,

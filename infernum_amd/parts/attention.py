@@ -16,6 +16,7 @@ infernum-cuda/src/inner/weights/generic_impl.rs:153-180).
 from __future__ import annotations
 
 import math
+import os
 from typing import Any, Dict, Mapping, Optional
 
 import torch
@@ -47,6 +48,7 @@ class Attention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         if kernels not in ("auto", "generic"):
             raise ValueError("kernels must be 'auto' or 'generic'")
+        self.rotate_in_attention = os.environ.get("INFERNUM_DECODE_ROTATE", "attention") != "separate"
         self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
                          and K.attention_mfma_available(self.d))
 
@@ -75,6 +77,16 @@ class Attention(Mixer):
         if cache.k_pages is None:
             raise K.KernelError("attention needs pages of the cache")
         g = cache.group
+        if (self.use_mfma and self.rotate_in_attention and ctx.num_decode == x.shape[0]
+                and cache.k_pages.shape[2] % 4 == 0):
+            # every request brings one token: rotation, the write to the pages and attention are one launch
+            w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
+            qkv = linear(x, w, keep_split=True)
+            out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+            K.attention_decode_rotating(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
+                                        ctx.slots[g] if cache.writable else None, cache.k_pages, cache.v_pages, out,
+                                        ctx.block_tables[g], nh, nkv, d, self.scale, self.window, ctx.max_total_len)
+            return linear(out, self.w_o, keep_split=True)
         q_out = None
         if cache.writable:
             qkv = linear(x, self.w_qkv, keep_split=True)

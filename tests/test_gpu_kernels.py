@@ -622,9 +622,59 @@ def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
     assert err <= 2e-2, err
 
 
+@pytest.mark.parametrize("gemm_splits", [0, 1, 3])
+@pytest.mark.parametrize("splits", [None, 1, 5])
+@pytest.mark.parametrize("nh,nkv,d,ps,window,rot", [(8, 2, 128, 16, 0, 128), (6, 3, 48, 4, 0, 48), (32, 8, 128, 16, 0, 128),
+                                                    (40, 2, 64, 8, 0, 32), (5, 5, 16, 16, 0, 0), (2, 1, 256, 64, 0, 256),
+                                                    (8, 2, 128, 16, 100, 128), (4, 1, 96, 4, 17, 96)])
+def test_attention_decode_rotating_equals_rotation_then_attention(nh, nkv, d, ps, window, rot, splits, gemm_splits):
+    """One launch for rotation, write to the pages and attention against the two kernels one after the other:
+    the same attention output and the same pages, bit for bit.  The QKV product comes as bf16 rows
+    (gemm_splits 0) or as fp32 partial sums; the slot of the token's own key holds NaN before the call."""
+    lens = [70, 1, 331, 64, 150, 16, 17, 65]
+    B = len(lens)
+    case = _paged_case(nh, nkv, d, ps, lens, [1] * B, torch.bfloat16, seed=d + nh + 7)
+    g = torch.Generator().manual_seed(5)
+    W = (nh + 2 * nkv) * d
+    if gemm_splits == 0:
+        qkv = torch.randn(B, W, generator=g).to(torch.bfloat16).to(DEV)
+    else:
+        qkv = K().SplitSum(torch.randn(gemm_splits, B, W, generator=g).to(DEV))
+    inv_freq = None
+    if rot:
+        inv_freq = (10000.0 ** (-torch.arange(0, rot, 2, dtype=torch.float64) / rot)).to(DEV)
+    pos = case["positions"]
+    slots = torch.tensor([int(case["bt"][b, (L - 1) // ps]) * ps + (L - 1) % ps for b, L in enumerate(lens)],
+                         dtype=torch.int32, device=DEV)
+    for b, L in enumerate(lens):                   # whatever lies in the token's own slot must not be read
+        pg, off = int(slots[b]) // ps, int(slots[b]) % ps
+        case["kp"][pg, :, off] = float("nan")
+        case["vp"][pg, :, :, off] = float("nan")
+    scale = 1.0 / math.sqrt(d)
+    kp1, vp1 = case["kp"].clone(), case["vp"].clone()
+    q = K().rope_kv_append(qkv if gemm_splits else qkv.clone(), pos, inv_freq, nh, nkv, d, rot, slots, kp1, vp1)
+    want = torch.full((B, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K().attention_decode(q, kp1, vp1, want, pos, case["bt"], nh, nkv, d, scale, window, max(lens), num_splits=splits)
+    assert not want.isnan().any()
+    kp2, vp2 = case["kp"].clone(), case["vp"].clone()
+    out = torch.full_like(want, float("nan"))
+    K().attention_decode_rotating(qkv, pos, inv_freq, rot, slots, kp2, vp2, out, case["bt"], nh, nkv, d, scale, window,
+                                  max(lens), num_splits=splits)
+    assert torch.equal(out, want)
+    assert torch.equal(kp2.view(torch.int16), kp1.view(torch.int16))
+    assert torch.equal(vp2.view(torch.int16), vp1.view(torch.int16))
+    # without slots: queries only, over pages that already hold the token's key and value
+    out2 = torch.full_like(want, float("nan"))
+    kp3, vp3 = kp1.clone(), vp1.clone()
+    K().attention_decode_rotating(qkv, pos, inv_freq, rot, None, kp3, vp3, out2, case["bt"], nh, nkv, d, scale, window,
+                                  max(lens), num_splits=splits)
+    assert torch.equal(out2, want)
+    assert torch.equal(kp3.view(torch.int16), kp1.view(torch.int16)) and torch.equal(vp3.view(torch.int16), vp1.view(torch.int16))
+
+
 @pytest.mark.parametrize("splits", [1, 3])
 def test_attention_mfma_decode_block_table_longer_than_its_lds_slice(splits):
-    """18,000 keys in pages of 4: 4,500 block-table entries, more than the 4,096 the decode kernel keeps in LDS;
+    """18,000 keys in pages of 4: 4,500 block-table entries, more than the 2,048 the decode kernel keeps in LDS;
     the rest is read from global memory.  One far key is loud, so a wrong page shows."""
     nh, nkv, d, ps = 4, 2, 32, 4
     lens = [18000, 5]
