@@ -27,6 +27,23 @@ from .base import (CacheSpec, CacheView, Mixer, PartSpec, Runtime, StepContext, 
 from .linear import linear
 
 
+DECODE_ROTATIONS = ("attention", "separate")
+_decode_rotation = os.environ.get("INFERNUM_DECODE_ROTATE", "attention")
+if _decode_rotation not in DECODE_ROTATIONS:
+    raise ValueError(f"INFERNUM_DECODE_ROTATE={_decode_rotation!r}: one of {DECODE_ROTATIONS}")
+
+
+def set_decode_rotation(name: str) -> str:
+    """Where a step of single tokens rotates queries and keys and writes the pages, for attention parts made
+    from now on: inside the attention kernel ("attention") or in the rotary kernel before it ("separate"; the
+    same bits).  Returns the previous choice."""
+    global _decode_rotation
+    if name not in DECODE_ROTATIONS:
+        raise ValueError(f"decode rotation {name!r}: one of {DECODE_ROTATIONS}")
+    previous, _decode_rotation = _decode_rotation, name
+    return previous
+
+
 class Attention(Mixer):
     graph_safe = True
     def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -48,7 +65,7 @@ class Attention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         if kernels not in ("auto", "generic"):
             raise ValueError("kernels must be 'auto' or 'generic'")
-        self.rotate_in_attention = os.environ.get("INFERNUM_DECODE_ROTATE", "attention") != "separate"
+        self.rotate_in_attention = _decode_rotation == "attention"
         self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
                          and K.attention_mfma_available(self.d))
 

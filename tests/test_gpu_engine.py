@@ -91,6 +91,25 @@ def test_whole_with_the_hand_written_prefill_gemm(models):
     assert worst <= 2e-2 * rms, f"own and library products differ by {worst:.3e} at {where}"
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_tail_one_by_one_rotation_inside_attention_or_before_it(models, name):
+    """Steps of single tokens rotate queries and keys and write the pages inside the attention kernel; with the
+    rotary kernel in front of it instead, every logit has the same bits."""
+    import importlib
+    A = importlib.import_module("infernum_amd.parts.attention")
+    d, cfg, reqs, ref = models[(name, "bfloat16")]
+    got = TT.run_steps(_engine(d, "bfloat16", PAGE[name], 64), TT.trace_tail_one_by_one(reqs, 32))
+    previous = A.set_decode_rotation("separate")
+    try:
+        eng = _engine(d, "bfloat16", PAGE[name], 64)
+        other = TT.run_steps(eng, TT.trace_tail_one_by_one(reqs, 32))
+    finally:
+        A.set_decode_rotation(previous)
+    assert got.keys() == other.keys()
+    for key in got:
+        assert torch.equal(got[key], other[key]), key
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_tail_one_by_one(models, name, dtype):
