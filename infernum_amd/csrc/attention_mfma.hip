@@ -431,12 +431,22 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
     int out_row_stride, int nh, int num_splits) {
   const int b = blockIdx.x / nh, h = blockIdx.x - b * nh, lane = threadIdx.x;
   const size_t rec0 = (size_t)blockIdx.x * num_splits;
+  // the first parts' outputs are asked for together with the statistics, not after them
+  constexpr int PRE = 4, NC = (HD + 63) / 64;
+  float pre[PRE][NC];
+#pragma unroll
+  for (int j = 0; j < PRE; ++j)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int dim = lane + 64 * c;
+      pre[j][c] = (j < num_splits && dim < HD) ? part_o[(rec0 + j) * HD + dim] : 0.f;
+    }
   float M = -INFINITY;
   for (int s = lane; s < num_splits; s += 64) M = fmaxf(M, part_ml[(rec0 + s) * 2]);
   M = wave_max(M);
-  float acc[(HD + 63) / 64];
+  float acc[NC];
 #pragma unroll
-  for (int c = 0; c < (HD + 63) / 64; ++c) acc[c] = 0.f;
+  for (int c = 0; c < NC; ++c) acc[c] = 0.f;
   float L = 0.f;
   for (int s0 = 0; s0 < num_splits; s0 += 64) {
     const int s = s0 + lane;
@@ -447,11 +457,22 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
       wl = wgt * part_ml[(rec0 + s) * 2 + 1];
     }
     const int cnt = (num_splits - s0) < 64 ? (num_splits - s0) : 64;
-    for (int j = 0; j < cnt; ++j) {
+    int j = 0;
+    if (s0 == 0) {
+#pragma unroll
+      for (; j < PRE; ++j) {
+        if (j >= cnt) break;
+        L += __shfl(wl, j, IA_WAVE);
+        const float wj = __shfl(wgt, j, IA_WAVE);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[c] += (wj != 0.f) ? wj * pre[j][c] : 0.f;
+      }
+    }
+    for (; j < cnt; ++j) {
       L += __shfl(wl, j, IA_WAVE);
       const float wj = __shfl(wgt, j, IA_WAVE);
 #pragma unroll
-      for (int c = 0; c < (HD + 63) / 64; ++c) {
+      for (int c = 0; c < NC; ++c) {
         const int dim = lane + 64 * c;
         // every part was written (an empty one holds zeros), so the load needs no guard and does not wait
         const float v = dim < HD ? part_o[(rec0 + s0 + j) * HD + dim] : 0.f;
