@@ -251,8 +251,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
       if (idx < heads_here * half) {
         const int c = idx / half, i = idx - c * half;
         const TS* x = row + (size_t)(g * G + ht * 16 + c) * HD + i;
-        qa[u] = load_split_sum(x, F.gsplits, F.split_stride);
-        qb[u] = load_split_sum(x + half, F.gsplits, F.split_stride);
+        qa[u] = load_split_sum_together(x, F.gsplits, F.split_stride);
+        qb[u] = load_split_sum_together(x + half, F.gsplits, F.split_stride);
       }
     }
   }
@@ -306,10 +306,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
     if (own_key) {
       if (tid < half) {
         const TS* x = row + (size_t)(nh + g) * HD + tid;
-        ka = load_split_sum(x, F.gsplits, F.split_stride);
-        kb = load_split_sum(x + half, F.gsplits, F.split_stride);
+        ka = load_split_sum_together(x, F.gsplits, F.split_stride);
+        kb = load_split_sum_together(x + half, F.gsplits, F.split_stride);
       }
-      if (tid < HD) vv = load_split_sum(row + (size_t)(nh + nkv + g) * HD + tid, F.gsplits, F.split_stride);
+      if (tid < HD) vv = load_split_sum_together(row + (size_t)(nh + nkv + g) * HD + tid, F.gsplits, F.split_stride);
     }
     for (int i = tid; i < half; i += NT) rope_sincos(p, F.inv_freq, F.freq_f64, i, s_sin[i], s_cos[i]);
     // barriers without the fence of __syncthreads(), which would wait for every load in flight: only LDS

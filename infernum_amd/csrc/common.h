@@ -86,6 +86,20 @@ __device__ __forceinline__ float load_split_sum(const TS* p, int splits, size_t 
   return v;
 }
 
+// The same sum with the loads of up to eight parts asked for together, before the first is added (more parts:
+// the loop above).  Same order of additions, so the same bits.
+template <typename TS>
+__device__ __forceinline__ float load_split_sum_together(const TS* p, int splits, size_t split_stride) {
+  if (splits > 8) return load_split_sum(p, splits, split_stride);
+  float x[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) x[k] = k < splits ? to_float(p[k * split_stride]) : 0.f;
+  float v = x[0];
+#pragma unroll
+  for (int k = 1; k < 8; ++k) v = k < splits ? v + x[k] : v;
+  return v;
+}
+
 // Sine and cosine of position * frequency i.  With a table of float64 frequencies the product is formed in
 // float64 and brought into [-pi, pi] there before the fp32 sine and cosine, so that the angle is good to
 // 3e-7 rad at any position; with a table of fp32 frequencies the product is the fp32 one.
