@@ -151,11 +151,12 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
   float* hr = h + (size_t)src * H;
   const TD* dr = delta ? delta + (size_t)src * H : nullptr;
   const bool store = (rows == nullptr) && (delta != nullptr);
-  float4 v[MAXV];
+  float4 v[MAXV], g[MAXV];     // the norm's weights are asked for with the row, not after the sum of squares
 #pragma unroll
   for (int c = 0; c < MAXV; ++c) {
     const int i = (threadIdx.x + c * NT) * 4;
     v[c] = (i < H) ? load4(hr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    g[c] = (i < H) ? load4_any(w, w_dtype, i) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
   if (dr) {
     float4 ds[MAXV];
@@ -215,10 +216,9 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
 #pragma unroll
   for (int c = 0; c < MAXV; ++c) {
     const int i = (threadIdx.x + c * NT) * 4;
-    if (i < H) {
-      const float4 g = load4_any(w, w_dtype, i);
-      store4(o + i, make_float4(v[c].x * inv * g.x, v[c].y * inv * g.y, v[c].z * inv * g.z, v[c].w * inv * g.w));
-    }
+    if (i < H)
+      store4(o + i, make_float4(v[c].x * inv * g[c].x, v[c].y * inv * g[c].y, v[c].z * inv * g[c].z,
+                                v[c].w * inv * g[c].w));
   }
 }
 
