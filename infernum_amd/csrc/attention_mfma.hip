@@ -98,26 +98,31 @@ struct DecGeom {                 // what does not change from tile to tile
   const uint16_t* new_v;         // [HD] in LDS
 };
 
+// POW2: the page size is a power of two (a shift and a mask; a division by a size known only at run time costs
+// some twenty vector instructions, and the compiler would work out both and pick one).
+template <bool POW2>
 __device__ __forceinline__ int dec_page(const DecGeom& G, int key) {
-  const int idx = G.ps_shift >= 0 ? key >> G.ps_shift : key / G.ps;
+  const int idx = POW2 ? key >> G.ps_shift : key / G.ps;
   const int rel = idx - G.bt_first;
   return (unsigned)rel < (unsigned)G.bt_count ? G.bt_lds[rel] : G.bt_global[idx];
 }
+template <bool POW2>
 __device__ __forceinline__ int dec_offset(const DecGeom& G, int key) {
-  return G.ps_shift >= 0 ? key & (G.ps - 1) : key % G.ps;
+  return POW2 ? key & (G.ps - 1) : key % G.ps;
 }
 
+template <bool POW2>
 __device__ __forceinline__ void dec_load(const DecGeom& G, int t0, int j, int qd, DecTile& T) {
   const int key = t0 + j;
   const int keyc = key < G.key_lo ? G.key_lo : (key > G.key_hi ? G.key_hi : key);
-  const int page = dec_page(G, keyc);
+  const int page = dec_page<POW2>(G, keyc);
   const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
-  load_row_operand(G.k_base + (size_t)(page_ok ? page : 0) * G.page_elems + (size_t)dec_offset(G, keyc) * HD, qd, T.k);
+  load_row_operand(G.k_base + (size_t)(page_ok ? page : 0) * G.page_elems + (size_t)dec_offset<POW2>(G, keyc) * HD, qd, T.k);
   const int kg = t0 + 4 * qd;    // this lane brings the values of the keys kg .. kg+3 (one quad, one page)
   const int kgc = kg < G.key_lo ? (G.key_lo & ~3) : (kg > G.key_hi ? (G.key_hi & ~3) : kg);
-  const int pagev = dec_page(G, kgc);
+  const int pagev = dec_page<POW2>(G, kgc);
   const bool pagev_ok = (unsigned)pagev < (unsigned)G.num_pages;
-  const uint16_t* vq = G.v_base + (size_t)(pagev_ok ? pagev : 0) * G.page_elems + dec_offset(G, kgc);
+  const uint16_t* vq = G.v_base + (size_t)(pagev_ok ? pagev : 0) * G.page_elems + dec_offset<POW2>(G, kgc);
   // keep the values of keys key_lo .. key_hi, zero the others (16 bits each)
   uint32_t mlo = 0u, mhi = 0u;
   if (kg == kgc && pagev_ok) {
@@ -214,7 +219,7 @@ struct DecFused {
 // FUSED: q is not read; every workgroup rotates the queries of its heads into LDS, the workgroups whose keys
 // include the token's own also make its key and value, use them from LDS (the loads from the page are replaced
 // in registers) and one of them (the first tile of heads) writes them to the page.
-template <bool FUSED, typename TS>
+template <bool FUSED, typename TS, bool POW2>
 __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_decode_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, uint16_t* k_pages, uint16_t* v_pages,
     uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -282,8 +287,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
   // the slice of the block table that this workgroup's keys need
   {
     const int k_from = ta * 16 < lo0 ? lo0 : ta * 16, k_to = tb * 16 - 1 > p ? p : tb * 16 - 1;
-    const int first = geo.ps_shift >= 0 ? k_from >> geo.ps_shift : k_from / ps;
-    const int last = geo.ps_shift >= 0 ? k_to >> geo.ps_shift : k_to / ps;
+    const int first = POW2 ? k_from >> geo.ps_shift : k_from / ps;
+    const int last = POW2 ? k_to >> geo.ps_shift : k_to / ps;
     int count = ta < tb ? last - first + 1 : 0;
     if (count > DEC_BT_LDS) count = DEC_BT_LDS;
     geo.bt_first = first;
@@ -316,7 +321,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
     // traffic has to be through
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    if (t < tb) dec_load(geo, t * 16, j, qd, A);             // the first tile's loads fly during the rotation
+    if (t < tb) dec_load<POW2>(geo, t * 16, j, qd, A);             // the first tile's loads fly during the rotation
 #pragma unroll
     for (int u = 0; u < QPT; ++u) {
       const int idx = tid + u * NT;
@@ -354,18 +359,18 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
     if (col_ok) load_row_operand(q + (size_t)b * q_row_stride + (size_t)h * HD, qd, qreg);
     else zero_row_operand(qreg);
     __syncthreads();
-    if (t < tb) dec_load(geo, t * 16, j, qd, A);
+    if (t < tb) dec_load<POW2>(geo, t * 16, j, qd, A);
   }
   // two tiles in flight: the loads of the next tile of this wave are issued before this one is worked on
   while (t < tb) {
     const bool more1 = t + DEC_WAVES < tb;
-    if (more1) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, B);
+    if (more1) dec_load<POW2>(geo, (t + DEC_WAVES) * 16, j, qd, B);
     dec_finish(geo, t * 16, j, qd, A);
     dec_compute(t * 16, A, qreg, pos, lo0, qd, scale_log2, o, m, l);
     t += DEC_WAVES;
     if (!more1) break;
     const bool more2 = t + DEC_WAVES < tb;
-    if (more2) dec_load(geo, (t + DEC_WAVES) * 16, j, qd, A);
+    if (more2) dec_load<POW2>(geo, (t + DEC_WAVES) * 16, j, qd, A);
     dec_finish(geo, t * 16, j, qd, B);
     dec_compute(t * 16, B, qreg, pos, lo0, qd, scale_log2, o, m, l);
     t += DEC_WAVES;
@@ -509,7 +514,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 #define PF_VROW 40              // bf16 per dim row of V^T in LDS (32 keys + 8 of padding)
 #define PF_LAZY 6.0f            // log2 of how far the running maximum may run ahead of the reference point
 
-template <int CT, int HGW>
+template <int CT, int HGW, bool POW2>
 __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
@@ -588,8 +593,9 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
   int pgk[KPT], pgv;
   // page size: a shift when it is a power of two (the usual case), a division otherwise
   const int ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;
-  auto page_index = [&](int key) { return ps_shift >= 0 ? key >> ps_shift : key / ps; };
-  auto page_offset = [&](int key) { return ps_shift >= 0 ? key & (ps - 1) : key % ps; };
+  // a page size that is a power of two (POW2) needs a shift and a mask, no division
+  auto page_index = [&](int key) { return POW2 ? key >> ps_shift : key / ps; };
+  auto page_offset = [&](int key) { return POW2 ? key & (ps - 1) : key % ps; };
   const size_t page_elems = (size_t)nkv * ps * HD;                 // elements of one page (all heads)
   // what does not change from tile to tile
   int k_row[KPT], k_col[KPT];
@@ -823,9 +829,13 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
   const int G = nh / nkv, HT = (G + 15) / 16;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(B, nkv * HT, num_splits);
-  attn_decode_kernel<false, bf16_t><<<grid, DEC_WAVES * 64, 0, stream>>>(
-      (const uint16_t*)q, q_row_stride, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o,
-      part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{});
+#define DEC_LAUNCH(P2)                                                                                             \
+  attn_decode_kernel<false, bf16_t, P2><<<grid, DEC_WAVES * 64, 0, stream>>>(                                        \
+      (const uint16_t*)q, q_row_stride, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, \
+      part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{})
+  if ((ps & (ps - 1)) == 0) DEC_LAUNCH(true);
+  else DEC_LAUNCH(false);
+#undef DEC_LAUNCH
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
     attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,
@@ -865,12 +875,18 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
   F.freq_f64 = freq_f64;
   F.rot = rot;
   dim3 grid(B, nkv * HT, num_splits);
-#define DEC_FUSED_LAUNCH(TS)                                                                                        \
-  attn_decode_kernel<true, TS><<<grid, DEC_WAVES * 64, 0, stream>>>(                                                \
+#define DEC_FUSED_LAUNCH(TS, P2)                                                                                    \
+  attn_decode_kernel<true, TS, P2><<<grid, DEC_WAVES * 64, 0, stream>>>(                                            \
       nullptr, 0, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, part_ml, positions, \
       block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, F)
-  if (src_dtype == IA_F32) DEC_FUSED_LAUNCH(float);
-  else DEC_FUSED_LAUNCH(bf16_t);
+  const bool pow2 = (ps & (ps - 1)) == 0;
+  if (src_dtype == IA_F32) {
+    if (pow2) DEC_FUSED_LAUNCH(float, true);
+    else DEC_FUSED_LAUNCH(float, false);
+  } else {
+    if (pow2) DEC_FUSED_LAUNCH(bf16_t, true);
+    else DEC_FUSED_LAUNCH(bf16_t, false);
+  }
 #undef DEC_FUSED_LAUNCH
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
@@ -910,10 +926,15 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   if ((long long)nkv * HC > 65535) return IA_ERR_UNSUPPORTED;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(num_tiles, nkv * HC);
-#define PF_LAUNCH(C, W)                                                                                           \
-  attn_prefill_kernel<C, W><<<grid, 4 * W * 64, 0, stream>>>(                                                     \
+#define PF_LAUNCH_P(C, W, P2)                                                                                     \
+  attn_prefill_kernel<C, W, P2><<<grid, 4 * W * 64, 0, stream>>>(                                                 \
       (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
       out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window)
+#define PF_LAUNCH(C, W)                      \
+  do {                                       \
+    if ((ps & (ps - 1)) == 0) PF_LAUNCH_P(C, W, true); \
+    else PF_LAUNCH_P(C, W, false);           \
+  } while (0)
   if (HGW == 1) PF_LAUNCH(1, 1);
   else if (HGW == 2) PF_LAUNCH(1, 2);
   else {
@@ -924,6 +945,7 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
 #endif
   }
 #undef PF_LAUNCH
+#undef PF_LAUNCH_P
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
