@@ -607,7 +607,8 @@ def test_prefill_heads_per_workgroup():
 
 @pytest.mark.parametrize("splits", [None, 1, 3, 7])
 @pytest.mark.parametrize("nh,nkv,d,ps,window", [(8, 2, 128, 16, 0), (6, 3, 48, 4, 0), (32, 8, 128, 16, 0), (40, 2, 64, 8, 0),
-                                                (5, 5, 16, 16, 0), (2, 1, 256, 64, 0), (8, 2, 128, 16, 100), (4, 1, 96, 4, 17)])
+                                                (5, 5, 16, 16, 0), (2, 1, 256, 64, 0), (8, 2, 128, 16, 100), (4, 1, 96, 4, 17),
+                                                (3, 1, 80, 12, 0), (6, 2, 64, 20, 33)])      # pages of 12 and 20: no power of two
 def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
     lens = [70, 1, 331, 64, 150, 16, 17]
     q_lens = [1] * len(lens)
@@ -626,7 +627,8 @@ def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
 @pytest.mark.parametrize("splits", [None, 1, 5])
 @pytest.mark.parametrize("nh,nkv,d,ps,window,rot", [(8, 2, 128, 16, 0, 128), (6, 3, 48, 4, 0, 48), (32, 8, 128, 16, 0, 128),
                                                     (40, 2, 64, 8, 0, 32), (5, 5, 16, 16, 0, 0), (2, 1, 256, 64, 0, 256),
-                                                    (8, 2, 128, 16, 100, 128), (4, 1, 96, 4, 17, 96)])
+                                                    (8, 2, 128, 16, 100, 128), (4, 1, 96, 4, 17, 96),
+                                                    (3, 1, 80, 12, 0, 80), (6, 2, 64, 20, 33, 64)])   # pages: no power of two
 def test_attention_decode_rotating_equals_rotation_then_attention(nh, nkv, d, ps, window, rot, splits, gemm_splits):
     """One launch for rotation, write to the pages and attention against the two kernels one after the other:
     the same attention output and the same pages, bit for bit.  The QKV product comes as bf16 rows
