@@ -623,7 +623,7 @@ def test_attention_mfma_decode(nh, nkv, d, ps, window, splits):
     assert err <= 2e-2, err
 
 
-@pytest.mark.parametrize("gemm_splits", [0, 1, 3])
+@pytest.mark.parametrize("gemm_splits", [0, 1, 3, 10])   # above eight parts the sums are read one after the other
 @pytest.mark.parametrize("splits", [None, 1, 5])
 @pytest.mark.parametrize("nh,nkv,d,ps,window,rot", [(8, 2, 128, 16, 0, 128), (6, 3, 48, 4, 0, 48), (32, 8, 128, 16, 0, 128),
                                                     (40, 2, 64, 8, 0, 32), (5, 5, 16, 16, 0, 0), (2, 1, 256, 64, 0, 256),
