@@ -98,7 +98,7 @@ class Attention(Mixer):
         if cache.k_pages is None:
             raise K.KernelError("attention needs pages of the cache")
         g = cache.group
-        if (self.use_mfma and self.rotate_in_attention and ctx.num_decode == x.shape[0]
+        if (self.use_mfma and self.rotate_in_attention and 0 < ctx.num_decode == x.shape[0]
                 and x.shape[0] <= ROTATE_IN_ATTENTION_UP_TO and cache.k_pages.shape[2] % 4 == 0):
             # every request brings one token: rotation, the write to the pages and attention are one launch
             w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
