@@ -175,6 +175,14 @@ class CacheManager:
         """The request's number in the native bookkeeping."""
         return self._id(req)
 
+    def request_ids(self, reqs: Sequence[Hashable]) -> List[int]:
+        """The numbers of several requests, all admitted."""
+        ids = self._ids
+        try:
+            return [ids[r] for r in reqs]
+        except KeyError as e:
+            raise PageError(f"request {e.args[0]!r} is not admitted") from None
+
     # ---- requests -------------------------------------------------------------
     def has(self, req: Hashable) -> bool:
         return req in self._ids
@@ -236,20 +244,22 @@ class CacheManager:
             self._h, n, (ctypes.c_int64 * max(n, 1))(*[i or 0 for i in ids]),
             (ctypes.c_int * max(n, 1))(*[int(i is not None) for i in ids]), (ctypes.c_int * max(n, 1))(*q_lens)) == 1
 
-    def _step_arrays(self, reqs: Sequence[Hashable], q_lens: Sequence[int]):
+    def step_arrays(self, reqs: Sequence[Hashable], q_lens: Sequence[int]):
+        """A step's requests (all admitted) and token counts as the native calls take them; ``reserve_step`` and
+        ``commit_step`` of one step can share them."""
         n = len(reqs)
-        return n, (ctypes.c_int64 * max(n, 1))(*[self._id(r) for r in reqs]), (ctypes.c_int * max(n, 1))(*q_lens)
+        return n, (ctypes.c_int64 * max(n, 1))(*self.request_ids(reqs)), (ctypes.c_int * max(n, 1))(*q_lens)
 
-    def reserve_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int]) -> bool:
+    def reserve_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int], arrays=None) -> bool:
         """Pages for ``q_lens[i]`` more tokens of every ``reqs[i]`` (all admitted), or nothing at all."""
-        rc = self._lib.ia_cache_reserve_step(self._h, *self._step_arrays(reqs, q_lens))
+        rc = self._lib.ia_cache_reserve_step(self._h, *(arrays or self.step_arrays(reqs, q_lens)))
         if rc == native.HOST_ERROR:
             self._fail()
         return rc == 1
 
-    def commit_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int]) -> None:
+    def commit_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int], arrays=None) -> None:
         """``commit`` for every request of a step."""
-        if self._lib.ia_cache_commit_step(self._h, *self._step_arrays(reqs, q_lens)) != 0:
+        if self._lib.ia_cache_commit_step(self._h, *(arrays or self.step_arrays(reqs, q_lens))) != 0:
             self._fail()
         self._poison()
 

@@ -70,19 +70,27 @@ class PackedStep:
 
 
 def check_entries(entries: Sequence[StepEntry], vocab_size: int, max_tokens: int) -> None:
-    seen = set()
+    total = 0
     for e in entries:
-        if e.request in seen:
-            raise StepError(f"request {e.request!r} stands twice in one step")
-        seen.add(e.request)
-        if len(e.tokens) == 0:
+        toks = e.tokens
+        n = len(toks)
+        total += n
+        if n == 1:                              # the common case of a decoding request, without min() and max()
+            if not 0 <= toks[0] < vocab_size:
+                raise StepError(f"request {e.request!r}: token id outside the vocabulary [0, {vocab_size})")
+        elif n == 0:
             raise StepError(f"request {e.request!r} brings no tokens")
-        for w in e.want:
-            if not 0 <= w < len(e.tokens):
-                raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
-        if min(e.tokens) < 0 or max(e.tokens) >= vocab_size:
+        elif min(toks) < 0 or max(toks) >= vocab_size:
             raise StepError(f"request {e.request!r}: token id outside the vocabulary [0, {vocab_size})")
-    total = sum(len(e.tokens) for e in entries)
+        for w in e.want:
+            if not 0 <= w < n:
+                raise StepError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
+    if len({e.request for e in entries}) != len(entries):
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} stands twice in one step")
+            seen.add(e.request)
     if total > max_tokens:
         raise StepError(f"a step of {total} tokens is above max_tokens_per_step {max_tokens}")
 
@@ -96,25 +104,37 @@ def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optio
     G = len(cache.groups)
     q_lens_in = [len(e.tokens) for e in entries]
     want_counts = [len(e.want) for e in entries]
-    tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=sum(q_lens_in))
-    wants = np.fromiter((w for e in entries for w in e.want), dtype=np.int32, count=sum(want_counts))
+    if max(q_lens_in, default=0) == 1:       # a step of single tokens: no nested walk
+        flat_tokens = [e.tokens[0] for e in entries]
+    else:
+        flat_tokens = [t for e in entries for t in e.tokens]
+    flat_wants = [w for e in entries for w in e.want]
     S = 8 + 2 * G
-    meta = np.empty(7 + 2 * S + G + 2 * n, dtype=np.int32)
+    meta_len = 7 + 2 * S + G + 2 * n
+    meta = (ctypes.c_int32 * meta_len)()
     lib, h = native.lib(), cache.native_handle()
-    i32 = ctypes.POINTER(ctypes.c_int32)
+    # short lists go over as ctypes arrays (a microsecond each); a prompt's many tokens through numpy
+    if len(flat_tokens) <= 256:
+        tokens = (ctypes.c_int32 * max(len(flat_tokens), 1))(*flat_tokens)
+    else:
+        keep = np.array(flat_tokens, dtype=np.int32)
+        tokens = keep.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
     rc = lib.ia_cache_pack_step(
-        h, n, (ctypes.c_int64 * max(n, 1))(*[cache.request_id(e.request) for e in entries]),
-        (ctypes.c_int * max(n, 1))(*q_lens_in), tokens.ctypes.data_as(i32), (ctypes.c_int * max(n, 1))(*want_counts),
-        wants.ctypes.data_as(i32), int(bt_width or 0), PREFILL_TILE_ROWS, meta.ctypes.data_as(i32), int(meta.size))
+        h, n, (ctypes.c_int64 * max(n, 1))(*cache.request_ids([e.request for e in entries])),
+        (ctypes.c_int * max(n, 1))(*q_lens_in), tokens, (ctypes.c_int * max(n, 1))(*want_counts),
+        (ctypes.c_int32 * max(len(flat_wants), 1))(*flat_wants), int(bt_width or 0), PREFILL_TILE_ROWS, meta, meta_len)
     if rc != 0:
         cache._fail()
-    total, num_decode, num_tiles, num_rows = (int(v) for v in meta[:4])
-    offsets = [int(v) for v in meta[7:7 + S]]
-    sizes = [int(v) for v in meta[7 + S:7 + 2 * S]]
-    cols = [int(v) for v in meta[7 + 2 * S:7 + 2 * S + G]]
-    order = [int(v) for v in meta[7 + 2 * S + G:7 + 2 * S + G + n]]
-    ctx_lens = [int(v) for v in meta[7 + 2 * S + G + n:7 + 2 * S + G + 2 * n]]
-    host = np.ctypeslib.as_array(lib.ia_cache_packed(h), shape=(total,)).copy()
+    m = meta[:]
+    total, num_decode, num_tiles, num_rows = m[:4]
+    offsets = m[7:7 + S]
+    sizes = m[7 + S:7 + 2 * S]
+    cols = m[7 + 2 * S:7 + 2 * S + G]
+    order = m[7 + 2 * S + G:7 + 2 * S + G + n]
+    ctx_lens = m[7 + 2 * S + G + n:7 + 2 * S + G + 2 * n]
+    buf = (ctypes.c_int32 * total)()         # a copy of the native buffer, which the next step overwrites
+    ctypes.memmove(buf, lib.ia_cache_packed(h), total * 4)
+    host = np.frombuffer(buf, dtype=np.int32)
     batch = [entries[i] for i in order]
     return PackedStep(host, offsets, sizes, [(n, c) for c in cols], batch, [q_lens_in[i] for i in order], ctx_lens,
                       num_decode, num_tiles, num_rows)

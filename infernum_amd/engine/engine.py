@@ -126,7 +126,8 @@ class Engine:
         for r in reqs:
             if not cache.has(r):
                 cache.admit(r)
-        if not cache.reserve_step(reqs, q_lens):
+        arrays = cache.step_arrays(reqs, q_lens)        # once for the reservation and the commit
+        if not cache.reserve_step(reqs, q_lens, arrays):
             raise OutOfPages("the pages this step was checked for are gone")   # step_fits said they were there
         if all(len(e.tokens) == 1 for e in entries):
             logits = self._decode_step(entries)
@@ -134,7 +135,7 @@ class Engine:
             packed = pack_step(cache, entries)
             ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
             logits = self.model.forward(ctx, self.views)
-        cache.commit_step(reqs, q_lens)
+        cache.commit_step(reqs, q_lens, arrays)
         self.steps_run += 1
         return logits
 
