@@ -43,7 +43,7 @@ CORE_SOURCES = [
     "attention_generic.hip",
     "sampling.hip",
 ]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
 HOST_SOURCES = ["host_core.cpp"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]

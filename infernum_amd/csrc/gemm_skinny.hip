@@ -296,3 +296,53 @@ extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dty
   if (out_dtype == IA_F32) return launch_join<float>(workspace, (float*)C, M, N, splits, epilogue, stream);
   return launch_join<uint16_t>(workspace, (uint16_t*)C, M, N, splits, epilogue, stream);
 }
+
+// ---- the same product for callers that cannot allocate: the workspace is an array of this library ----------
+#include <mutex>
+#include "no_alloc.h"
+
+#define IA_MAX_DEVICES 64
+
+// Partial sums of a split product.  In host code this name only stands for the array (it is no device address);
+// hipGetSymbolAddress gives the address on the current device, and host code uses that and nothing else.
+static __device__ __align__(256) float scratch[IA_SKINNY_SCRATCH_FLOATS];
+static float* scratch_on_device[IA_MAX_DEVICES];      // each GPU has its own copy of the array at its own address
+static std::mutex scratch_lock;
+
+static int scratch_of_current_device(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= IA_MAX_DEVICES) return IA_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (scratch_on_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return IA_ERR_BAD_ARG;
+    scratch_on_device[dev] = static_cast<float*>(p);
+  }
+  *out = scratch_on_device[dev];
+  return IA_OK;
+}
+
+extern "C" size_t ia_gemm_skinny_no_alloc_capacity(void) { return IA_SKINNY_SCRATCH_FLOATS; }
+
+extern "C" size_t ia_gemm_skinny_no_alloc_needs(int M, int N, int K, int epilogue) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int splits = skinny_splits(N, K);
+  (void)epilogue;      // with one part the activation is done in the product's own epilogue, without a workspace
+  return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N : 0;
+}
+
+extern "C" int ia_gemm_skinny_no_alloc(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
+                                       int epilogue, hipStream_t stream) {
+  if (X == nullptr || W == nullptr || C == nullptr) return IA_ERR_BAD_ARG;
+  if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
+  const size_t needs = ia_gemm_skinny_no_alloc_needs(M, N, K, epilogue);
+  if (needs > IA_SKINNY_SCRATCH_FLOATS) return IA_ERR_SCRATCH_TOO_SMALL;
+  float* ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc != IA_OK) return rc;
+  return ia_gemm_skinny(X, W, C, out_dtype, M, N, K, epilogue, ws, IA_SKINNY_SCRATCH_FLOATS, stream);
+}
