@@ -257,6 +257,14 @@ class CacheManager:
             self._fail()
         return rc == 1
 
+    def unreserve_step(self, reqs: Sequence[Hashable]) -> None:
+        """A step whose pages were reserved did not run: the pages beyond what each request's stored tokens
+        need go back to the pools."""
+        n = len(reqs)
+        if self._lib.ia_cache_unreserve_step(self._h, n, (ctypes.c_int64 * max(n, 1))(*self.request_ids(reqs))) != 0:
+            self._fail()
+        self._poison()
+
     def commit_step(self, reqs: Sequence[Hashable], q_lens: Sequence[int], arrays=None) -> None:
         """``commit`` for every request of a step."""
         if self._lib.ia_cache_commit_step(self._h, *(arrays or self.step_arrays(reqs, q_lens))) != 0:

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "ia_cache_step_fits": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int), POINTER(c_int)]),
     "ia_cache_reserve_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int)]),
     "ia_cache_commit_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int)]),
+    "ia_cache_unreserve_step": (c_int, [c_void_p, c_int, POINTER(c_int64)]),
     "ia_cache_check": (c_int, [c_void_p]),
     "ia_cache_token_slots": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, POINTER(c_int32)]),
     "ia_cache_pack_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int), POINTER(c_int32), POINTER(c_int),

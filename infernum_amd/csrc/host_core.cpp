@@ -357,6 +357,31 @@ int ia_cache_reserve_step(void* h, int n, const int64_t* reqs, const int* q_lens
   return 1;
 }
 
+// undo of ia_cache_reserve_step for a step that did not run: pages beyond what each request's stored tokens
+// need go back to the pools (ia_cache_last_freed names them)
+int ia_cache_unreserve_step(void* h, int n, const int64_t* reqs) {
+  Cache* c = static_cast<Cache*>(h);
+  for (int i = 0; i < n; ++i)
+    if (!c->admitted(reqs[i])) return c->fail(req_name(reqs[i]) + " is not admitted");
+  c->last_freed.clear();
+  for (int i = 0; i < n; ++i)
+    for (size_t gi = 0; gi < c->groups.size(); ++gi) {
+      Group& g = c->groups[gi];
+      Table& t = g.tables[reqs[i]];
+      const size_t keep = (size_t)g.pages_for(t.num_tokens);
+      while (t.pages.size() > keep) {
+        const int p = t.pages.back();
+        t.pages.pop_back();
+        if (p != NO_PAGE) {
+          g.pool.release(p);
+          c->last_freed.push_back((int)gi);
+          c->last_freed.push_back(p);
+        }
+      }
+    }
+  return 0;
+}
+
 // ia_cache_commit for every entry of a step; ia_cache_last_freed then covers all of them.  Entries before
 // a failing one stay committed.
 int ia_cache_commit_step(void* h, int n, const int64_t* reqs, const int* q_lens) {

@@ -28,6 +28,12 @@ class OutOfPages(RuntimeError):
     """The pool has too few free pages (or state slots) for this step; nothing was changed."""
 
 
+# Recorded decode steps kept at a time.  Each holds its own logits ([requests, vocabulary] fp32) and its
+# inputs; in continuous batching the number of live requests takes every value up to the largest batch, times
+# a handful of table widths, so the table is bounded and the shape used longest ago makes room.
+MAX_RECORDED_STEPS = 64
+
+
 class _DecodeGraph:
     """A recorded decode step of one shape: its int32 inputs, the recorded launches, its logits."""
 
@@ -57,6 +63,7 @@ class Engine:
         self._shape_seen: Dict[tuple, int] = {}
         self._graph_pool = None
         self.graph_replays = 0
+        self.max_recorded_steps = MAX_RECORDED_STEPS
 
     # ---- building ------------------------------------------------------------------
     @staticmethod
@@ -123,18 +130,29 @@ class Engine:
             raise OutOfPages(f"not enough free pages or state slots for a step of {total} tokens")
         cache = self.cache
         reqs, q_lens = [e.request for e in entries], [len(e.tokens) for e in entries]
-        for r in reqs:
-            if not cache.has(r):
-                cache.admit(r)
-        arrays = cache.step_arrays(reqs, q_lens)        # once for the reservation and the commit
-        if not cache.reserve_step(reqs, q_lens, arrays):
-            raise OutOfPages("the pages this step was checked for are gone")   # step_fits said they were there
-        if all(len(e.tokens) == 1 for e in entries):
-            logits = self._decode_step(entries)
-        else:
-            packed = pack_step(cache, entries)
-            ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
-            logits = self.model.forward(ctx, self.views)
+        fresh = [r for r in reqs if not cache.has(r)]
+        for r in fresh:
+            cache.admit(r)
+        reserved = False
+        try:
+            arrays = cache.step_arrays(reqs, q_lens)        # once for the reservation and the commit
+            if not cache.reserve_step(reqs, q_lens, arrays):
+                raise OutOfPages("the pages this step was checked for are gone")   # step_fits said they were there
+            reserved = True
+            if all(n == 1 for n in q_lens):
+                logits = self._decode_step(entries)
+            else:
+                packed = pack_step(cache, entries)
+                ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
+                logits = self.model.forward(ctx, self.views)
+        except BaseException:
+            # the step did not run to its end: requests that came with it leave again, the others give back
+            # the pages that were reserved for it; what earlier steps stored stays as it was
+            for r in fresh:
+                cache.release(r)
+            if reserved:
+                cache.unreserve_step([r for r in reqs if r not in fresh])
+            raise
         cache.commit_step(reqs, q_lens, arrays)
         self.steps_run += 1
         return logits
@@ -150,6 +168,7 @@ class Engine:
         key = (len(entries), width, packed.num_logit_rows)
         g = self._graphs.get(key)
         if g is not None:
+            self._graphs[key] = self._graphs.pop(key)       # most recently used last
             g.inputs.copy_(torch.from_numpy(packed.host))
             g.graph.replay()
             self.graph_replays += 1
@@ -162,6 +181,10 @@ class Engine:
         if not self.use_graphs or seen < 1:
             return self.model.forward(ctx, self.views)
         # second time this shape comes: record it (kernels were loaded by the first, eager run)
+        while len(self._graphs) >= self.max_recorded_steps:
+            oldest = next(iter(self._graphs))
+            del self._graphs[oldest]                        # its memory returns to the graphs' pool
+            self._shape_seen.pop(oldest, None)
         torch.cuda.synchronize(self.rt.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self._graph_pool):

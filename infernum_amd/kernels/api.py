@@ -69,6 +69,8 @@ class on_current_stream:
 
     def __enter__(self):
         global _fixed_stream
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: infernum_amd runs on a gfx950 GPU only (there is no CPU fallback)")
         self._before = _fixed_stream
         _fixed_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         return self

@@ -1,7 +1,9 @@
 """Random weights from a configuration and a seed.
 
-Every tensor is drawn from its own generator, seeded from (seed, tensor name),
-so values do not depend on the order in which tensors are made.  Matrices and
+Every tensor is a function of (seed, tensor name, element index) alone, so
+values depend neither on the order in which tensors are made nor on the device
+that makes them: a model filled on the GPU and a folder written on the host
+from the same seed hold the same numbers.  Matrices and
 the embedding are N(0, std), norm weights are what the spec says (ones, or a
 uniform range).  ``write_random_model`` writes a model folder (config.json,
 model.safetensors) that loads like any other; ``random_weights_on_device``
@@ -25,22 +27,80 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
+# ---- one generator for the CPU and the GPU -------------------------------------------------------------
+# Element i of a tensor gets the 32-bit number hash(key of (seed, name), i): integer operations only, which
+# give the same bits on every device.  A normal deviate is read from a table of 65,537 quantiles of the
+# standard normal distribution (made once on the host, without a device's mathematical functions) with a
+# linear step between two entries: a gather, a subtraction, a product by a multiple of 2^-16 and an addition
+# in fp32, each rounded the same way everywhere.  The distribution is the normal one with a density that is
+# constant within each 1/65,536 of probability, cut at 4.9 standard deviations.
+_MASK32 = 0xFFFFFFFF
+_CHUNK = 1 << 24                      # elements made at a time (bounds the temporaries)
+_quantiles: Dict[torch.device, torch.Tensor] = {}
+
+
+def _mix32(x: torch.Tensor) -> torch.Tensor:
+    """A 32-bit integer hash on values kept in int64 (the low 32 bits of a product survive its wrap)."""
+    x = x ^ (x >> 16)
+    x = (x * 0x7FEB352D) & _MASK32
+    x = x ^ (x >> 15)
+    x = (x * 0x846CA68B) & _MASK32
+    return x ^ (x >> 16)
+
+
+def _uniform_bits(n: int, first: int, key: int, device: torch.device) -> torch.Tensor:
+    """32 random bits (int64 in [0, 2^32)) for elements first .. first+n-1 of the tensor with this key."""
+    k0, k1 = key & _MASK32, (key >> 32) & _MASK32
+    i = torch.arange(first, first + n, dtype=torch.int64, device=device)
+    x = _mix32((i & _MASK32) ^ k0)
+    x = _mix32(((x + k1) & _MASK32) ^ (i >> 32))
+    return x
+
+
+def _normal_quantiles(device: torch.device) -> torch.Tensor:
+    t = _quantiles.get(device)
+    if t is None:
+        from statistics import NormalDist
+        inv = NormalDist().inv_cdf
+        n = 65536
+        q = [inv(1.0 / (16 * n))] + [inv(k / n) for k in range(1, n)] + [-inv(1.0 / (16 * n))]
+        t = _quantiles[device] = torch.tensor(q, dtype=torch.float64).to(torch.float32).to(device)
+    return t
+
+
+def _standard_normal(n: int, first: int, key: int, device: torch.device) -> torch.Tensor:
+    u = _uniform_bits(n, first, key, device)
+    table = _normal_quantiles(device)
+    idx = u >> 16
+    frac = (u & 0xFFFF).to(torch.float32) * (1.0 / 65536.0)
+    lo = table[idx]
+    step = table[idx + 1] - lo
+    step.mul_(frac)                     # a product, then a sum: two roundings, never a fused one
+    return lo.add_(step)
+
+
 def draw(spec: WeightSpec, seed: int, name: str, device: torch.device) -> torch.Tensor:
-    """An fp32 tensor of the spec's shape on ``device``."""
-    gen = torch.Generator(device=device)
-    gen.manual_seed(_tensor_seed(seed, name))
+    """An fp32 tensor of the spec's shape on ``device``: the same bits on every device."""
     kind = spec.init[0]
-    if kind == "normal":
-        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
-        return t.normal_(0.0, float(spec.init[1]), generator=gen)
-    if kind == "uniform":
-        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
-        return t.uniform_(float(spec.init[1]), float(spec.init[2]), generator=gen)
     if kind == "ones":
         return torch.ones(spec.shape, dtype=torch.float32, device=device)
     if kind == "zeros":
         return torch.zeros(spec.shape, dtype=torch.float32, device=device)
-    raise ValueError(f"unknown init {spec.init!r} for {name}")
+    if kind not in ("normal", "uniform"):
+        raise ValueError(f"unknown init {spec.init!r} for {name}")
+    key = _tensor_seed(seed, name)
+    out = torch.empty(spec.shape, dtype=torch.float32, device=device)
+    flat = out.view(-1)
+    for first in range(0, flat.numel(), _CHUNK):
+        n = min(_CHUNK, flat.numel() - first)
+        if kind == "normal":
+            z = _standard_normal(n, first, key, device)
+            flat[first:first + n] = z.mul_(float(spec.init[1]))
+        else:
+            lo, hi = float(spec.init[1]), float(spec.init[2])
+            u = (_uniform_bits(n, first, key, device) >> 8).to(torch.float32) * (1.0 / (1 << 24))   # exact in fp32
+            flat[first:first + n] = u.mul_(hi - lo).add_(lo)
+    return out
 
 
 def _cpu_model(config: Any, dtype: torch.dtype, **spec_kw: Any):

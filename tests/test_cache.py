@@ -204,3 +204,34 @@ def test_random_orders_lose_no_page(seed):
     m.check()
     assert all(g.allocator.num_free == g.allocator.num_pages for g in m.groups)
     assert m.slots.num_free == 5
+
+
+def test_a_step_that_fails_leaves_the_cache_as_it_was():
+    """Engine.step: when the forward pass raises (here: no GPU, so the first kernel call does), requests that
+    came with the step are gone again and the others hold what they held before."""
+    import torch
+    import tiny_models as TM
+    from infernum_amd import CacheConfig, Engine
+    from infernum_amd.kernels.api import KernelError
+    from infernum_amd.weights.random_init import _cpu_model
+    if torch.cuda.is_available():
+        pytest.skip("the forward pass must fail for this test: it needs a machine without a GPU")
+    model = _cpu_model(TM.tiny_config("C"), torch.float32)       # two groups: all keys, and a window
+    eng = Engine(model, CacheConfig(page_size=4, num_pages=16, num_state_slots=3))
+    cache = eng.cache
+    cache.admit("old")
+    assert cache.reserve("old", 6)
+    cache.commit("old", 6)
+    free_before = [cache.free_pages(g) for g in range(len(cache.groups))]
+    table_before = [cache.block_table(g, "old").pages for g in range(len(cache.groups))]
+    for entries in ([("new", [1, 2, 3, 4, 5], [4])],                       # a request that comes with the step
+                    [("old", [7], [0])],                                   # one that was there, a single token
+                    [("old", [7, 8, 9, 1, 2, 3, 4], [6]), ("new", [5, 6], [])]):   # both, more pages for "old"
+        with pytest.raises(KernelError):
+            eng.step(entries)
+        assert cache.requests() == ["old"] and cache.num_tokens("old") == 6
+        assert [cache.free_pages(g) for g in range(len(cache.groups))] == free_before
+        assert [cache.block_table(g, "old").pages for g in range(len(cache.groups))] == table_before
+        assert cache.slots.num_free == 2
+        cache.check()
+    assert eng.steps_run == 0

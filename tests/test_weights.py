@@ -203,3 +203,21 @@ def test_write_random_model_writes_a_folder_that_reads_back(tmp_path):
     from infernum_amd.config import load_config
     assert load_config(d) == cfg
     assert all(e.dtype == torch.bfloat16 for e in open_model_tensors(d).values())
+
+
+def test_random_values_are_a_function_of_the_element_alone(monkeypatch):
+    """The same numbers whether a tensor is made in one piece or in several, and a normal distribution."""
+    from infernum_amd.parts.base import WeightSpec
+    from infernum_amd.weights import random_init as R
+    spec = WeightSpec((37, 1001), ("normal", 0.5))
+    whole = R.draw(spec, 3, "w", torch.device("cpu"))
+    monkeypatch.setattr(R, "_CHUNK", 1000)
+    assert torch.equal(R.draw(spec, 3, "w", torch.device("cpu")), whole)
+    assert not torch.equal(R.draw(spec, 3, "v", torch.device("cpu")), whole)
+    z = R.draw(WeightSpec((1 << 20,), ("normal", 1.0)), 0, "z", torch.device("cpu")).double()
+    assert abs(z.mean().item()) < 5e-3 and abs(z.var().item() - 1) < 5e-3
+    assert abs((z ** 3).mean().item()) < 2e-2 and abs((z ** 4).mean().item() - 3) < 5e-2
+    assert abs((z[1:] * z[:-1]).mean().item()) < 5e-3            # neighbours are not correlated
+    assert 4.0 < z.abs().max().item() < 5.0
+    u = R.draw(WeightSpec((1 << 16,), ("uniform", -1.0, 3.0)), 0, "u", torch.device("cpu")).double()
+    assert -1.0 <= u.min().item() < -0.99 and 2.99 < u.max().item() < 3.0 and abs(u.mean().item() - 1.0) < 2e-2
