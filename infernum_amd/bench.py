@@ -19,6 +19,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("n_gen", nargs="?", type=int, default=128, help="number of tokens to generate")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"], help="compute dtype")
     ap.add_argument("--prefill", type=int, default=512, help="also time a prompt of this many tokens (0: skip)")
+    ap.add_argument("--kernels", default="auto", choices=["auto", "generic"],
+                    help="generic: the plain twins of the fast kernels (slow; for comparisons)")
     ap.add_argument("--gpus", type=int, default=1, help="one GPU only: this engine has no multi-GPU path")
     a = ap.parse_args(argv)
     if a.gpus != 1:
@@ -34,7 +36,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     need = max(a.prefill, 8 + a.n_gen) + 64
     bc = BatchConfig(max_batch_size=4, max_prefill_tokens=max(a.prefill, 512), block_size=16,
                      num_blocks=2 * (need // 16 + 2), max_tokens_per_step=max(a.prefill, 512) + 4)
-    rt = Runtime.from_pretrained(a.model, dtype=dtype, batch_config=bc)
+    rt = Runtime.from_pretrained(a.model, dtype=dtype, batch_config=bc, kernels=a.kernels)
     print(f"Model loaded: {config.num_hidden_layers} layers, {config.hidden_size} hidden, dtype={a.dtype}",
           file=sys.stderr)
     rng = random.Random(0)

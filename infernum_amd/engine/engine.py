@@ -67,7 +67,8 @@ class Engine:
 
     # ---- building ------------------------------------------------------------------
     @staticmethod
-    def runtime(dtype: Any = "bfloat16", device: Any = "cuda:0", max_tokens_per_step: int = 8192) -> Runtime:
+    def runtime(dtype: Any = "bfloat16", device: Any = "cuda:0", max_tokens_per_step: int = 8192,
+                kernels: str = "auto") -> Runtime:
         from ..kernels.api import KernelError
         dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
               "f32": torch.float32, torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}.get(dtype)
@@ -76,12 +77,14 @@ class Engine:
         dev = torch.device(device)
         if dev.type != "cuda" or not torch.cuda.is_available():
             raise KernelError("infernum_amd runs on a gfx950 GPU only: no GPU is visible (there is no CPU fallback)")
-        return Runtime(dev, dt, max_tokens_per_step)
+        return Runtime(dev, dt, max_tokens_per_step, kernels)
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", cache_config: Optional[CacheConfig] = None,
                         device: Any = "cuda:0", use_graphs: bool = True, **runtime_kw: Any) -> "Engine":
-        """Model class by config.json's model_type, weights from the folder's safetensors."""
+        """Model class by config.json's model_type, weights from the folder's safetensors.
+        ``kernels="generic"`` (a runtime keyword) runs every matrix product and the attention on the plain
+        twins of the fast kernels, in either type."""
         from .. import models  # noqa: F401  (registers the architectures)
         from ..config.registry import load_config, model_spec_for
         from ..weights.loader import load_weights

@@ -61,10 +61,10 @@ class Runtime:
     # ---- building ---------------------------------------------------------------------
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", batch_config: Optional[BatchConfig] = None,
-                        max_seq_len: Optional[int] = None, device: Any = "cuda:0") -> "Runtime":
+                        max_seq_len: Optional[int] = None, device: Any = "cuda:0", kernels: str = "auto") -> "Runtime":
         bc = batch_config or BatchConfig()
         engine = Engine.from_pretrained(
-            model_dir, dtype=dtype, device=device, max_tokens_per_step=bc.max_tokens_per_step,
+            model_dir, dtype=dtype, device=device, max_tokens_per_step=bc.max_tokens_per_step, kernels=kernels,
             cache_config=CacheConfig(page_size=bc.block_size, num_pages=bc.num_blocks,
                                      num_state_slots=bc.max_batch_size))
         return cls(engine, load_tokenizer(model_dir), bc, max_seq_len)

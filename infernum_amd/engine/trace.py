@@ -23,7 +23,7 @@ MAX_LIVE_REQUESTS = 4
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, stream: IO[str], done: IO[str],
-           page_size: int = PAGE_SIZE, poison: bool = False) -> int:
+           page_size: int = PAGE_SIZE, poison: bool = False, kernels: str = "auto") -> int:
     from ..cache import CacheConfig
     from .engine import Engine, StepEntry
 
@@ -35,7 +35,7 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, stream: IO
         model_dir, dtype=dtype,
         cache_config=CacheConfig(page_size=page_size, num_pages=num_pages, num_state_slots=2 * MAX_LIVE_REQUESTS,
                                  poison_freed_pages=poison),
-        max_tokens_per_step=max(8192, int(max_tokens)))
+        max_tokens_per_step=max(8192, int(max_tokens)), kernels=kernels)
     print(f"[trace_run] ready: {num_pages} pages of {page_size} tokens", file=sys.stderr, flush=True)
     for line in stream:
         line = line.strip()
@@ -65,10 +65,13 @@ def main(argv: Optional[list] = None) -> int:
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
+    ap.add_argument("--kernels", default="auto", choices=["auto", "generic"],
+                    help="generic: every matrix product and the attention on the plain twins of the fast kernels")
     ap.add_argument("--page-size", type=int, default=PAGE_SIZE, help=argparse.SUPPRESS)
     ap.add_argument("--poison-freed-pages", action="store_true", help=argparse.SUPPRESS)
     a = ap.parse_args(argv)
-    return replay(a.model, a.dtype, a.out, a.max_tokens, sys.stdin, sys.stdout, a.page_size, a.poison_freed_pages)
+    return replay(a.model, a.dtype, a.out, a.max_tokens, sys.stdin, sys.stdout, a.page_size, a.poison_freed_pages,
+                  a.kernels)
 
 
 if __name__ == "__main__":

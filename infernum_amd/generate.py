@@ -5,7 +5,7 @@ reference's ``generate`` example (infernum-examples/examples/generate.rs:37-86):
         [-t 0.7] [-p 0.9] [-s 42] [-r 1.1] [--repetition-penalty-window 64] [--max-seq-len N]
 
 Added here: ``--prompt-ids 1,2,3`` for model folders without a tokenizer (token
-ids in, token ids out), ``--dtype bfloat16|float32``, and the cache's settings
+ids in, token ids out), ``--dtype bfloat16|float32``, ``--kernels auto|generic``, and the cache's settings
 (``--block-size``, ``--num-blocks``, ``--max-batch``, ``--chunk``).  The model class
 is chosen by config.json's ``model_type``, as everywhere in the package.
 """
@@ -38,6 +38,8 @@ def build_parser() -> argparse.ArgumentParser:
                     help="longest sequence (prompt and generated tokens); default min(model max, 4096)")
     ap.add_argument("--prompt-ids", default=None, help="comma-separated token ids instead of a text prompt")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "f32"])
+    ap.add_argument("--kernels", default="auto", choices=["auto", "generic"],
+                    help="generic: the plain twins of the fast kernels for every product and the attention")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache")
     ap.add_argument("--num-blocks", type=int, default=None, help="pages in the pool (default: for max-seq-len)")
     ap.add_argument("--max-batch", type=int, default=32, help="most requests running at once")
@@ -57,7 +59,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     num_blocks = a.num_blocks or (-(-max_seq_len // a.block_size) + 1)
     bc = BatchConfig(max_batch_size=a.max_batch, max_prefill_tokens=a.chunk, block_size=a.block_size,
                      num_blocks=num_blocks, max_tokens_per_step=max(a.chunk + a.max_batch, 2048))
-    rt = Runtime.from_pretrained(a.model, dtype=a.dtype, batch_config=bc, max_seq_len=max_seq_len)
+    rt = Runtime.from_pretrained(a.model, dtype=a.dtype, batch_config=bc, max_seq_len=max_seq_len, kernels=a.kernels)
     print(f"Model loaded ({config.num_hidden_layers} layers, {config.hidden_size} hidden, {config.vocab_size} vocab)")
 
     sampling = None if a.greedy else SamplingParams(a.temperature, a.top_p, a.seed, a.repetition_penalty,

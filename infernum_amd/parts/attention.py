@@ -61,14 +61,14 @@ class Attention(Mixer):
         self.hidden_size, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.window = int(window) if window else 0
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
-        self.kernels = kernels
+        if kernels not in ("auto", "generic"):
+            raise ValueError("kernels must be 'auto' or 'generic'")
+        self.kernels = kernels = "generic" if rt.kernels == "generic" else kernels
         self.init_std = init_std
         pos_spec = PartSpec(**position) if isinstance(position, Mapping) else (position or PartSpec("none"))
         self.position = make_part("position", pos_spec, rt)
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
-        if kernels not in ("auto", "generic"):
-            raise ValueError("kernels must be 'auto' or 'generic'")
         self.rotate_in_attention = _decode_rotation == "attention"
         self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
                          and K.attention_mfma_available(self.d))
@@ -102,29 +102,29 @@ class Attention(Mixer):
                 and x.shape[0] <= ROTATE_IN_ATTENTION_UP_TO and cache.k_pages.shape[2] % 4 == 0):
             # every request brings one token: rotation, the write to the pages and attention are one launch
             w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
-            qkv = linear(x, w, keep_split=True)
+            qkv = linear(x, w, keep_split=True, kernels=self.rt.kernels)
             out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
             K.attention_decode_rotating(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                                         ctx.slots[g] if cache.writable else None, cache.k_pages, cache.v_pages, out,
                                         ctx.block_tables[g], nh, nkv, d, self.scale, self.window, ctx.max_total_len)
-            return linear(out, self.w_o, keep_split=True)
+            return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
         q_out = None
         if cache.writable:
-            qkv = linear(x, self.w_qkv, keep_split=True)
+            qkv = linear(x, self.w_qkv, keep_split=True, kernels=self.rt.kernels)
             if isinstance(qkv, K.SplitSum):
                 q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
             q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
                                  ctx.slots[g], cache.k_pages, cache.v_pages, q_out=q_out)
         else:
             # keys and values of another run of a layer: only queries are made here
-            qkv = linear(x, self.w_qkv[: nh * d], keep_split=True)
+            qkv = linear(x, self.w_qkv[: nh * d], keep_split=True, kernels=self.rt.kernels)
             if isinstance(qkv, K.SplitSum):
                 q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
             q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
                                  q_out=q_out)
         out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
         self.attend(q, out, ctx, cache)
-        return linear(out, self.w_o, keep_split=True)
+        return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d

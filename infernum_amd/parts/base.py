@@ -114,6 +114,13 @@ class Runtime:
     device: torch.device
     dtype: torch.dtype                       # torch.bfloat16 or torch.float32: activations, matrices, cache
     max_tokens_per_step: int = 8192
+    # "auto": the fast kernel for each operation where it takes the size; "generic": the plain twins only
+    # (one fp32 multiply-add chain per output element, one wave per token and head in attention), in either type
+    kernels: str = "auto"
+
+    def __post_init__(self) -> None:
+        if self.kernels not in ("auto", "generic"):
+            raise ValueError(f"kernels must be 'auto' or 'generic', got {self.kernels!r}")
 
     @property
     def is_fp32(self) -> bool:

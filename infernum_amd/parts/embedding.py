@@ -54,7 +54,7 @@ class LinearHead(Head):
         self.weight = tensors["weight"]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(x, self.weight, out_dtype=torch.float32)
+        return linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
 
 
 register_part("embedding", "token", TokenEmbedding)

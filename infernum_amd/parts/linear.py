@@ -59,17 +59,23 @@ def prefill_gemm() -> str:
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           epilogue: Optional[str] = None, keep_split: bool = False) -> Union[torch.Tensor, SplitSum]:
+           epilogue: Optional[str] = None, keep_split: bool = False,
+           kernels: str = "auto") -> Union[torch.Tensor, SplitSum]:
+    """``kernels="generic"``: the plain product (fp32 multiply-adds in a fixed order) for every size and type."""
     M, Kdim = x.shape
     N = w.shape[0]
     out_dtype = out_dtype or x.dtype
     n_out = N // 2 if epilogue == "swiglu" else N
     if M == 0:
         return torch.empty((0, n_out), dtype=out_dtype, device=x.device)
-    if x.dtype == torch.bfloat16 and K.gemm_skinny_supported(M, N, Kdim) and x.is_contiguous() and \
+    if kernels == "generic":
+        if x.dtype not in (torch.float32, torch.bfloat16):
+            raise K.KernelError(f"linear: dtype {x.dtype} is not supported")
+        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
+    elif x.dtype == torch.bfloat16 and K.gemm_skinny_supported(M, N, Kdim) and x.is_contiguous() and \
             (M <= SKINNY_ROWS_ANY_WIDTH or N < SKINNY_WIDE or out_dtype != torch.bfloat16):
         return K.gemm_skinny(x, w, epilogue=epilogue, keep_split=keep_split, out_dtype=out_dtype)
-    if x.dtype == torch.float32:
+    elif x.dtype == torch.float32:
         y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
     elif x.dtype != torch.bfloat16:
         raise K.KernelError(f"linear: dtype {x.dtype} is not supported")

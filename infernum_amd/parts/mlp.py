@@ -36,8 +36,8 @@ class SwiGLUFeedForward(FeedForward):
         self.w_down = tensors["down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):
-        act = linear(x, self.w_gate_up, epilogue="swiglu")
-        return linear(act, self.w_down, keep_split=True)
+        act = linear(x, self.w_gate_up, epilogue="swiglu", kernels=self.rt.kernels)
+        return linear(act, self.w_down, keep_split=True, kernels=self.rt.kernels)
 
 
 register_part("feed_forward", "swiglu", SwiGLUFeedForward)

@@ -110,25 +110,27 @@ def _cpu_model(config: Any, dtype: torch.dtype, **spec_kw: Any):
     return DecoderModel(spec, Runtime(torch.device("cpu"), dtype))
 
 
-def random_tensors(config: Any, seed: int, dtype: torch.dtype = torch.bfloat16,
+def random_tensors(config: Any, seed: int, dtype: torch.dtype = torch.bfloat16, made_on: Any = "cpu",
                    **spec_kw: Any) -> Iterator[Tuple[str, torch.Tensor]]:
-    """(name, CPU tensor) for every tensor a file of this model holds; matrices in ``dtype``."""
+    """(name, CPU tensor) for every tensor a file of this model holds; matrices in ``dtype``.
+    ``made_on``: the device that works the numbers out (the same numbers on any; a GPU makes a large
+    model's in seconds where the host takes minutes)."""
     model = _cpu_model(config, dtype, **spec_kw)
     for name, spec in sorted(model.expected_weights().items()):
         if not spec.write_when_random:
             continue
-        t = draw(spec, seed, name, torch.device("cpu"))
-        yield name, t.to(dtype)
+        t = draw(spec, seed, name, torch.device(made_on))
+        yield name, t.to(dtype).cpu()
 
 
 def write_random_model(config: Any, out_dir: str, seed: int, dtype: torch.dtype = torch.bfloat16,
-                       **spec_kw: Any) -> str:
+                       made_on: Any = "cpu", **spec_kw: Any) -> str:
     """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``; returns out_dir."""
     from .safetensors_io import write_safetensors
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, "config.json"), "w") as f:
         json.dump(config.to_dict(), f, indent=2)
-    write_safetensors(os.path.join(out_dir, "model.safetensors"), random_tensors(config, seed, dtype, **spec_kw))
+    write_safetensors(os.path.join(out_dir, "model.safetensors"), random_tensors(config, seed, dtype, made_on, **spec_kw))
     return out_dir
 
 
@@ -140,9 +142,9 @@ def random_weights_on_device(model, seed: int) -> None:
     for name, spec in sorted(expected.items()):
         if not spec.write_when_random and spec.fallback is not None:
             continue                              # shares its fallback's buffer, below
-        t = draw(spec, seed, name, rt.device)
-        target = rt.dtype if (spec.follows_compute_dtype or rt.dtype == torch.float32) else torch.float32
-        tensors[name] = t.to(target)
+        # what loading the folder that write_random_model(dtype=rt.dtype) writes would give: every tensor
+        # rounded to that type once, also those that do not follow the compute type
+        tensors[name] = draw(spec, seed, name, rt.device).to(rt.dtype)
     for name, spec in expected.items():          # a tied head whose fallback sorts after it
         if name not in tensors:
             tensors[name] = tensors[spec.fallback]

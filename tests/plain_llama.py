@@ -112,15 +112,22 @@ def rope(x: torch.Tensor, positions: torch.Tensor, freqs: torch.Tensor) -> torch
     return torch.cat([a * cos - b * sin, a * sin + b * cos], dim=-1)
 
 
+def rounded(x: torch.Tensor, to: Optional[torch.dtype]) -> torch.Tensor:
+    """x with every value rounded to the nearest of ``to`` (kept in x's own dtype); x itself without ``to``."""
+    return x if to is None else x.to(to).to(x.dtype)
+
+
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-                     window: Optional[int] = None) -> torch.Tensor:
+                     window: Optional[int] = None, round_to: Optional[torch.dtype] = None) -> torch.Tensor:
     """q [T, nh, d], k, v [T, nkv, d] of one whole sequence -> [T, nh, d].
 
     Query head h reads key/value head h * nkv // nh
     (infernum-cuda/kernels/paged_decode_attention.cu:342); scores scale * <q, k_j>
     over keys j <= t, and j >= t - window + 1 with a window
     (kernels/flash_prefill_attention_v2.cu:85-88); softmax with the maximum
-    subtracted; output sum_j w_j v_j.
+    subtracted; output sum_j w_j v_j.  With ``round_to`` the exponentials are rounded before they
+    are summed and multiplied with the values, as a kernel does that feeds them to a matrix unit
+    (the reference's kernels keep them in fp32, paged_decode_attention.cu:540-644).
     """
     T, nh, d = q.shape
     nkv = k.shape[1]
@@ -130,9 +137,8 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
         for t in range(T):
             lo = 0 if not window else max(0, t - window + 1)
             s = (k[lo:t + 1, g, :] @ q[t, h, :]) * scale
-            w = torch.exp(s - s.max())
-            w = w / w.sum()
-            out[t, h, :] = w @ v[lo:t + 1, g, :]
+            w = rounded(torch.exp(s - s.max()), round_to)
+            out[t, h, :] = (w @ v[lo:t + 1, g, :]) / w.sum()
     return out
 
 
@@ -152,10 +158,18 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
     return cfg.get("sliding_window")
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: Sequence[int], dtype=torch.float64) -> torch.Tensor:
+def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: Sequence[int], dtype=torch.float64,
+            round_to: Optional[torch.dtype] = None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.  Order of operations:
-    infernum-llama/src/graph_builder.rs:442-536."""
+    infernum-llama/src/graph_builder.rs:442-536.
+
+    ``round_to`` (torch.bfloat16) rounds every activation that an engine serving in that type stores between
+    two operations: the outputs of norms, projections, the rotation, attention (and its exponentials), the
+    activation function, as the reference's bf16 path does (one rounding at each kernel's store,
+    infernum-cuda/kernels/rmsnorm.cu:314, matmul.rs:111); the residual stream and the logits stay unrounded.
+    It tells how far rounding alone takes the logits from the exact ones."""
     W = {k: v.to(dtype) for k, v in w.items()}
+    r = lambda t: rounded(t, round_to)      # noqa: E731
     nh = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads") or nh
     H = cfg["hidden_size"]
@@ -168,17 +182,17 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: Sequence[int], dtype=tor
     h = embedding(W["model.embed_tokens.weight"], ids)
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        n = rms_norm(h, W[p + "input_layernorm.weight"], eps)
-        q = linear(n, W[p + "self_attn.q_proj.weight"]).reshape(T, nh, d)
-        k = linear(n, W[p + "self_attn.k_proj.weight"]).reshape(T, nkv, d)
-        v = linear(n, W[p + "self_attn.v_proj.weight"]).reshape(T, nkv, d)
-        q, k = rope(q, pos, freqs), rope(k, pos, freqs)
-        a = causal_attention(q, k, v, 1.0 / math.sqrt(d), layer_window(cfg, i)).reshape(T, nh * d)
-        h = h + linear(a, W[p + "self_attn.o_proj.weight"])
-        m = rms_norm(h, W[p + "post_attention_layernorm.weight"], eps)
-        act = swiglu(linear(m, W[p + "mlp.gate_proj.weight"]), linear(m, W[p + "mlp.up_proj.weight"]))
-        h = h + linear(act, W[p + "mlp.down_proj.weight"])
-    f = rms_norm(h, W["model.norm.weight"], eps)
+        n = r(rms_norm(h, W[p + "input_layernorm.weight"], eps))
+        q = r(linear(n, W[p + "self_attn.q_proj.weight"])).reshape(T, nh, d)
+        k = r(linear(n, W[p + "self_attn.k_proj.weight"])).reshape(T, nkv, d)
+        v = r(linear(n, W[p + "self_attn.v_proj.weight"])).reshape(T, nkv, d)
+        q, k = r(rope(q, pos, freqs)), r(rope(k, pos, freqs))
+        a = r(causal_attention(q, k, v, 1.0 / math.sqrt(d), layer_window(cfg, i), round_to)).reshape(T, nh * d)
+        h = h + r(linear(a, W[p + "self_attn.o_proj.weight"]))
+        m = r(rms_norm(h, W[p + "post_attention_layernorm.weight"], eps))
+        act = r(swiglu(r(linear(m, W[p + "mlp.gate_proj.weight"])), r(linear(m, W[p + "mlp.up_proj.weight"]))))
+        h = h + r(linear(act, W[p + "mlp.down_proj.weight"]))
+    f = r(rms_norm(h, W["model.norm.weight"], eps))
     # the head is the embedding matrix when the file has no lm_head.weight
     # (infernum-cuda/src/inner/cuda_graph_engine.rs:225-232)
     head = W["lm_head.weight"] if "lm_head.weight" in W else W["model.embed_tokens.weight"]
@@ -199,6 +213,21 @@ def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt: Sequence[int], n_new: 
             break
         out.append(tok)
         ids.append(tok)
+    return out
+
+
+def greedy_shortfalls(cfg: dict, w: Dict[str, torch.Tensor], prompt: Sequence[int], tokens: Sequence[int],
+                      dtype=torch.float64) -> List[float]:
+    """For a continuation that somebody else chose greedily: for each of its tokens, how far the plain model's
+    logit of that token lies below the plain model's largest logit at that place, as a fraction of the RMS of
+    the logits there (0: the plain model's own choice).  An engine whose logits are within e of the plain
+    model's can only choose tokens with a shortfall of at most 2 e."""
+    ids = list(prompt) + list(tokens)
+    logits = forward(cfg, w, ids, dtype)
+    out = []
+    for i, t in enumerate(tokens):
+        row = logits[len(prompt) + i - 1]
+        out.append(float((row.max() - row[t]) / row.pow(2).mean().sqrt()))
     return out
 
 

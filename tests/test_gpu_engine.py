@@ -45,15 +45,15 @@ def models(tmp_path_factory):
     return out
 
 
-def _engine(model_dir, dtype, page_size, num_pages, poison=True):
+def _engine(model_dir, dtype, page_size, num_pages, poison=True, **kw):
     from infernum_amd import CacheConfig, Engine
-    return Engine.from_pretrained(model_dir, dtype=dtype,
+    return Engine.from_pretrained(model_dir, dtype=dtype, **kw,
                                   cache_config=CacheConfig(page_size=page_size, num_pages=num_pages,
                                                            num_state_slots=8, poison_freed_pages=poison))
 
 
-def _check(got, ref, dtype, what):
-    worst, rms, where = TT.error_against(got, ref)
+def _check(got, ref, dtype, what, every_place=True):
+    worst, rms, where = TT.error_against(got, ref, every_place)
     print(f"{what}: max|diff| = {worst:.3e}, rms of logits = {rms:.3e}, ratio {worst / rms:.2e} at {where}")
     assert worst == worst, f"{what}: NaN in the logits at {where}"
     assert worst <= TOL[dtype] * rms, f"{what}: max|diff| {worst:.3e} > {TOL[dtype]} * rms {rms:.3e} at {where}"
@@ -171,15 +171,41 @@ def test_cutting_does_not_change_fp32_logits(models):
         assert torch.equal(a[k], c[k]), k
 
 
-def test_trace_run_program(models, tmp_path):
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_plain_twins_of_the_fast_kernels_through_the_engine(models, name):
+    """``kernels="generic"``: every matrix product and the attention on the plain kernels, also in bfloat16.
+    Against the plain model, against the fast kernels (two sets of roundings of the same numbers), and in
+    32-bit the very bits of the default path, which has no other kernels."""
+    d, cfg, reqs, ref = models[(name, "bfloat16", "mixed")]
+    prompt_len = {r: max(2, len(t) - 20) for r, t in reqs.items()}
+    steps, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=5)
+    plain = _engine(d, "bfloat16", PAGE[name], max_tokens // PAGE[name], kernels="generic")
+    assert not plain.model.blocks[0].mixer.use_mfma and plain.rt.kernels == "generic"
+    got = TT.run_steps(plain, steps)
+    _check(got, ref, "bfloat16", f"{name} bfloat16 mixed, plain kernels")
+    fast = TT.run_steps(_engine(d, "bfloat16", PAGE[name], max_tokens // PAGE[name]), steps)
+    worst, rms, where = TT.error_against(got, {r: torch.stack([fast[(r, i)] for i in range(len(t))])
+                                               for r, t in reqs.items()})
+    print(f"{name}: plain and fast kernels differ by {worst / rms:.2e} of the logits' RMS at {where}")
+    assert worst <= 2 * TOL["bfloat16"] * rms
+    d32, _, reqs32, _ = models[(name, "float32")]
+    a = TT.run_steps(_engine(d32, "float32", PAGE[name], 64, kernels="generic"), TT.trace_portions(reqs32))
+    b = TT.run_steps(_engine(d32, "float32", PAGE[name], 64), TT.trace_portions(reqs32))
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    with pytest.raises(ValueError):
+        _engine(d, "bfloat16", 8, 8, kernels="fastest")
+
+
+@pytest.mark.parametrize("dtype,kernels", [("float32", "auto"), ("bfloat16", "generic")])
+def test_trace_run_program(models, tmp_path, dtype, kernels):
     """bin/trace_run as a user starts it: steps on standard input, files out."""
-    d, cfg, reqs, ref = models[("A", "float32")]
+    d, cfg, reqs, ref = models[("A", dtype)]
     prompt_len = {r: max(2, len(t) - 10) for r, t in reqs.items()}
     steps, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=9)
     out = tmp_path / "out"
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", "float32",
-                           "--out", str(out), "--max-tokens", str(max_tokens)],
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(max_tokens), "--kernels", kernels],
                           input="".join(json.dumps(s) + "\n" for s in steps), text=True, capture_output=True,
                           timeout=600)
     assert proc.returncode == 0, proc.stderr[-3000:]
@@ -196,7 +222,7 @@ def test_trace_run_program(models, tmp_path):
                 got[(e["id"], base + w)] = torch.from_numpy(arr[row].copy())
                 row += 1
             pos[e["id"]] = base + len(e["tokens"])
-    _check(got, ref, "float32", "trace_run A float32 mixed")
+    _check(got, ref, dtype, f"trace_run A {dtype} mixed, kernels {kernels}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -232,4 +258,5 @@ def test_recorded_decode_steps_equal_eager_ones(models, name, dtype):
                 eng.end("x")
     assert graphed.graph_replays >= 30
     got = {(r, fed[r] - 1): graphed.step([StepEntry(r, reqs[r][fed[r]:fed[r] + 1], [0])])[0].cpu() for r in names[:1]}
-    _check({(names[0], fed[names[0]]): got[(names[0], fed[names[0]] - 1)]}, ref, dtype, f"{name} {dtype} recorded decode")
+    _check({(names[0], fed[names[0]]): got[(names[0], fed[names[0]] - 1)]}, ref, dtype, f"{name} {dtype} recorded decode",
+           every_place=False)

@@ -106,14 +106,96 @@ def test_too_few_pages_changes_no_greedy_token(folders):
     assert tight.engine.cache.free_pages() == 18
 
 
-def test_bfloat16_generation_runs_and_mostly_agrees(folders):
+def _record_logits(rt):
+    """Wraps the engine's step function: (request, place) -> the logits row that came back for it."""
+    seen, real_step = {}, rt.engine.step
+
+    def step(entries):
+        before = {e.request: (rt.engine.cache.num_tokens(e.request) if rt.engine.cache.has(e.request) else 0)
+                  for e in entries}
+        logits = real_step(entries)
+        rows = logits.detach().double().cpu()
+        k = 0
+        for e in entries:
+            for wanted in e.want:
+                seen.setdefault(e.request, {})[before[e.request] + wanted] = rows[k]
+                k += 1
+        assert k == rows.shape[0]
+        return logits
+    rt.engine.step = step
+    return seen
+
+
+@pytest.mark.parametrize("num_blocks", [64, 14])
+def test_bfloat16_generation_through_the_scheduler_token_by_token(tmp_path, num_blocks):
+    """Greedy generation in bfloat16 through scheduler, step function and sampler, prompts in portions beside
+    decoded tokens (and, with 14 pages, requests set back and computed again): at every place where a token was
+    chosen the engine's logits are the plain model's for the same history within the bfloat16 tolerance, the
+    token is the first largest of the engine's logits, and its plain logit is within twice the tolerance of the
+    plain model's largest."""
     from infernum_amd import GenerateOptions
+    TOL = 6e-2
+    d = TM.write_tiny("B", str(tmp_path / "B16"), dtype=torch.bfloat16)
+    cfg, w = P.read_model(d)
+    g = torch.Generator().manual_seed(8)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (21, 9, 33, 14)]
+    rt = _runtime(d, "bfloat16", block_size=8, num_blocks=num_blocks, max_batch_size=4, max_prefill_tokens=8,
+                  max_tokens_per_step=16)
+    seen = _record_logits(rt)
+    seqs = [rt.submit(p, GenerateOptions(max_new_tokens=18)) for p in prompts]
+    n_back = 0
+    while not rt.scheduler.is_idle():
+        n_back += len(rt.step().set_back)
+    assert (n_back > 0) == (num_blocks == 14), f"{n_back} requests were set back with {num_blocks} pages"
+    worst = 0.0
+    for s, p in zip(seqs, prompts):
+        out = list(s.generated_ids)
+        assert len(out) == 18 and s.error is None
+        ref = P.forward(cfg, w, p + out)
+        for i, t in enumerate(out):
+            place = len(p) + i - 1
+            row = seen[s.id][place]                       # after a set-back: the row computed last for the place
+            rms = ref[place].pow(2).mean().sqrt()
+            worst = max(worst, float((row - ref[place]).abs().max() / rms))
+            assert int(torch.argmax(row)) == t
+            assert float((ref[place].max() - ref[place][t]) / rms) <= 2 * TOL
+    print(f"bfloat16 generation with {num_blocks} pages: worst |diff| / rms {worst:.2e}, {n_back} set back")
+    assert worst <= TOL
+    rt.scheduler.reap(rt.engine.cache)
+    rt.engine.cache.check()
+    assert rt.engine.cache.free_pages() == num_blocks
+
+
+def test_too_few_pages_changes_no_sampled_token(folders):
+    """Sampled requests that are set back and computed again draw the same tokens: the draw is keyed by the
+    seed and the number of tokens generated so far, and the logits of a history do not depend on how it was
+    computed.  Against the plain sampler on the plain model's logits as well."""
+    from infernum_amd import GenerateOptions, SamplingParams
     d, cfg, w = folders["B"]
-    prompt = list(range(40, 60))
-    want = P.greedy(cfg, w, prompt, 8)
-    got = _runtime(d, "bfloat16", block_size=8, num_blocks=16, max_batch_size=2).generate(
-        prompt, GenerateOptions(max_new_tokens=8))
-    assert len(got) == 8 and got[0] == want[0]
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (9, 17, 6, 12)]
+    sp = [SamplingParams(temperature=0.8, top_p=0.95, seed=7 + i, repetition_penalty=1.05,
+                         repetition_penalty_window=6) for i in range(4)]
+    opts = [GenerateOptions(max_new_tokens=16, sampling=s) for s in sp]
+    roomy = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=4, max_prefill_tokens=8)
+    want = roomy.generate_batch(prompts, opts)
+    tight = _runtime(d, "float32", block_size=4, num_blocks=17, max_batch_size=4, max_prefill_tokens=8)
+    seqs = [tight.submit(p, o) for p, o in zip(prompts, opts)]
+    n_back = 0
+    while not tight.scheduler.is_idle():
+        n_back += len(tight.step().set_back)
+    assert n_back > 0, "the pool was meant to run out"
+    assert [list(s.generated_ids) for s in seqs] == want
+    for p, s, out in zip(prompts, sp, want):
+        toks = list(p)
+        for i, t in enumerate(out):
+            u = P.uniform_for_token(s.seed, i)
+            assert P.sample_token(P.forward(cfg, w, toks)[-1], s.temperature, s.top_p, u, s.repetition_penalty,
+                                  toks[-6:]) == t
+            toks.append(t)
+    tight.scheduler.reap(tight.engine.cache)
+    tight.engine.cache.check()
+    assert tight.engine.cache.free_pages() == 17
 
 
 def test_command_line(folders):

@@ -71,16 +71,18 @@ def test_first_tokens(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n", [40, 100, 150])
 @pytest.mark.parametrize("name", ["B", "C"])
-def test_many_requests_decoded_together(models, name, dtype):
-    """150 requests in one decode step: more rows than the decode GEMM kernel takes (64), so the products go
-    the way of many rows while attention and the rest stay on the decode kernels."""
+def test_many_requests_decoded_together(models, name, n, dtype):
+    """Many requests in one decode step, against the plain model.  150: more rows than the decode GEMM kernel
+    takes, so the products go the way of many rows while attention and the rest stay on the decode kernels.
+    100 (the live requests go from 100 down to about 85): the decode GEMM's variant for 65 to 128 rows, with the
+    rotary kernel in front of the attention.  40: the variant for up to 64 rows, rotation inside the attention."""
     import random
     from infernum_amd import CacheConfig, Engine
     from infernum_amd.engine import StepEntry
     d, cfg, w = models[(name, dtype)]
     rng = random.Random(1)
-    n = 150
     reqs = {f"r{i}": [rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(3, 20))] for i in range(n)}
     ref = {r: P.forward(cfg, w, t) for r, t in reqs.items()}
     eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=8, num_pages=n * 4,
@@ -89,15 +91,18 @@ def test_many_requests_decoded_together(models, name, dtype):
     fed = {r: max(1, len(reqs[r]) - 4) for r in names}
     for i in range(0, n, 30):
         eng.step([StepEntry(r, reqs[r][:fed[r]], []) for r in names[i:i + 30]])
-    worst = 0.0
+    worst, live_counts = 0.0, []
     while any(fed[r] < len(reqs[r]) for r in names):
         live = [r for r in names if fed[r] < len(reqs[r])]
+        live_counts.append(len(live))
         logits = eng.step([StepEntry(r, [reqs[r][fed[r]]], [0]) for r in live]).double().cpu()
         for k, r in enumerate(live):
             want = ref[r][fed[r]].double()
             worst = max(worst, float((logits[k] - want).abs().max() / want.pow(2).mean().sqrt()))
             fed[r] += 1
     assert worst <= TOL[dtype], f"worst |diff| / rms {worst:.2e}"
+    lo, hi = {40: (1, 64), 100: (65, 128), 150: (129, 150)}[n]
+    assert all(lo <= c <= hi for c in live_counts), live_counts
     for r in names:
         eng.end(r)
     assert eng.cache.free_pages() == n * 4

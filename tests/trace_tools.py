@@ -115,8 +115,14 @@ def run_steps(engine, steps) -> Dict[Tuple[str, int], torch.Tensor]:
     return out
 
 
-def error_against(got: Dict[Tuple[str, int], torch.Tensor], want: Dict[str, torch.Tensor]):
-    """Largest |difference| over all rows, the RMS of the wanted logits, and where the largest is."""
+def error_against(got: Dict[Tuple[str, int], torch.Tensor], want: Dict[str, torch.Tensor], every_place: bool = True):
+    """Largest |difference| over all rows, the RMS of the wanted logits, and where the largest is.
+    ``every_place``: the replay must have returned a row for every place of every request of ``want``
+    (the traces of this file want them all), so that a row that never came back cannot pass."""
+    if every_place:
+        missing = [(r, p) for r, ref in want.items() for p in range(ref.shape[0]) if (r, p) not in got]
+        assert not missing, f"{len(missing)} places have no logits, the first {missing[:5]}"
+        assert len(got) == sum(ref.shape[0] for ref in want.values()), "rows for places that no request has"
     worst, where = 0.0, None
     sq, n = 0.0, 0
     for (r, p), row in got.items():
