@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0                 # MI355X HBM3E, published
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+FP32_CHECK_TOKENS = (96, 64)          # two prompts through the bfloat16 and the 32-bit path of the same model
 
 LLAMA_8B = dict(
     model_type="llama", num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
@@ -118,6 +119,43 @@ def time_decode(engine, batch, steps, warmup, prompt_len=PROMPT_LEN):
     return dt, ctx_mid
 
 
+def check_prompts(cfg):
+    import torch
+    g = torch.Generator().manual_seed(11)
+    return [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in FP32_CHECK_TOKENS]
+
+
+def check_logits(engine, cfg):
+    """Logits at every place of the check's prompts (one step, two requests), on the host."""
+    from infernum_amd.engine import StepEntry
+    prompts = check_prompts(cfg)
+    logits = engine.step([StepEntry(f"chk{i}", p, list(range(len(p)))) for i, p in enumerate(prompts)])
+    for i in range(len(prompts)):
+        engine.end(f"chk{i}")
+    return logits.float().cpu()
+
+
+def fp32_check(bf16_logits, cfg, full_layers: int, seed: int) -> dict:
+    """The same model (the bfloat16 numbers, widened) through the true 32-bit path: how far the bfloat16 path's
+    logits are from it.  (The reference can run the whole model in f32, infernum-examples/examples/bench.rs:97-99.)"""
+    import torch
+    from infernum_amd import CacheConfig, Engine
+    n = sum(FP32_CHECK_TOKENS)
+    eng = Engine.from_config(cfg, seed=seed, dtype="float32", stored_as="bfloat16", use_graphs=False,
+                             cache_config=CacheConfig(page_size=PAGE_SIZE, num_pages=n // PAGE_SIZE + 4,
+                                                      num_state_slots=4))
+    ref = check_logits(eng, cfg).double()
+    del eng
+    torch.cuda.empty_cache()
+    diff = (bf16_logits.double() - ref).abs()
+    rms = float(ref.pow(2).mean().sqrt())
+    return {"layers": cfg.num_hidden_layers, "layers_of_config": full_layers, "tokens": n,
+            "max_abs": round(float(diff.max()), 5), "rms_of_logits": round(rms, 5),
+            "max_abs_over_rms": round(float(diff.max()) / rms, 5),
+            "rms_diff_over_rms": round(float(diff.pow(2).mean().sqrt()) / rms, 5),
+            "same_argmax": round(float((bf16_logits.argmax(-1) == ref.argmax(-1)).float().mean()), 4)}
+
+
 def time_prefill(engine, cfg, dtype: str, repeats: int = 3) -> dict:
     """One prompt of 2,048 tokens in one step, logits at its last place; the best of a few runs after the first."""
     import torch
@@ -204,6 +242,9 @@ def main() -> int:
     ap.add_argument("--shape", default="8b", choices=["8b", "13b"],
                     help="8b: Llama-3.1-8B (the default, the headline); 13b: Llama-2-13B (40 key/value heads)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every request's prompt")
+    ap.add_argument("--peaks", action="store_true",
+                    help="only measure this GPU's streaming read bandwidth and bf16 matrix rate; a JSON line of its own")
+    ap.add_argument("--no-fp32-check", action="store_true", help="skip the comparison with the 32-bit path")
     ap.add_argument("--serve", action="store_true",
                     help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
     ap.add_argument("--serve-requests", type=int, default=128)
@@ -217,6 +258,10 @@ def main() -> int:
 
     if a.serve:
         return serve(a)
+    if a.peaks:
+        from infernum_amd.peaks import measure
+        print(json.dumps(measure()))
+        return 0
     import torch
     from infernum_amd import CacheConfig, Engine, LlamaConfig
 
@@ -271,6 +316,20 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * steps / d, 2)
         out["points"] = points
         out["prefill"] = time_prefill(engine, cfg, a.dtype)
+        # the same fractions against what a bare stream of loads and a bare chain of matrix instructions reach here
+        from infernum_amd.peaks import measure
+        peaks = measure()
+        out["roofline"]["measured_peak"] = peaks["hbm_read_gbs"]
+        out["roofline"]["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
+        if a.dtype == "bf16":
+            out["prefill"]["measured_peak_tflops"] = peaks["bf16_mfma_tflops"]
+            out["prefill"]["frac_of_measured"] = round(
+                out["prefill"]["frac"] * PEAK_TFLOPS["bf16"] / peaks["bf16_mfma_tflops"], 4)
+        if a.dtype == "bf16" and not a.no_fp32_check:
+            logits = check_logits(engine, cfg)
+            del engine
+            torch.cuda.empty_cache()
+            out["fp32_check"] = fp32_check(logits, cfg, full_layers, seed=0)
     print(json.dumps(out))
     return 0
 

@@ -4,8 +4,9 @@ per request, and slots for per-request state of fixed size.
 Layer runs whose mixers need the same thing of the cache (all keys; a window
 of them) form a group.  A group has its own pool of pages and its own block
 tables; all runs of a group share the block table of a request, each with pages
-of its own ([num_pages, nkv, page_size, d] for keys, the same for values;
-the reference keeps [num_pages, page_size, nkv, d] per layer,
+of its own (what a page holds is declared by the mixer's CacheSpec as named tensors with a per-token
+shape; for attention [num_pages, nkv, page_size, d] for keys and the transposed [num_pages, nkv, d,
+page_size] for values; the reference keeps [num_pages, page_size, nkv, d] per layer,
 infernum-cuda/src/inner/cuda/paged_kv_cache.rs:88-102, and has one group only).
 Pages go back to the pool when a request ends (infernum-runtime/src/scheduler.rs:
 289-305) or, in a window group, when every later query's window has passed them
@@ -135,18 +136,15 @@ class CacheManager:
         self._names: Dict[int, Hashable] = {}
         self._next_id = 0
         self._per_group = (ctypes.c_int * max(G, 1))()
-        # device memory
-        self.k_pages: List[Optional[torch.Tensor]] = [None] * len(needs)
-        self.v_pages: List[Optional[torch.Tensor]] = [None] * len(needs)
+        # device memory: per schedule entry the pools that its mixer's CacheSpec declares, by name
+        self.pages: List[Dict[str, torch.Tensor]] = [{} for _ in needs]
         self.state: List[Optional[torch.Tensor]] = [None] * len(needs)
         if device is not None:
             for i, (cs, ss) in enumerate(needs):
                 if cs is not None:
-                    # values are kept transposed within a page: what the PV product of the matrix cores reads
-                    self.k_pages[i] = torch.zeros((config.num_pages, cs.num_kv_heads, self.page_size, cs.head_dim),
-                                                  dtype=dtype, device=device)
-                    self.v_pages[i] = torch.zeros((config.num_pages, cs.num_kv_heads, cs.head_dim, self.page_size),
-                                                  dtype=dtype, device=device)
+                    for pt in cs.payload:
+                        self.pages[i][pt.name] = torch.zeros(pt.pool_shape(int(config.num_pages), self.page_size),
+                                                             dtype=pt.dtype or dtype, device=device)
                 if ss is not None:
                     self.state[i] = torch.zeros((config.num_state_slots,) + tuple(ss.shape), dtype=ss.dtype,
                                                 device=device)
@@ -167,6 +165,15 @@ class CacheManager:
         if i is None:
             raise PageError(f"request {req!r} is not admitted")
         return i
+
+    @property
+    def k_pages(self) -> List[Optional[torch.Tensor]]:
+        """Per schedule entry the pool named "k" (None where the entry has none)."""
+        return [p.get("k") for p in self.pages]
+
+    @property
+    def v_pages(self) -> List[Optional[torch.Tensor]]:
+        return [p.get("v") for p in self.pages]
 
     def native_handle(self) -> ctypes.c_void_p:
         return self._h
@@ -316,8 +323,9 @@ class CacheManager:
                 continue
             idx = torch.tensor(pages, dtype=torch.long, device=self.device)
             for e in g.entries:
-                self.k_pages[e].index_fill_(0, idx, float("nan"))
-                self.v_pages[e].index_fill_(0, idx, float("nan"))
+                for pool in self.pages[e].values():
+                    if pool.dtype.is_floating_point:
+                        pool.index_fill_(0, idx, float("nan"))
 
     # ---- what a step needs --------------------------------------------------------
     def free_pages(self, group: int = 0) -> int:
@@ -347,8 +355,8 @@ class CacheManager:
         out = []
         for i, src in enumerate(self._cache_of):
             j = i if src is None else src
-            out.append(CacheView(group=self._entry_group[j], k_pages=self.k_pages[j], v_pages=self.v_pages[j],
-                                 writable=src is None, state=self.state[j]))
+            out.append(CacheView(group=self._entry_group[j], pages=self.pages[j], writable=src is None,
+                                 state=self.state[j]))
         return out
 
     # ---- invariants (tests) ---------------------------------------------------------

@@ -42,6 +42,7 @@ CORE_SOURCES = [
     "gemm_mfma.hip",
     "attention_generic.hip",
     "sampling.hip",
+    "peaks.hip",
 ]
 HEADERS = ["common.h", "no_alloc.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.

@@ -22,7 +22,6 @@ import torch
 from ..cache import CacheManager, native
 from ..parts.base import StepContext
 
-PREFILL_TILE_ROWS = 64      # query rows per workgroup tile of the MFMA prefill attention
 POW2_WIDTH = -1             # for pack_step's bt_width
 
 
@@ -51,6 +50,7 @@ class PackedStep:
     num_decode: int
     num_tiles: int
     num_logit_rows: int
+    tile_rows: int = 0                   # height of the row tiles that were packed (0: none)
 
     def context(self, dev: torch.Tensor) -> StepContext:
         """The step as the parts see it, over ``dev``, the device copy of ``host``."""
@@ -65,7 +65,7 @@ class PackedStep:
             slots=[seg(8 + 2 * g) for g in range(n_groups)],
             q_lens=self.q_lens, ctx_lens=self.ctx_lens, max_q_len=max(self.q_lens),
             max_total_len=max(c + q for c, q in zip(self.ctx_lens, self.q_lens)),
-            prefill_tiles=seg(7).view(-1, 2), num_prefill_tiles=self.num_tiles,
+            packed_row_tiles={self.tile_rows: (seg(7).view(-1, 2), self.num_tiles)} if self.tile_rows else {},
         )
 
 
@@ -95,10 +95,12 @@ def check_entries(entries: Sequence[StepEntry], vocab_size: int, max_tokens: int
         raise StepError(f"a step of {total} tokens is above max_tokens_per_step {max_tokens}")
 
 
-def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optional[int] = None) -> PackedStep:
+def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optional[int] = None,
+              tile_rows: int = 0) -> PackedStep:
     """Pages for the entries' tokens must be reserved already.  ``bt_width`` widens the block
     tables to a fixed number of columns (filled with NO_PAGE); ``POW2_WIDTH`` to the power of two
-    (at least 8) that holds the longest table of any group.  The arrays are laid out natively
+    (at least 8) that holds the longest table of any group.  ``tile_rows``: the height of the row tiles
+    that a part of the model asked for (``Part.step_needs``), 0 for none.  The arrays are laid out natively
     (``ia_cache_pack_step``); the buffer returned is a copy of the native one."""
     n = len(entries)
     G = len(cache.groups)
@@ -122,7 +124,7 @@ def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optio
     rc = lib.ia_cache_pack_step(
         h, n, (ctypes.c_int64 * max(n, 1))(*cache.request_ids([e.request for e in entries])),
         (ctypes.c_int * max(n, 1))(*q_lens_in), tokens, (ctypes.c_int * max(n, 1))(*want_counts),
-        (ctypes.c_int32 * max(len(flat_wants), 1))(*flat_wants), int(bt_width or 0), PREFILL_TILE_ROWS, meta, meta_len)
+        (ctypes.c_int32 * max(len(flat_wants), 1))(*flat_wants), int(bt_width or 0), int(tile_rows) if tile_rows > 0 else (1 << 30), meta, meta_len)
     if rc != 0:
         cache._fail()
     m = meta[:]
@@ -137,4 +139,4 @@ def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optio
     host = np.frombuffer(buf, dtype=np.int32)
     batch = [entries[i] for i in order]
     return PackedStep(host, offsets, sizes, [(n, c) for c in cols], batch, [q_lens_in[i] for i in order], ctx_lens,
-                      num_decode, num_tiles, num_rows)
+                      num_decode, num_tiles, num_rows, int(tile_rows))

@@ -57,8 +57,14 @@ class Engine:
         self.cache = CacheManager(model.cache_needs(), [e.cache_of for e in model.spec.schedule], cache_config,
                                   dtype=self.rt.dtype, device=self.rt.device)
         self.views = self.cache.views()
+        # row tiles that parts asked for: one height is laid out with the step's arrays, further ones are
+        # made when a part asks (StepContext.row_tiles)
+        heights = sorted(model.step_needs().get("row_tiles", ()))
+        self._tile_rows = int(heights[0]) if heights else 0
         self.steps_run = 0
-        self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and model.graph_safe()
+        from ..kernels.api import profiling
+        self.use_graphs = (bool(use_graphs) and self.rt.device.type == "cuda" and model.graph_safe()
+                           and not profiling())         # a replayed launch has no call to time
         self._graphs: Dict[tuple, _DecodeGraph] = {}
         self._shape_seen: Dict[tuple, int] = {}
         self._graph_pool = None
@@ -102,8 +108,10 @@ class Engine:
     def from_config(cls, config: Any, seed: int = 0, dtype: Any = "bfloat16",
                     cache_config: Optional[CacheConfig] = None, device: Any = "cuda:0",
                     spec_kw: Optional[Dict[str, Any]] = None, use_graphs: bool = True,
-                    **runtime_kw: Any) -> "Engine":
-        """Random weights made on the device from (config, seed); nothing is read or written."""
+                    stored_as: Any = None, **runtime_kw: Any) -> "Engine":
+        """Random weights made on the device from (config, seed); nothing is read or written.  They are the
+        numbers of the folder that ``write_random_model`` writes from the same seed in ``stored_as`` (default:
+        the compute type)."""
         from .. import models  # noqa: F401
         from ..config.registry import model_spec_for
         from ..weights.random_init import random_weights_on_device
@@ -111,7 +119,8 @@ class Engine:
         rt = cls.runtime(dtype, device, **runtime_kw)
         load_library("core")
         model = DecoderModel(model_spec_for(config, **(spec_kw or {})), rt)
-        random_weights_on_device(model, seed)
+        stored = {None: None, "bfloat16": torch.bfloat16, "float32": torch.float32}.get(stored_as, stored_as)
+        random_weights_on_device(model, seed, stored)
         eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs)
         eng.config = config
         return eng
@@ -145,7 +154,7 @@ class Engine:
             if all(n == 1 for n in q_lens):
                 logits = self._decode_step(entries)
             else:
-                packed = pack_step(cache, entries)
+                packed = pack_step(cache, entries, tile_rows=self._tile_rows)
                 ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
                 logits = self.model.forward(ctx, self.views)
         except BaseException:
@@ -165,10 +174,10 @@ class Engine:
         kernels are told that width as the longest length, so that a shape's launches are the same from
         step to step, recorded or not."""
         cache = self.cache
-        packed = pack_step(cache, entries, bt_width=POW2_WIDTH)
-        width = packed.bt_shapes[0][1] if packed.bt_shapes else None
-        limit = (width or 0) * cache.page_size
-        key = (len(entries), width, packed.num_logit_rows)
+        packed = pack_step(cache, entries, bt_width=POW2_WIDTH, tile_rows=self._tile_rows)
+        widths = tuple(shape[1] for shape in packed.bt_shapes)           # one width per group of the cache
+        limit = max(widths, default=0) * cache.page_size
+        key = (len(entries), widths, packed.num_logit_rows)
         g = self._graphs.get(key)
         if g is not None:
             self._graphs[key] = self._graphs.pop(key)       # most recently used last

@@ -8,8 +8,12 @@ built library a call raises :class:`KernelError`.
 """
 from __future__ import annotations
 
+import atexit
 import ctypes
-from typing import Dict, Optional, Sequence
+import functools
+import os
+import sys
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -480,6 +484,9 @@ def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[t
         "attention_decode_rotating")
 
 
+PREFILL_TILE_ROWS = 64      # query rows of a workgroup's tile in attention_prefill
+
+
 def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
                       tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, d: int, scale: float,
@@ -487,7 +494,7 @@ def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     """bf16 causal attention of portions of prompts over their pages, on MFMA.
 
     Request s brings rows seq_starts[s] .. seq_starts[s+1]-1 of qkv and had seq_ctx[s] tokens cached
-    before; tiles[i] = (s, first row of a block of 64 among the request's rows).  ``heads_per_workgroup``:
+    before; tiles[i] = (s, first row of a block of PREFILL_TILE_ROWS among the request's rows).  ``heads_per_workgroup``:
     0 for the kernel's own choice, or 1, 2, 4 (see :func:`prefill_heads_per_workgroup`); the result has the
     same bits whichever is taken.
     """
@@ -586,3 +593,89 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 def attention_mfma_available(d: int) -> bool:
     """Whether the MFMA attention kernels take head size d (their library is built at its first use)."""
     return d in _build.SUPPORTED_HEAD_DIMS
+
+
+# ------------------------------------------------- time per kernel, by the device's clock
+# INFERNUM_PROFILE=1 in the environment (or ``set_profile(True)``): every call of a kernel function of this
+# module is bracketed by two events on its stream, and a table of calls and device time per function goes to
+# standard error when the process ends (``profile_report`` gives it at any time).  The reference's switch of the
+# same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
+# are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
+_PROFILED = ("embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
+             "gemm_library", "gemm_skinny", "attention_generic", "attention_decode", "attention_decode_rotating",
+             "attention_prefill", "argmax", "repetition_penalty", "sample")
+_profile_on = False
+_profile_open: List[Tuple[str, "torch.cuda.Event", "torch.cuda.Event"]] = []
+_profile_sum: Dict[str, List[float]] = {}          # function -> [calls, milliseconds]
+_plain = {name: globals()[name] for name in _PROFILED}
+
+
+def _fold_profile() -> None:
+    if _profile_open:
+        torch.cuda.synchronize()
+        for name, a, b in _profile_open:
+            acc = _profile_sum.setdefault(name, [0, 0.0])
+            acc[0] += 1
+            acc[1] += a.elapsed_time(b)
+        _profile_open.clear()
+
+
+def _timed(name: str, fn):
+    @functools.wraps(fn)
+    def call(*args, **kw):
+        if not _profile_on or torch.cuda.is_current_stream_capturing():
+            return fn(*args, **kw)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        try:
+            return fn(*args, **kw)
+        finally:
+            b.record()
+            _profile_open.append((name, a, b))
+            if len(_profile_open) >= 4096:
+                _fold_profile()
+    return call
+
+
+for _name in _PROFILED:
+    globals()[_name] = _timed(_name, _plain[_name])
+
+
+def profiling() -> bool:
+    return _profile_on
+
+
+def set_profile(on: bool) -> bool:
+    """Switch the timing of every kernel call on or off; returns what it was.  Engines made while it is on
+    do not record their decode steps into graphs."""
+    global _profile_on
+    before, _profile_on = _profile_on, bool(on)
+    return before
+
+
+def profile_report(reset: bool = False) -> Dict[str, Tuple[int, float]]:
+    """function -> (calls, milliseconds on the device) since the start or the last reset."""
+    _fold_profile()
+    out = {k: (int(v[0]), float(v[1])) for k, v in _profile_sum.items()}
+    if reset:
+        _profile_sum.clear()
+    return out
+
+
+def _print_profile() -> None:
+    try:
+        rep = profile_report()
+    except Exception:                                   # the device is gone at exit: nothing to print
+        return
+    if not rep:
+        return
+    total = sum(ms for _, ms in rep.values())
+    print(f"[infernum_amd profile] {total:.3f} ms in {sum(c for c, _ in rep.values())} kernel calls", file=sys.stderr)
+    for name, (calls, ms) in sorted(rep.items(), key=lambda kv: -kv[1][1]):
+        print(f"[infernum_amd profile] {name:28s} {calls:8d} calls {ms:12.3f} ms {ms / calls * 1e3:10.1f} us/call "
+              f"{100 * ms / total:5.1f} %", file=sys.stderr)
+
+
+if os.environ.get("INFERNUM_PROFILE") == "1":
+    _profile_on = True
+atexit.register(_print_profile)

@@ -25,10 +25,11 @@ class DecoderModel:
         self.blocks: List[Block] = []
         for ls in spec.layers:
             mixer = self._make("mixer", ls.mixer)
-            ff = self._make("feed_forward", ls.feed_forward)
-            n1 = self._make("norm", ls.mixer_norm)
-            n2 = self._make("norm", ls.feed_forward_norm)
-            extra = {name: self._make("norm", ps) for name, ps in ls.extra.items()}
+            ff = self._make("feed_forward", ls.feed_forward) if ls.feed_forward is not None else None
+            n1 = self._make("norm", ls.mixer_norm) if ls.mixer_norm is not None else None
+            n2 = self._make("norm", ls.feed_forward_norm) if ls.feed_forward_norm is not None else None
+            extra = {name: (self._make("norm", ps) if isinstance(ps, PartSpec) else self._make(*ps))
+                     for name, ps in ls.extra.items()}
             self.blocks.append(block_factory(ls.block)(rt, mixer, ff, n1, n2, extra))
         self.final_norm = self._make("norm", spec.final_norm) if spec.final_norm is not None else None
         self.head = self._make("head", spec.head)
@@ -78,6 +79,14 @@ class DecoderModel:
             wanted = part.weights()
             if wanted:
                 part.load({local: tensors[prefix + local] for local in wanted})
+
+    def step_needs(self) -> Dict[str, set]:
+        """What the parts want packed with every step: kind of array -> the set of its parameters."""
+        out: Dict[str, set] = {}
+        for _, part in self._parts:
+            for kind, param in part.step_needs().items():
+                out.setdefault(kind, set()).add(param)
+        return out
 
     # ---- cache needs ---------------------------------------------------------
     def cache_needs(self) -> List[Tuple[Optional[CacheSpec], Optional[StateSpec]]]:

@@ -77,6 +77,10 @@ class Attention(Mixer):
     def cache_spec(self) -> CacheSpec:
         return CacheSpec("window" if self.window else "full", self.nkv, self.d, self.window)
 
+    def step_needs(self) -> Dict[str, Any]:
+        # the MFMA kernel for portions of prompts works on tiles of 64 query rows
+        return {"row_tiles": K.PREFILL_TILE_ROWS} if self.use_mfma else {}
+
     def weights(self) -> Dict[str, WeightSpec]:
         nh, nkv, d, H = self.nh, self.nkv, self.d, self.hidden_size
         init = ("normal", self.init_std)
@@ -143,8 +147,9 @@ class Attention(Mixer):
             if hpw is None:             # once per step for all layers of this shape
                 hpw = ctx.extras[key] = K.prefill_heads_per_workgroup(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:],
                                                                       self.window, qkv.device)
+            tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
             K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
-                                ctx.prefill_tiles, ctx.num_prefill_tiles, nh, nkv, d, self.scale, self.window, hpw)
+                                tiles, num_tiles, nh, nkv, d, self.scale, self.window, hpw)
 
 
 register_part("mixer", "attention", Attention)

@@ -45,14 +45,46 @@ class WeightSpec:
 
 
 @dataclass(frozen=True)
+class PageTensor:
+    """One tensor of a page's payload.  ``shape`` is what one token stores; the page holds ``page_size`` tokens
+    along a new axis put in at ``token_axis``: the pool is [num_pages, *shape[:token_axis], page_size,
+    *shape[token_axis:]].  ``dtype`` None: the compute type."""
+
+    name: str
+    shape: Tuple[int, ...]
+    token_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def pool_shape(self, num_pages: int, page_size: int) -> Tuple[int, ...]:
+        if not 0 <= self.token_axis <= len(self.shape):
+            raise ValueError(f"page tensor {self.name!r}: token_axis {self.token_axis} is outside its shape {self.shape}")
+        return (num_pages,) + tuple(self.shape[:self.token_axis]) + (page_size,) + tuple(self.shape[self.token_axis:])
+
+
+@dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer needs of the paged cache: keys and values of all positions
-    ('full') or of the last ``window`` positions ('window')."""
+    """What a mixer needs of the paged cache: which positions are kept (all of them, 'full', or the last
+    ``window``, 'window'), and what a page holds for them (``payload``: named tensors with a per-token shape).
+    With ``num_kv_heads`` and ``head_dim`` and no payload it is keys and values as the attention kernels read
+    them: "k" [nkv, page_size, d] and "v", transposed within the page, [nkv, d, page_size]."""
 
     kind: str                      # "full" | "window"
-    num_kv_heads: int
-    head_dim: int
+    num_kv_heads: int = 0
+    head_dim: int = 0
     window: int = 0
+    payload: Tuple[PageTensor, ...] = ()
+
+    def __post_init__(self) -> None:
+        if not self.payload:
+            if self.num_kv_heads <= 0 or self.head_dim <= 0:
+                raise ValueError("a CacheSpec needs a payload, or num_kv_heads and head_dim for keys and values")
+            object.__setattr__(self, "payload", (
+                PageTensor("k", (self.num_kv_heads, self.head_dim), token_axis=1),
+                # values are kept transposed within a page: what the PV product of the matrix cores reads
+                PageTensor("v", (self.num_kv_heads, self.head_dim), token_axis=2)))
+        names = [t.name for t in self.payload]
+        if len(set(names)) != len(names):
+            raise ValueError(f"page tensors of one CacheSpec need different names, got {names}")
 
     def group_key(self) -> Tuple:
         """Layers with equal keys share page tables (one group of the cache manager)."""
@@ -69,14 +101,16 @@ class StateSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: how its parts are arranged (``block``) and the parts themselves."""
+    """One layer: how its parts are arranged (``block``) and the parts themselves.  An arrangement that has no
+    use for one of the four leaves it None; what it needs beyond them goes into ``extra`` under names of its
+    own: a PartSpec (a norm), or (category, PartSpec) for a part of any category."""
 
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
-    extra: Mapping[str, PartSpec] = field(default_factory=dict)   # further norms of other arrangements
+    feed_forward: Optional[PartSpec] = None
+    mixer_norm: Optional[PartSpec] = None
+    feed_forward_norm: Optional[PartSpec] = None
+    extra: Mapping[str, Any] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -131,17 +165,25 @@ class Runtime:
 class CacheView:
     """What one run of a layer sees of the cache.
 
-    k_pages/v_pages: [num_pages, nkv, page_size, d] of its schedule entry (or of
-    the entry it reads); ``group`` indexes the step's block tables and slots;
-    ``writable`` is False when the pages belong to another entry.  ``state`` is
-    the entry's [num_slots, *shape] tensor when the mixer declared a StateSpec.
+    ``pages``: the pools of its schedule entry (or of the entry it reads) by the names of the mixer's
+    CacheSpec payload, each [num_pages, ...] with the page's tokens along the declared axis; ``k_pages`` and
+    ``v_pages`` are the "k" and "v" of them.  ``group`` indexes the step's block tables and slots;
+    ``writable`` is False when the pages belong to another entry.  ``state`` is the entry's
+    [num_slots, *shape] tensor when the mixer declared a StateSpec.
     """
 
     group: int = -1
-    k_pages: Optional[torch.Tensor] = None
-    v_pages: Optional[torch.Tensor] = None
+    pages: Mapping[str, torch.Tensor] = field(default_factory=dict)
     writable: bool = True
     state: Optional[torch.Tensor] = None
+
+    @property
+    def k_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("v")
 
 
 @dataclass
@@ -170,9 +212,22 @@ class StepContext:
     ctx_lens: Sequence[int] = ()
     max_q_len: int = 0
     max_total_len: int = 0                  # largest ctx + q over the batch
-    prefill_tiles: Optional[torch.Tensor] = None   # [n_tiles, 2] int32 (request, first row) for tiled attention
-    num_prefill_tiles: int = 0
+    # lists of row tiles by tile height, as far as the step's packing made them (see ``row_tiles``)
+    packed_row_tiles: Dict[int, Tuple[torch.Tensor, int]] = field(default_factory=dict)
     extras: Dict[str, Any] = field(default_factory=dict)
+
+    def row_tiles(self, rows: int) -> Tuple[torch.Tensor, int]:
+        """The portions of prompts of this step cut into tiles of ``rows`` rows: an int32 tensor [n, 2] of
+        (request, first row of the tile among the request's rows) on the device, and n.  A part that wants
+        them says so in ``step_needs`` ({"row_tiles": rows}); then they came with the step's one copy.
+        Otherwise they are made here, once per step and height, and copied over."""
+        hit = self.packed_row_tiles.get(rows)
+        if hit is None:
+            pairs = [(s, first) for s in range(self.num_decode, self.num_seqs)
+                     for first in range(0, self.q_lens[s], rows)]
+            t = torch.tensor(pairs or [(0, 0)], dtype=torch.int32).to(self.token_ids.device)
+            hit = self.packed_row_tiles[rows] = (t, len(pairs))
+        return hit
 
 
 # ------------------------------------------------------------------ interfaces
@@ -195,6 +250,11 @@ class Part:
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Take the tensors of ``weights`` (by local name), already on the device."""
+
+    def step_needs(self) -> Dict[str, Any]:
+        """Arrays that the part wants packed with every step beyond those every step has.  Known:
+        ``{"row_tiles": rows}``: the list of :meth:`StepContext.row_tiles` for that height."""
+        return {}
 
 
 class Norm(Part):
@@ -262,8 +322,8 @@ class Block:
     category = "block"
     graph_safe = False
 
-    def __init__(self, rt: Runtime, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 feed_forward_norm: Norm, extra: Mapping[str, Part]):
+    def __init__(self, rt: Runtime, mixer: Mixer, feed_forward: Optional[FeedForward], mixer_norm: Optional[Norm],
+                 feed_forward_norm: Optional[Norm], extra: Mapping[str, Part]):
         self.rt = rt
         self.mixer = mixer
         self.feed_forward = feed_forward

@@ -134,8 +134,10 @@ def write_random_model(config: Any, out_dir: str, seed: int, dtype: torch.dtype 
     return out_dir
 
 
-def random_weights_on_device(model, seed: int) -> None:
-    """Fill a model with random weights made on its own device (nothing is written)."""
+def random_weights_on_device(model, seed: int, stored_as: Optional[torch.dtype] = None) -> None:
+    """Fill a model with random weights made on its own device (nothing is written): the model that loading
+    the folder of ``write_random_model(dtype=stored_as)`` would give; ``stored_as`` defaults to the model's
+    compute type (a 32-bit model with ``stored_as=torch.bfloat16`` holds the numbers of the bfloat16 one)."""
     rt: Runtime = model.rt
     expected = model.expected_weights()
     tensors: Dict[str, torch.Tensor] = {}
@@ -144,7 +146,7 @@ def random_weights_on_device(model, seed: int) -> None:
             continue                              # shares its fallback's buffer, below
         # what loading the folder that write_random_model(dtype=rt.dtype) writes would give: every tensor
         # rounded to that type once, also those that do not follow the compute type
-        tensors[name] = draw(spec, seed, name, rt.device).to(rt.dtype)
+        tensors[name] = draw(spec, seed, name, rt.device).to(stored_as or rt.dtype).to(rt.dtype)
     for name, spec in expected.items():          # a tied head whose fallback sorts after it
         if name not in tensors:
             tensors[name] = tensors[spec.fallback]

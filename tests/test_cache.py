@@ -235,3 +235,38 @@ def test_a_step_that_fails_leaves_the_cache_as_it_was():
         assert cache.slots.num_free == 2
         cache.check()
     assert eng.steps_run == 0
+
+
+def test_pools_are_what_the_mixers_declare():
+    """A page's payload comes from the mixer's CacheSpec: named tensors with a per-token shape and the axis
+    that the page's tokens run along; keys and values in the attention kernels' layouts are the default."""
+    import torch
+    from infernum_amd.parts import CacheSpec, PageTensor
+    latent = CacheSpec("window", window=6, payload=(PageTensor("latent", (12,), 0, torch.float32),
+                                                    PageTensor("scale", (), 0)))
+    kv = CacheSpec("full", 2, 16)
+    assert [(t.name, t.shape, t.token_axis) for t in kv.payload] == [("k", (2, 16), 1), ("v", (2, 16), 2)]
+    m = CacheManager([(latent, None), (kv, None), (None, None)], [None, None, 1],
+                     CacheConfig(page_size=4, num_pages=8, poison_freed_pages=True), dtype=torch.bfloat16,
+                     device=torch.device("cpu"))
+    shapes = [{k: (tuple(v.shape), v.dtype) for k, v in p.items()} for p in m.pages]
+    assert shapes == [{"latent": ((8, 4, 12), torch.float32), "scale": ((8, 4), torch.bfloat16)},
+                      {"k": ((8, 2, 4, 16), torch.bfloat16), "v": ((8, 2, 16, 4), torch.bfloat16)}, {}]
+    views = m.views()
+    assert views[0].k_pages is None and views[0].pages["latent"] is m.pages[0]["latent"]
+    assert views[2].pages is views[1].pages and not views[2].writable and views[2].k_pages is m.pages[1]["k"]
+    # freed pages are poisoned in every pool of their group
+    m.admit("a")
+    assert m.reserve("a", 9)
+    m.commit("a", 9)
+    pages = {g: m.block_table(g, "a").pages for g in range(2)}
+    m.release("a")
+    assert all(bool(m.pages[0]["latent"][p].isnan().all()) and bool(m.pages[0]["scale"][p].isnan().all())
+               for p in pages[0] if p >= 0)
+    assert all(bool(m.pages[1]["k"][p].isnan().all()) for p in pages[1])
+    with pytest.raises(ValueError):
+        CacheSpec("full")
+    with pytest.raises(ValueError):
+        CacheSpec("full", payload=(PageTensor("x", (3,)), PageTensor("x", (4,))))
+    with pytest.raises(ValueError):
+        PageTensor("x", (3,), token_axis=2).pool_shape(4, 4)

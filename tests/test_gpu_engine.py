@@ -260,3 +260,27 @@ def test_recorded_decode_steps_equal_eager_ones(models, name, dtype):
     got = {(r, fed[r] - 1): graphed.step([StepEntry(r, reqs[r][fed[r]:fed[r] + 1], [0])])[0].cpu() for r in names[:1]}
     _check({(names[0], fed[names[0]]): got[(names[0], fed[names[0]] - 1)]}, ref, dtype, f"{name} {dtype} recorded decode",
            every_place=False)
+
+
+def test_time_per_kernel_switch(models):
+    """INFERNUM_PROFILE=1 / set_profile: every kernel call is timed on the device and summed by function; an
+    engine made meanwhile records no graphs; the logits are those of an engine without it."""
+    from infernum_amd.kernels import api as K
+    d, cfg, reqs, ref = models[("B", "bfloat16")]
+    plain = TT.run_steps(_engine(d, "bfloat16", 8, 64), TT.trace_tail_one_by_one(reqs, 8))
+    before = K.set_profile(True)
+    try:
+        K.profile_report(reset=True)
+        eng = _engine(d, "bfloat16", 8, 64)
+        assert not eng.use_graphs
+        timed = TT.run_steps(eng, TT.trace_tail_one_by_one(reqs, 8))
+        rep = K.profile_report(reset=True)
+    finally:
+        K.set_profile(before)
+    assert all(torch.equal(plain[k], timed[k]) for k in plain)
+    steps = len(TT.trace_tail_one_by_one(reqs, 8))
+    layers = cfg["num_hidden_layers"]
+    assert rep["embed"][0] == steps and rep["add_rmsnorm"][0] == steps * (2 * layers + 1)
+    assert {"attention_decode_rotating", "attention_prefill", "gemm_skinny", "rope_kv_append"} <= set(rep)
+    assert all(calls > 0 and ms > 0 for calls, ms in rep.values())
+    assert K.profile_report() == {}

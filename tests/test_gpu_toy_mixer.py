@@ -331,3 +331,154 @@ def test_routed_feed_forward_and_another_position_encoding(tmp_path):
         worst, rms, where = TT.error_against(got, ref)
         print(f"toy2 {name}: {worst / rms:.2e} at {where}")
         assert worst == worst and worst <= 3e-5 * rms, (name, worst / rms, where)
+
+
+# ------------------------------------------------------------------------------------------------
+# A mixer whose pages hold one tensor of its own (a latent per token instead of keys and values), in an
+# arrangement of its own (mixer and two feed-forwards side by side on one norm): again without a change to
+# the framework's files.
+from infernum_amd.parts import Block, CacheSpec, PageTensor        # noqa: E402
+
+
+class LatentMixer(Mixer):
+    """c_t = W_c x_t is what a token leaves in the cache (``rank`` numbers);
+    y_t = W_o sum_j softmax_j(<W_q x_t, c_j> / sqrt(rank)) c_j over the tokens j <= t of the request (the last
+    ``window`` of them when a window is set)."""
+
+    def __init__(self, rt, hidden_size, rank, window=0):
+        super().__init__(rt)
+        self.H, self.r, self.window = hidden_size, rank, window
+
+    def cache_spec(self):
+        return CacheSpec("window" if self.window else "full", window=self.window,
+                         payload=(PageTensor("latent", (self.r,), token_axis=0, dtype=torch.float32),))
+
+    def weights(self):
+        return {"c_proj.weight": WeightSpec((self.r, self.H), ("normal", 0.2)),
+                "q_proj.weight": WeightSpec((self.r, self.H), ("normal", 0.2)),
+                "o_proj.weight": WeightSpec((self.H, self.r), ("normal", 0.2))}
+
+    def load(self, tensors):
+        self.t = tensors
+
+    def forward(self, x, ctx, cache):
+        pool = cache.pages["latent"]                       # [num_pages, page_size, rank]
+        assert cache.k_pages is None and pool.dtype == torch.float32 and pool.shape[2] == self.r
+        ps, g = pool.shape[1], cache.group
+        flat = pool.view(-1, self.r)
+        if cache.writable:                                 # else: the latents of another run of a layer are read
+            flat[ctx.slots[g].long()] = x.float() @ self.t["c_proj.weight"].float().t()
+        q = x.float() @ self.t["q_proj.weight"].float().t()
+        out = torch.empty_like(q)
+        tables = ctx.block_tables[g].tolist()
+        row = 0
+        for b, (n, before) in enumerate(zip(ctx.q_lens, ctx.ctx_lens)):
+            for i in range(n):
+                t = before + i
+                first = max(0, t - self.window + 1) if self.window else 0
+                where = torch.tensor([tables[b][p // ps] * ps + p % ps for p in range(first, t + 1)], device=x.device)
+                assert int(where.min()) >= 0, "a position inside the window has no page"
+                c = flat[where]
+                s = torch.softmax(c @ q[row] / math.sqrt(self.r), dim=0)
+                out[row] = s @ c
+                row += 1
+        return (out @ self.t["o_proj.weight"].float().t()).to(x.dtype)
+
+
+class SideBySideBlock(Block):
+    """h += mixer(n) + feed_forward(n) + second(n) with n = norm(h): one norm, nothing in a row."""
+
+    def forward(self, h, pending, ctx, cache):
+        n = self.mixer_norm.forward(h, pending)
+        parts = [self.mixer.forward(n, ctx, cache), self.feed_forward.forward(n, ctx),
+                 self.extra["second"].forward(n, ctx)]
+        parts = [p.joined(n.dtype) if hasattr(p, "joined") else p for p in parts]
+        return (parts[0].float() + parts[1].float() + parts[2].float()).to(n.dtype)
+
+
+@dataclass(frozen=True)
+class Toy3Config:
+    vocab_size: int = 61
+    hidden_size: int = 40
+    rank: int = 12
+    intermediate_size: int = 56
+    window: int = 7
+    model_type: str = "toy-latent"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return Toy3Config(**{k: v for k, v in raw.items() if k in Toy3Config.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy3_spec(cfg: Toy3Config) -> ModelSpec:
+    H = cfg.hidden_size
+    norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "init": ("uniform", 0.5, 1.5)}, prefix)
+    ff = lambda prefix: PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size,
+                                            "init_std": 0.1}, prefix)
+    layers = [LayerSpec("side_by_side",
+                        PartSpec("latent", {"hidden_size": H, "rank": cfg.rank, "window": w}, f"l.{i}.mix."),
+                        ff(f"l.{i}.ff."), norm(f"l.{i}.n."), None,
+                        extra={"second": ("feed_forward", ff(f"l.{i}.ff2."))})
+              for i, w in enumerate((0, cfg.window))]
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.5}, "emb."),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_of=0)],
+                     final_norm=norm("fn."),
+                     head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.1}, "head."))
+
+
+def plain_forward3(cfg: Toy3Config, w, ids):
+    W = {k: v.double() for k, v in w.items()}
+    T = len(ids)
+    h = P.embedding(W["emb.weight"], ids)
+    kept = {}
+    for run, (l, reads) in enumerate(((0, None), (1, None), (0, 0))):
+        n = P.rms_norm(h, W[f"l.{l}.n.weight"], 1e-5)
+        if reads is None:
+            kept[run] = P.linear(n, W[f"l.{l}.mix.c_proj.weight"])
+        c = kept[run if reads is None else reads]
+        q = P.linear(n, W[f"l.{l}.mix.q_proj.weight"])
+        window = cfg.window if l == 1 else 0
+        a = torch.zeros_like(q)
+        for t in range(T):
+            first = max(0, t - window + 1) if window else 0
+            s = torch.softmax(c[first:t + 1] @ q[t] / math.sqrt(cfg.rank), dim=0)
+            a[t] = s @ c[first:t + 1]
+        delta = P.linear(a, W[f"l.{l}.mix.o_proj.weight"])
+        for f in ("ff", "ff2"):
+            delta = delta + P.linear(P.swiglu(P.linear(n, W[f"l.{l}.{f}.gate_proj.weight"]),
+                                              P.linear(n, W[f"l.{l}.{f}.up_proj.weight"])),
+                                     W[f"l.{l}.{f}.down_proj.weight"])
+        h = h + delta
+    return P.linear(P.rms_norm(h, W["fn.weight"], 1e-5), W["head.weight"])
+
+
+def test_a_mixer_with_a_page_payload_of_its_own_in_an_arrangement_of_its_own(tmp_path):
+    register_part("mixer", "latent", LatentMixer, replace=True)
+    register_part("block", "side_by_side", SideBySideBlock, replace=True)
+    register_architecture("toy-latent", Toy3Config, toy3_spec, replace=True)
+    cfg = Toy3Config()
+    d = write_random_model(cfg, str(tmp_path / "toy3"), seed=12, dtype=torch.float32)
+    _, w = P.read_model(d)
+    eng = Engine.from_pretrained(d, dtype="float32", cache_config=CacheConfig(page_size=4, num_pages=40,
+                                                                              num_state_slots=4, poison_freed_pages=True))
+    # two groups (all positions; a window of 7), pools as the mixer declared them, the third run reads the first's
+    assert [(g.kind, g.window) for g in eng.cache.groups] == [("full", 0), ("window", cfg.window)]
+    assert [sorted(p) for p in eng.cache.pages] == [["latent"], ["latent"], []]
+    assert tuple(eng.cache.pages[0]["latent"].shape) == (40, 4, cfg.rank)
+    assert eng.views[2].pages is eng.views[0].pages and not eng.views[2].writable
+    assert eng.model.step_needs() == {} and not eng.use_graphs
+    reqs = TT.make_requests(cfg.vocab_size, (33, 6, 50, 21), seed=3)
+    ref = {r: plain_forward3(cfg, w, t) for r, t in reqs.items()}
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=2)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy3 {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= 3e-5 * rms, (name, worst / rms, where)
+        eng.cache.check()
+        assert all(g.allocator.num_free == 40 for g in eng.cache.groups)

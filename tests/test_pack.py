@@ -6,7 +6,9 @@ import numpy as np
 import pytest
 
 from infernum_amd.cache import NO_PAGE, CacheConfig, CacheManager, PageError
-from infernum_amd.engine.batch import POW2_WIDTH, PREFILL_TILE_ROWS, StepEntry, pack_step
+from infernum_amd.engine.batch import POW2_WIDTH, StepEntry, pack_step
+
+PREFILL_TILE_ROWS = 64
 from infernum_amd.parts import CacheSpec
 
 FULL = CacheSpec("full", 2, 16)
@@ -85,7 +87,7 @@ def test_native_packing_equals_plain_packing(seed):
             while width < max(len(cache.block_table(g, e.request).pages) for g in range(len(needs)) for e in entries):
                 width *= 2
         # the native side finds that power of two itself when asked to
-        packed = pack_step(cache, entries, bt_width=POW2_WIDTH if width and step % 2 else width)
+        packed = pack_step(cache, entries, bt_width=POW2_WIDTH if width and step % 2 else width, tile_rows=PREFILL_TILE_ROWS)
         batch, q, ctx, want = plain_pack(cache, entries, width)
         assert [e.request for e in packed.batch] == [e.request for e in batch]
         assert packed.q_lens == q and packed.ctx_lens == ctx
