@@ -46,7 +46,7 @@ CORE_SOURCES = [
 ]
 HEADERS = ["common.h", "no_alloc.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
-HOST_SOURCES = ["host_core.cpp"]
+HOST_SOURCES = ["host_core.cpp", "step_program.cpp"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 # The binding of the vendor's GEMM library (hipBLASLt): host code too, against ROCm's headers and libraries.
 BLASLT_SOURCES = ["gemm_library.cpp"]

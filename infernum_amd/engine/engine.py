@@ -13,6 +13,7 @@ int32 buffer, copies it to the device once, and runs the model's forward pass.
 """
 from __future__ import annotations
 
+import os
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
 import torch
@@ -50,7 +51,8 @@ class Engine:
     the graph's own input buffer first; pages, state and weights are where they always are.  Models with a
     part that is not marked ``graph_safe`` (one that reads device memory on the host, say) run without."""
 
-    def __init__(self, model: DecoderModel, cache_config: CacheConfig, use_graphs: bool = True):
+    def __init__(self, model: DecoderModel, cache_config: CacheConfig, use_graphs: bool = True,
+                 executor: Optional[str] = None):
         self.model = model
         self.rt: Runtime = model.rt
         self.spec = model.spec
@@ -70,6 +72,16 @@ class Engine:
         self._graph_pool = None
         self.graph_replays = 0
         self.max_recorded_steps = MAX_RECORDED_STEPS
+        # "native": the step's launches are made by the host library from one call where every part of the
+        # model has a native description (engine/program.py); "parts": by the parts' own forward, one Python
+        # call per launch.  The same launches either way.
+        executor = executor or os.environ.get("INFERNUM_EXECUTOR", "native")
+        if executor not in ("native", "parts"):
+            raise ValueError(f"executor must be 'native' or 'parts', got {executor!r}")
+        self.program = None
+        if executor == "native" and self.rt.device.type == "cuda":
+            from .program import build
+            self.program = build(model, self.views, self.rt.max_tokens_per_step)
 
     # ---- building ------------------------------------------------------------------
     @staticmethod
@@ -87,7 +99,8 @@ class Engine:
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: Any = "bfloat16", cache_config: Optional[CacheConfig] = None,
-                        device: Any = "cuda:0", use_graphs: bool = True, **runtime_kw: Any) -> "Engine":
+                        device: Any = "cuda:0", use_graphs: bool = True, executor: Optional[str] = None,
+                        **runtime_kw: Any) -> "Engine":
         """Model class by config.json's model_type, weights from the folder's safetensors.
         ``kernels="generic"`` (a runtime keyword) runs every matrix product and the attention on the plain
         twins of the fast kernels, in either type."""
@@ -100,7 +113,7 @@ class Engine:
         config = load_config(model_dir)
         model = DecoderModel(model_spec_for(config), rt)
         load_weights(model, model_dir)
-        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs)
+        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs, executor=executor)
         eng.config = config
         return eng
 
@@ -108,7 +121,7 @@ class Engine:
     def from_config(cls, config: Any, seed: int = 0, dtype: Any = "bfloat16",
                     cache_config: Optional[CacheConfig] = None, device: Any = "cuda:0",
                     spec_kw: Optional[Dict[str, Any]] = None, use_graphs: bool = True,
-                    stored_as: Any = None, **runtime_kw: Any) -> "Engine":
+                    stored_as: Any = None, executor: Optional[str] = None, **runtime_kw: Any) -> "Engine":
         """Random weights made on the device from (config, seed); nothing is read or written.  They are the
         numbers of the folder that ``write_random_model`` writes from the same seed in ``stored_as`` (default:
         the compute type)."""
@@ -121,7 +134,7 @@ class Engine:
         model = DecoderModel(model_spec_for(config, **(spec_kw or {})), rt)
         stored = {None: None, "bfloat16": torch.bfloat16, "float32": torch.float32}.get(stored_as, stored_as)
         random_weights_on_device(model, seed, stored)
-        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs)
+        eng = cls(model, cache_config or CacheConfig(), use_graphs=use_graphs, executor=executor)
         eng.config = config
         return eng
 
@@ -156,7 +169,7 @@ class Engine:
             else:
                 packed = pack_step(cache, entries, tile_rows=self._tile_rows)
                 ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
-                logits = self.model.forward(ctx, self.views)
+                logits = self._forward(ctx)
         except BaseException:
             # the step did not run to its end: requests that came with it leave again, the others give back
             # the pages that were reserved for it; what earlier steps stored stays as it was
@@ -168,6 +181,13 @@ class Engine:
         cache.commit_step(reqs, q_lens, arrays)
         self.steps_run += 1
         return logits
+
+    def _forward(self, ctx) -> torch.Tensor:
+        if self.program is not None:
+            from ..kernels.api import on_current_stream
+            with on_current_stream():
+                return self.program.run(ctx)
+        return self.model.forward(ctx, self.views)
 
     def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Every request brings one token.  Block tables are widened to a power of two of pages, and the
@@ -191,7 +211,7 @@ class Engine:
         ctx = packed.context(inputs)
         ctx.max_total_len = max(limit, ctx.max_total_len)
         if not self.use_graphs or seen < 1:
-            return self.model.forward(ctx, self.views)
+            return self._forward(ctx)
         # second time this shape comes: record it (kernels were loaded by the first, eager run)
         while len(self._graphs) >= self.max_recorded_steps:
             oldest = next(iter(self._graphs))
@@ -200,7 +220,7 @@ class Engine:
         torch.cuda.synchronize(self.rt.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self._graph_pool):
-            logits = self.model.forward(ctx, self.views)
+            logits = self._forward(ctx)
         if self._graph_pool is None:
             self._graph_pool = graph.pool()
         self._graphs[key] = _DecodeGraph(inputs, graph, logits)

@@ -282,6 +282,14 @@ LIBRARY_WORKSPACE_BYTES = 128 << 20
 _library_workspace: Dict[torch.device, torch.Tensor] = {}
 
 
+def library_workspace(device: torch.device) -> torch.Tensor:
+    """The one workspace of the library's products on a device."""
+    ws = _library_workspace.get(device)
+    if ws is None:
+        ws = _library_workspace[device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return ws
+
+
 def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[M, N] = a[M, K] @ w[N, K]^T by the vendor's library (hipBLASLt), called directly: bf16 with fp32
     accumulation, or fp32 throughout.  The library's choice of an algorithm is asked once per shape and kept,
@@ -296,9 +304,7 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] =
     if out is None:
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
     _need(out.dtype == a.dtype and tuple(out.shape) == (M, N), f"gemm_library: out must be {a.dtype} [{M}, {N}]")
-    ws = _library_workspace.get(a.device)
-    if ws is None:
-        ws = _library_workspace[a.device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+    ws = library_workspace(a.device)
     lib = load_library("blaslt")
     code = lib.ia_gemm_lt(_p(a), _p(w), _p(out), M, N, K, DTYPE_CODE[a.dtype], _p(ws), ctypes.c_size_t(ws.numel()),
                           _stream())

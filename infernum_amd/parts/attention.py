@@ -130,6 +130,15 @@ class Attention(Mixer):
         self.attend(q, out, ctx, cache)
         return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
+    def native(self, program, view: CacheView) -> bool:
+        from . import rope
+        if type(self) is not Attention or type(self.position) not in (rope.RotaryEmbedding, rope.NoPositionEncoding):
+            return False                      # a subclass may do something else in forward
+        if view is None or view.k_pages is None or view.v_pages is None:
+            return False
+        program.add_attention(self, view)
+        return True
+
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d
         bt = ctx.block_tables[cache.group]

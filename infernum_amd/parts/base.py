@@ -251,6 +251,11 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Take the tensors of ``weights`` (by local name), already on the device."""
 
+    def native(self, program: Any, view: Optional["CacheView"], **kw: Any) -> bool:
+        """Add this part to the native program of a step (``engine.program.StepProgram``) as the operation that
+        makes the launches of ``forward``; False when it has none (the model then runs through the parts)."""
+        return False
+
     def step_needs(self) -> Dict[str, Any]:
         """Arrays that the part wants packed with every step beyond those every step has.  Known:
         ``{"row_tiles": rows}``: the list of :meth:`StepContext.row_tiles` for that height."""
@@ -334,6 +339,11 @@ class Block:
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
                 cache: CacheView) -> torch.Tensor:
         raise NotImplementedError
+
+    def native(self, program: Any, view: CacheView) -> bool:
+        """Add the arrangement's parts to the native program in the order ``forward`` runs them; False when
+        the arrangement or one of its parts has no native description."""
+        return False
 
 
 # -------------------------------------------------------------------- registry

@@ -24,5 +24,12 @@ class PreNormBlock(Block):
         n = self.feed_forward_norm.forward(h, a)
         return self.feed_forward.forward(n, ctx)
 
+    def native(self, program, view: CacheView) -> bool:
+        if type(self) is not PreNormBlock or self.extra or None in (self.feed_forward, self.mixer_norm,
+                                                                    self.feed_forward_norm):
+            return False
+        return (self.mixer_norm.native(program, None) and self.mixer.native(program, view)
+                and self.feed_forward_norm.native(program, None) and self.feed_forward.native(program, None))
+
 
 register_part("block", "prenorm", PreNormBlock)

@@ -36,6 +36,9 @@ class TokenEmbedding(Embedding):
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
         return K.embed(self.table, ctx.token_ids, h)
 
+    def native(self, program, view) -> bool:
+        return type(self) is TokenEmbedding       # the program reads ``table`` itself
+
 
 class LinearHead(Head):
     graph_safe = True
@@ -55,6 +58,12 @@ class LinearHead(Head):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
+
+    def native(self, program, view) -> bool:
+        if type(self) is not LinearHead:
+            return False
+        program.set_head(self.weight)
+        return True
 
 
 register_part("embedding", "token", TokenEmbedding)

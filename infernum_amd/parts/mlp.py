@@ -40,4 +40,11 @@ class SwiGLUFeedForward(FeedForward):
         return linear(act, self.w_down, keep_split=True, kernels=self.rt.kernels)
 
 
+    def native(self, program, view) -> bool:
+        if type(self) is not SwiGLUFeedForward:
+            return False
+        program.add_swiglu(self.w_gate_up, self.w_down)
+        return True
+
+
 register_part("feed_forward", "swiglu", SwiGLUFeedForward)

@@ -39,4 +39,11 @@ class RMSNorm(Norm):
         return K.add_rmsnorm(h, delta, self.weight, self.eps, out, rows)
 
 
+    def native(self, program, view, final: bool = False) -> bool:
+        if type(self) is not RMSNorm:
+            return False
+        program.add_norm(self.weight, self.eps, final=final)
+        return True
+
+
 register_part("norm", "rmsnorm", RMSNorm)

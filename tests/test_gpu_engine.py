@@ -284,3 +284,28 @@ def test_time_per_kernel_switch(models):
     assert {"attention_decode_rotating", "attention_prefill", "gemm_skinny", "rope_kv_append"} <= set(rep)
     assert all(calls > 0 and ms > 0 for calls, ms in rep.values())
     assert K.profile_report() == {}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_native_program_makes_the_launches_of_the_parts(models, name, dtype):
+    """A step run by the host library from one call (the default where every part has a native description)
+    gives the bits of the same step run by the parts' own forward, launch by launch from Python: whole prompts,
+    portions, single tokens (rotation inside the attention kernel), mixed steps, with pages used again."""
+    d, cfg, reqs, ref = models[(name, dtype, "mixed")]
+    prompt_len = {r: max(2, len(t) - 20) for r, t in reqs.items()}
+    mixed, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=5)
+    traces = (TT.trace_whole(reqs), TT.trace_portions(reqs), mixed)
+    native = _engine(d, dtype, PAGE[name], max_tokens // PAGE[name])
+    parts = _engine(d, dtype, PAGE[name], max_tokens // PAGE[name], executor="parts")
+    assert native.program is not None and parts.program is None
+    assert len(native.program.attentions) == cfg["num_hidden_layers"]
+    for steps in traces:
+        a, b = TT.run_steps(native, steps), TT.run_steps(parts, steps)
+        assert a.keys() == b.keys()
+        for k in a:
+            assert torch.equal(a[k], b[k]), k
+    for kernels in ("generic",):
+        a = TT.run_steps(_engine(d, dtype, PAGE[name], 64, kernels=kernels), TT.trace_portions(reqs))
+        b = TT.run_steps(_engine(d, dtype, PAGE[name], 64, kernels=kernels, executor="parts"), TT.trace_portions(reqs))
+        assert all(torch.equal(a[k], b[k]) for k in a)
