@@ -55,8 +55,9 @@ _SIGNATURES = {
     "ia_program_set_rotation": (None, [c_void_p, c_int]),
     "ia_program_set_functions": (c_int, [c_void_p, POINTER(c_void_p), c_int]),
     "ia_program_add_norm": (c_int, [c_void_p, c_void_p, c_int, c_float, c_int]),
-    "ia_program_add_attention": (c_int, [c_void_p, POINTER(c_int), c_int, c_float, POINTER(c_void_p), c_int]),
-    "ia_program_add_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
+    "ia_program_add_attention": (c_int, [c_void_p, POINTER(c_int), c_int, c_float, POINTER(c_void_p), c_int,
+                                         POINTER(c_int)]),
+    "ia_program_add_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "ia_program_set_head": (c_int, [c_void_p, c_void_p]),
     "ia_program_finish": (c_size_t, [c_void_p, c_int]),
     "ia_program_set_arena": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),

@@ -58,6 +58,7 @@ enum { FN_EMBED, FN_ADD_RMSNORM, FN_ROPE_KV_APPEND, FN_SWIGLU, FN_GEMM_GENERIC, 
 struct Weight {          // a matrix [N, K] in the activations' type
   const void* w = nullptr;
   int N = 0, K = 0, splits = 1;      // splits: parts of K in the weight-streaming product (a function of N, K)
+  int library_rows = -1;             // measured: bit b set = 16 b + 1 .. 16 b + 16 rows go to the library; -1: the rule
 };
 
 struct Op {
@@ -154,7 +155,9 @@ int linear(Program* p, const Step& s, const void* x, int M, const Weight& w, int
     rc = ((fn_gemm_generic)p->fns[FN_GEMM_GENERIC])(x, w.w, y, in_dtype, out_dtype, M, N, K, K, K, N, s.stream);
     if (rc) return fail(p, rc, "gemm_generic");
   } else if (skinny_supported(M, N, K) &&
-             (M <= p->skinny_rows_any_width || N < p->skinny_wide || out_dtype != DT_BF16)) {
+             (out_dtype != DT_BF16 ||
+              (w.library_rows >= 0 ? !((w.library_rows >> ((M - 1) / 16)) & 1)
+                                   : (M <= p->skinny_rows_any_width || N < p->skinny_wide)))) {
     fn_gemm_skinny skinny = (fn_gemm_skinny)p->fns[FN_GEMM_SKINNY];
     const size_t ws_floats = w.splits > 1 ? (size_t)w.splits * M * N : 0;
     if (keep_split && epilogue == EPI_NONE && w.splits > 1) {
@@ -414,7 +417,9 @@ int ia_program_add_norm(void* h, const void* weight, int weight_dtype, float eps
 // attention: pending = attention(x).  ints: [nh, nkv, d, window, rot, freq_f64, group, writable, use_mfma,
 // page_size, num_pages]; ptrs: [w_qkv, w_o, inv_freq or null, k_pages, v_pages, ia_attn_decode,
 // ia_attn_decode_fused, ia_attn_prefill (the three may be null without use_mfma)]
-int ia_program_add_attention(void* h, const int* ints, int n_ints, float scale, void* const* ptrs, int n_ptrs) {
+// library_rows: the measured choice of a product for the qkv, the queries-only and the output weight (see Weight)
+int ia_program_add_attention(void* h, const int* ints, int n_ints, float scale, void* const* ptrs, int n_ptrs,
+                             const int* library_rows) {
   Program* p = static_cast<Program*>(h);
   if (n_ints != 11 || n_ptrs != 8) return fail(p, ERR_BAD_ARG, "attention");
   Op op;
@@ -430,6 +435,9 @@ int ia_program_add_attention(void* h, const int* ints, int n_ints, float scale, 
   if (rc) return rc;
   rc = set_weight(p, &op.o, ptrs[1], p->H, op.nh * op.d);
   if (rc) return rc;
+  op.qkv.library_rows = library_rows[0];
+  op.q_only.library_rows = library_rows[1];
+  op.o.library_rows = library_rows[2];
   op.inv_freq = ptrs[2];
   op.k_pages = ptrs[3];
   op.v_pages = ptrs[4];
@@ -444,7 +452,8 @@ int ia_program_add_attention(void* h, const int* ints, int n_ints, float scale, 
 }
 
 // SwiGLU feed-forward: pending = down(silu(gate(x)) * up(x)); gate and up are one matrix [2 I, H]
-int ia_program_add_swiglu(void* h, const void* w_gate_up, const void* w_down, int I) {
+int ia_program_add_swiglu(void* h, const void* w_gate_up, const void* w_down, int I, int gate_up_library_rows,
+                          int down_library_rows) {
   Program* p = static_cast<Program*>(h);
   Op op;
   op.kind = OP_SWIGLU_FF;
@@ -452,6 +461,8 @@ int ia_program_add_swiglu(void* h, const void* w_gate_up, const void* w_down, in
   if (rc) return rc;
   rc = set_weight(p, &op.down, w_down, p->H, I);
   if (rc) return rc;
+  op.gate_up.library_rows = gate_up_library_rows;
+  op.down.library_rows = down_library_rows;
   p->ops.push_back(op);
   return 0;
 }

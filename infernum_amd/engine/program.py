@@ -103,15 +103,25 @@ class StepProgram:
         for name in ("ia_attn_decode", "ia_attn_decode_fused", "ia_attn_prefill"):
             ptrs.append(_fn(lib, name) if lib is not None else ctypes.c_void_p(0))
         self._keep += [part.w_qkv, part.w_o, inv_freq, k, v]
+        masks = (ctypes.c_int * 3)(self._route(part.w_qkv, None, True),
+                                   self._route(part.w_qkv[: part.nh * part.d], None, True),
+                                   self._route(part.w_o, None, True))
         self._check(self._lib.ia_program_add_attention(self._h, ints, 11, ctypes.c_float(part.scale),
-                                                       (ctypes.c_void_p * 8)(*ptrs), 8))
+                                                       (ctypes.c_void_p * 8)(*ptrs), 8, masks))
         self.attentions.append({"nh": part.nh, "nkv": part.nkv, "d": part.d, "window": part.window,
                                 "mfma": int(part.use_mfma and k.shape[2] % 4 == 0),
                                 "rotates": int(part.rotate_in_attention)})
 
+    @staticmethod
+    def _route(w: torch.Tensor, epilogue: Optional[str], keep_split: bool) -> int:
+        """The measured choice between the two products for this weight and use (parts/linear.py)."""
+        return linear_part.library_rows(w.shape[0], w.shape[1], epilogue, keep_split)
+
     def add_swiglu(self, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> None:
         self._keep += [w_gate_up, w_down]
-        self._check(self._lib.ia_program_add_swiglu(self._h, _ptr(w_gate_up), _ptr(w_down), w_down.shape[1]))
+        self._check(self._lib.ia_program_add_swiglu(self._h, _ptr(w_gate_up), _ptr(w_down), w_down.shape[1],
+                                                    self._route(w_gate_up, "swiglu", False),
+                                                    self._route(w_down, None, True)))
 
     def set_head(self, weight: torch.Tensor) -> None:
         self._keep.append(weight)
