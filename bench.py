@@ -228,6 +228,44 @@ def serve(a) -> int:
     return 0
 
 
+def long_contexts(a) -> int:
+    """Further points of the 8B shape: decode at batch 8 with 16,384 and 32,768 tokens of context, and the prefill of
+    one prompt of 8,192 and of 16,384 tokens in a single step.  One JSON line of its own."""
+    import torch
+    from infernum_amd import CacheConfig, Engine, LlamaConfig
+    from infernum_amd.engine import StepEntry
+    cfg = LlamaConfig.from_dict(dict(LLAMA_8B))
+    batch, longest = 8, 32768
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens_per_step=16384,
+                                cache_config=CacheConfig(page_size=PAGE_SIZE, num_state_slots=batch + 1,
+                                                         num_pages=batch * (longest + 64 + PAGE_SIZE) // PAGE_SIZE + 8))
+    out = {"metric": "long contexts, Llama-3-8B shape", "dtype": "bf16", "data": "synthetic", "batch": batch, "decode": {},
+           "prefill": {}}
+    for ctx_len in (16384, 32768):
+        steps = 32
+        dt, ctx_mid = time_decode(engine, batch, steps, 4, ctx_len)
+        gbs = decode_bytes(cfg, ctx_mid) / (dt / steps) / 1e9
+        out["decode"][str(ctx_len)] = {"tokens_per_s": round(batch * steps / dt, 1), "ms_per_step": round(dt / steps * 1e3, 3),
+                                       "gb_per_s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    g = torch.Generator().manual_seed(7)
+    for T in (8192, 16384):
+        prompt = torch.randint(0, cfg.vocab_size, (T,), generator=g).tolist()
+        best = None
+        for i in range(3):
+            sync()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(f"long{i}", prompt, [T - 1])])
+            sync()
+            t = time.perf_counter() - t0
+            engine.end(f"long{i}")
+            if i > 0:
+                best = t if best is None else min(best, t)
+        out["prefill"][str(T)] = {"tokens_per_s": round(T / best, 1), "ms": round(best * 1e3, 2),
+                                  "frac": round(prefill_flops(cfg, T) / best / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +282,8 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every request's prompt")
     ap.add_argument("--peaks", action="store_true",
                     help="only measure this GPU's streaming read bandwidth and bf16 matrix rate; a JSON line of its own")
+    ap.add_argument("--long", action="store_true",
+                    help="decode at 16k and 32k tokens of context and prefills of 8k and 16k tokens instead (a JSON line of its own)")
     ap.add_argument("--no-fp32-check", action="store_true", help="skip the comparison with the 32-bit path")
     ap.add_argument("--serve", action="store_true",
                     help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
@@ -258,6 +298,8 @@ def main() -> int:
 
     if a.serve:
         return serve(a)
+    if a.long:
+        return long_contexts(a)
     if a.peaks:
         from infernum_amd.peaks import measure
         print(json.dumps(measure()))

@@ -516,3 +516,54 @@ extern "C" int ia_swiglu(const void* gu, void* out, int act_dtype, int N, int I,
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// ------------------------------------------------------------ utilities: casts, copies of pages
+// dst[i] = src[i] in another type: fp32 -> bf16 rounds to nearest even, bf16 -> fp32 is exact
+// (the reference: infernum-cuda/kernels/cast.cu).
+template <typename TS, typename TD>
+__global__ __launch_bounds__(256) void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = from_float<TD>(to_float(src[i]));
+}
+
+extern "C" int ia_cast(const void* src, int src_dtype, void* dst, int dst_dtype, size_t n, hipStream_t stream) {
+  if ((src_dtype != IA_F32 && src_dtype != IA_BF16) || (dst_dtype != IA_F32 && dst_dtype != IA_BF16)) return IA_ERR_BAD_ARG;
+  if (n == 0) return IA_OK;
+  if (!src || !dst) return IA_ERR_BAD_ARG;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (src_dtype == IA_F32 && dst_dtype == IA_BF16)
+    cast_kernel<float, bf16_t><<<grid, 256, 0, stream>>>((const float*)src, (bf16_t*)dst, n);
+  else if (src_dtype == IA_BF16 && dst_dtype == IA_F32)
+    cast_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((const bf16_t*)src, (float*)dst, n);
+  else if (src_dtype == IA_F32)
+    cast_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, n);
+  else
+    cast_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)src, (bf16_t*)dst, n);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// Pages of a pool copied within it: page dst_pages[i] = page src_pages[i], page_bytes each (a multiple of 4).
+// A pair with a page outside [0, num_pages) is left out.  Pairs must not overlap each other's targets.
+__global__ __launch_bounds__(256) void copy_pages_kernel(uint32_t* __restrict__ pool, size_t page_words,
+                                                         const int* __restrict__ src_pages,
+                                                         const int* __restrict__ dst_pages, int num_pages) {
+  const int s = src_pages[blockIdx.y], d = dst_pages[blockIdx.y];
+  if (s < 0 || s >= num_pages || d < 0 || d >= num_pages || s == d) return;
+  const uint32_t* from = pool + (size_t)s * page_words;
+  uint32_t* to = pool + (size_t)d * page_words;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < page_words; i += stride) to[i] = from[i];
+}
+
+extern "C" int ia_copy_pages(void* pool, size_t page_bytes, int num_pages, const int* src_pages, const int* dst_pages,
+                             int n, hipStream_t stream) {
+  if (!pool || page_bytes == 0 || (page_bytes & 3) || num_pages <= 0 || n < 0 || n > 65535) return IA_ERR_BAD_ARG;
+  if (n == 0) return IA_OK;
+  if (!src_pages || !dst_pages) return IA_ERR_BAD_ARG;
+  const size_t words = page_bytes / 4;
+  dim3 grid((unsigned)((words + 255) / 256 < 64 ? (words + 255) / 256 : 64), (unsigned)n);
+  copy_pages_kernel<<<grid, 256, 0, stream>>>((uint32_t*)pool, words, src_pages, dst_pages, num_pages);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}

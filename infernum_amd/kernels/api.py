@@ -234,6 +234,32 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def cast(src: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``src`` in another of the two types (fp32 to bf16 rounds to nearest even; bf16 to fp32 is exact)."""
+    _dev(src, out)
+    _need(src.dtype in DTYPE_CODE and dtype in DTYPE_CODE, "cast: fp32 and bf16 only")
+    if out is None:
+        out = torch.empty(src.shape, dtype=dtype, device=src.device)
+    _need(out.dtype == dtype and out.numel() == src.numel(), "cast: out must have src's size and the asked type")
+    _ok(_core().ia_cast(_p(src), DTYPE_CODE[src.dtype], _p(out), DTYPE_CODE[dtype], ctypes.c_size_t(src.numel()),
+                        _stream()), "cast")
+    return out
+
+
+def copy_pages(pool: torch.Tensor, src_pages: torch.Tensor, dst_pages: torch.Tensor) -> None:
+    """pool[dst_pages[i]] = pool[src_pages[i]] for a pool [num_pages, ...]; pairs with a page outside the pool
+    are left out.  The targets must differ from each other and from every source."""
+    _dev(pool, src_pages, dst_pages)
+    n = src_pages.numel()
+    _need(pool.dim() >= 2 and pool.shape[0] > 0, "copy_pages: a pool [num_pages, ...]")
+    _i32(src_pages, n, "copy_pages sources")
+    _i32(dst_pages, n, "copy_pages targets")
+    page_bytes = pool[0].numel() * pool.element_size()
+    _need(page_bytes % 4 == 0 and n <= 65535, "copy_pages: pages of a multiple of 4 bytes, at most 65,535 pairs")
+    _ok(_core().ia_copy_pages(_p(pool), ctypes.c_size_t(page_bytes), pool.shape[0], _p(src_pages), _p(dst_pages), n,
+                              _stream()), "copy_pages")
+
+
 # ------------------------------------------------------------------ matrix products
 def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[M, N] = a[M, K] @ w[N, K]^T with fp32 multiply-adds in the order of k."""
@@ -607,7 +633,7 @@ def attention_mfma_available(d: int) -> bool:
 # standard error when the process ends (``profile_report`` gives it at any time).  The reference's switch of the
 # same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
 # are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
-_PROFILED = ("embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
+_PROFILED = ("cast", "copy_pages", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
              "gemm_library", "gemm_skinny", "attention_generic", "attention_decode", "attention_decode_rotating",
              "attention_prefill", "argmax", "repetition_penalty", "sample")
 _profile_on = False

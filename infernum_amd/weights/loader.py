@@ -47,7 +47,13 @@ def _convert(t: torch.Tensor, spec: WeightSpec, rt: Runtime) -> torch.Tensor:
     else:
         target = torch.bfloat16
     # on the device, so that a large matrix is converted there and the host copy stays mapped
-    return t.to(device=rt.device).to(target).contiguous()
+    t = t.to(device=rt.device).contiguous()
+    if t.dtype == target:
+        return t
+    if t.is_cuda and t.dtype in (torch.float32, torch.bfloat16):
+        from ..kernels import api as K
+        return K.cast(t, target)
+    return t.to(target).contiguous()                # float16 and float64 files, and hosts without a GPU
 
 
 def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], where: str) -> Dict[str, str]:

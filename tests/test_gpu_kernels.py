@@ -828,3 +828,30 @@ def test_sample_limits_and_frequencies():
     srt, idx = torch.sort(p, descending=True)
     n_keep = int(torch.nonzero(torch.cumsum(srt, 0) >= 0.5)[0]) + 1
     assert set(outs.tolist()) <= set(idx[:n_keep].tolist())
+
+
+# ------------------------------------------------------------------- utilities
+def test_cast_rounds_to_nearest_even_and_widens_exactly():
+    g = torch.Generator().manual_seed(3)
+    x = torch.cat([torch.randn(100003, generator=g) * 7.0,
+                   torch.tensor([0.0, -0.0, 1.0, 1.00390625, 1.01171875, float("inf"), -float("inf"), 3.0e38, 1e-40])]).to(DEV)
+    down = K().cast(x, torch.bfloat16)
+    assert down.dtype == torch.bfloat16 and torch.equal(down, x.to(torch.bfloat16))      # ties to even, as the library
+    up = K().cast(down, torch.float32)
+    assert torch.equal(up, down.float())
+    assert torch.isnan(K().cast(torch.tensor([float("nan")], device=DEV), torch.bfloat16)).all()
+    same = K().cast(x, torch.float32)
+    assert torch.equal(same, x) and same.data_ptr() != x.data_ptr()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_copy_pages(dtype):
+    pool = _rand(9, 3, 5, 6, dtype=dtype)              # pages of 90 values: no multiple of a thread block
+    before = pool.clone()
+    src = torch.tensor([0, 2, 7, 99, 4, -1], dtype=torch.int32, device=DEV)
+    dst = torch.tensor([1, 3, 8, 5, 4, 6], dtype=torch.int32, device=DEV)
+    K().copy_pages(pool, src, dst)
+    want = before.clone()
+    for s, d in ((0, 1), (2, 3), (7, 8)):              # a pair with a page outside the pool, or onto itself, is left out
+        want[d] = before[s]
+    assert torch.equal(pool, want)
