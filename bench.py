@@ -288,8 +288,8 @@ def main() -> int:
     ap.add_argument("--serve", action="store_true",
                     help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
     ap.add_argument("--serve-requests", type=int, default=128)
-    ap.add_argument("--serve-batch", type=int, default=64)
-    ap.add_argument("--serve-chunk", type=int, default=1024)
+    ap.add_argument("--serve-batch", type=int, default=128)
+    ap.add_argument("--serve-chunk", type=int, default=2048)
     ap.add_argument("--serve-blocks", type=int, default=16384)
     a = ap.parse_args()
     if a.gpus != 1:
