@@ -52,7 +52,8 @@ class Attention(Mixer):
     graph_safe = True
     def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[Mapping[str, Any]] = None, window: Optional[int] = None,
-                 scale: Optional[float] = None, kernels: str = "auto", init_std: float = 0.02):
+                 scale: Optional[float] = None, kernels: str = "auto", init_std: float = 0.02,
+                 qk_transform: Optional[Mapping[str, Any]] = None):
         super().__init__(rt)
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
@@ -67,6 +68,15 @@ class Attention(Mixer):
         self.init_std = init_std
         pos_spec = PartSpec(**position) if isinstance(position, Mapping) else (position or PartSpec("none"))
         self.position = make_part("position", pos_spec, rt)
+        # an optional part of category "qk_transform" that works on the projected heads before the rotation;
+        # with one, steps of single tokens take the separate kernels too (the fused one rotates what it projects)
+        self.qk_transform = None
+        if qk_transform is not None:
+            spec = PartSpec(**qk_transform) if isinstance(qk_transform, Mapping) else qk_transform
+            self.qk_transform = make_part("qk_transform", spec, rt)
+        # recordable into a graph only when the parts inside are
+        self.graph_safe = (getattr(self.position, "graph_safe", False)
+                           and (self.qk_transform is None or getattr(self.qk_transform, "graph_safe", False)))
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
         self.rotate_in_attention = _decode_rotation == "attention"
@@ -84,12 +94,18 @@ class Attention(Mixer):
     def weights(self) -> Dict[str, WeightSpec]:
         nh, nkv, d, H = self.nh, self.nkv, self.d, self.hidden_size
         init = ("normal", self.init_std)
-        return {
+        own = {
             "q_proj.weight": WeightSpec((nh * d, H), init),
             "k_proj.weight": WeightSpec((nkv * d, H), init),
             "v_proj.weight": WeightSpec((nkv * d, H), init),
             "o_proj.weight": WeightSpec((H, nh * d), init),
         }
+        if self.qk_transform is not None:
+            extra = self.qk_transform.weights()
+            if set(extra) & set(own):
+                raise ValueError(f"the qk_transform's tensors {sorted(set(extra) & set(own))} have the attention's names")
+            own.update(extra)
+        return own
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
@@ -97,6 +113,8 @@ class Attention(Mixer):
         self.w_o = tensors["o_proj.weight"].contiguous()
         measure_routes_for(self.rt, [(self.w_qkv, None, True), (self.w_qkv[: self.nh * self.d], None, True),
                                      (self.w_o, None, True)])
+        if self.qk_transform is not None:
+            self.qk_transform.load({name: tensors[name] for name in self.qk_transform.weights()})
 
     # ---- one step --------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView):
@@ -104,7 +122,7 @@ class Attention(Mixer):
         if cache.k_pages is None:
             raise K.KernelError("attention needs pages of the cache")
         g = cache.group
-        if (self.use_mfma and self.rotate_in_attention and 0 < ctx.num_decode == x.shape[0]
+        if (self.use_mfma and self.rotate_in_attention and 0 < ctx.num_decode == x.shape[0] and self.qk_transform is None
                 and x.shape[0] <= ROTATE_IN_ATTENTION_UP_TO and cache.k_pages.shape[2] % 4 == 0):
             # every request brings one token: rotation, the write to the pages and attention are one launch
             w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
@@ -115,7 +133,15 @@ class Attention(Mixer):
                                         ctx.block_tables[g], nh, nkv, d, self.scale, self.window, ctx.max_total_len)
             return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
         q_out = None
-        if cache.writable:
+        if self.qk_transform is not None:
+            w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
+            qkv = self.qk_transform.forward(linear(x, w, kernels=self.rt.kernels), nh, nkv if cache.writable else 0, d, ctx)
+            if cache.writable:
+                q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
+                                     ctx.slots[g], cache.k_pages, cache.v_pages)
+            else:
+                q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim)
+        elif cache.writable:
             qkv = linear(x, self.w_qkv, keep_split=True, kernels=self.rt.kernels)
             if isinstance(qkv, K.SplitSum):
                 q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
@@ -136,6 +162,8 @@ class Attention(Mixer):
         from . import rope
         if type(self) is not Attention or type(self.position) not in (rope.RotaryEmbedding, rope.NoPositionEncoding):
             return False                      # a subclass may do something else in forward
+        if self.qk_transform is not None:
+            return False                      # a part of the model's own between projection and rotation
         if view is None or view.k_pages is None or view.v_pages is None:
             return False
         program.add_attention(self, view)

@@ -277,6 +277,21 @@ class PositionEncoding(Part):
     category = "position"
 
 
+class QKTransform(Part):
+    """What an attention mixer may do to its projected queries and keys before they are rotated and the keys
+    are written to the cache (a norm per head, a bias, a scale): the seam between projection and rotation."""
+
+    category = "qk_transform"
+
+    def forward(self, qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                ctx: "StepContext") -> torch.Tensor:
+        """qkv [N, (num_q_heads + 2 num_kv_heads) head_dim] in the compute dtype: the query heads, then the key
+        heads, then the value heads of every token (num_kv_heads is 0 for a run that reads another run's keys
+        and values: then the rows hold queries only).  Returns the tensor to go on with (it may be qkv itself,
+        changed in place)."""
+        raise NotImplementedError
+
+
 class Mixer(Part):
     category = "mixer"
 

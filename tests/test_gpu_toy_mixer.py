@@ -482,3 +482,115 @@ def test_a_mixer_with_a_page_payload_of_its_own_in_an_arrangement_of_its_own(tmp
         assert worst == worst and worst <= 3e-5 * rms, (name, worst / rms, where)
         eng.cache.check()
         assert all(g.allocator.num_free == 40 for g in eng.cache.groups)
+
+
+# ------------------------------------------------------------------------------------------------
+# The seam between projection and rotation: a part of the test's own that normalises every query and key head
+# (with a weight per position of the head) before they are rotated and the keys are cached.
+from infernum_amd.parts import QKTransform        # noqa: E402
+
+
+class HeadNorm(QKTransform):
+    """q_h <- rmsnorm(q_h) * wq, k_h <- rmsnorm(k_h) * wk for every head h; values stay."""
+
+    def __init__(self, rt, head_dim, eps):
+        super().__init__(rt)
+        self.d, self.eps = head_dim, eps
+
+    def weights(self):
+        return {"q_norm.weight": WeightSpec((self.d,), ("uniform", 0.5, 1.5), follows_compute_dtype=False),
+                "k_norm.weight": WeightSpec((self.d,), ("uniform", 0.5, 1.5), follows_compute_dtype=False)}
+
+    def load(self, tensors):
+        self.wq, self.wk = tensors["q_norm.weight"].float(), tensors["k_norm.weight"].float()
+
+    def forward(self, qkv, num_q_heads, num_kv_heads, head_dim, ctx):
+        N = qkv.shape[0]
+        heads = qkv.float().view(N, -1, head_dim)
+        normed = heads * torch.rsqrt((heads * heads).mean(-1, keepdim=True) + self.eps)
+        out = heads.clone()
+        out[:, :num_q_heads] = normed[:, :num_q_heads] * self.wq
+        out[:, num_q_heads:num_q_heads + num_kv_heads] = normed[:, num_q_heads:num_q_heads + num_kv_heads] * self.wk
+        return out.view(N, -1).to(qkv.dtype)
+
+
+@dataclass(frozen=True)
+class Toy4Config:
+    vocab_size: int = 70
+    hidden_size: int = 64
+    num_heads: int = 4
+    num_kv_heads: int = 2
+    intermediate_size: int = 48
+    model_type: str = "toy-headnorm"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return Toy4Config(**{k: v for k, v in raw.items() if k in Toy4Config.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy4_spec(cfg: Toy4Config) -> ModelSpec:
+    H, d = cfg.hidden_size, cfg.hidden_size // cfg.num_heads
+    norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "init": ("uniform", 0.5, 1.5)}, prefix)
+    att = lambda prefix: PartSpec("attention", {
+        "hidden_size": H, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads, "head_dim": d, "init_std": 0.2,
+        "position": {"kind": "rope", "params": {"head_dim": d, "theta": 1000.0, "scaling": None}},
+        "qk_transform": {"kind": "head_norm", "params": {"head_dim": d, "eps": 1e-6}}}, prefix)
+    layers = [LayerSpec("prenorm", att(f"l.{i}.attn."),
+                        PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size,
+                                            "init_std": 0.1}, f"l.{i}.ff."), norm(f"l.{i}.n1."), norm(f"l.{i}.n2."))
+              for i in range(2)]
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.5}, "emb."),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, cache_of=1)],
+                     final_norm=norm("fn."),
+                     head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.1}, "head."))
+
+
+def plain_forward4(cfg: Toy4Config, w, ids):
+    W = {k: v.double() for k, v in w.items()}
+    H, nh, nkv = cfg.hidden_size, cfg.num_heads, cfg.num_kv_heads
+    d, T = H // nh, len(ids)
+    freqs, pos = P.rope_frequencies(d, 1000.0, None), torch.arange(T)
+    h = P.embedding(W["emb.weight"], ids)
+    kept = {}
+    for run, (l, reads) in enumerate(((0, None), (1, None), (1, 1))):
+        p = f"l.{l}.attn."
+        n = P.rms_norm(h, W[f"l.{l}.n1.weight"], 1e-5)
+        q = P.rms_norm(P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d), W[p + "q_norm.weight"], 1e-6)
+        if reads is None:
+            k = P.rms_norm(P.linear(n, W[p + "k_proj.weight"]).reshape(T, nkv, d), W[p + "k_norm.weight"], 1e-6)
+            kept[run] = (P.rope(k, pos, freqs), P.linear(n, W[p + "v_proj.weight"]).reshape(T, nkv, d))
+        k, v = kept[run if reads is None else reads]
+        a = P.causal_attention(P.rope(q, pos, freqs), k, v, 1.0 / math.sqrt(d)).reshape(T, H)
+        h = h + P.linear(a, W[p + "o_proj.weight"])
+        m = P.rms_norm(h, W[f"l.{l}.n2.weight"], 1e-5)
+        h = h + P.linear(P.swiglu(P.linear(m, W[f"l.{l}.ff.gate_proj.weight"]), P.linear(m, W[f"l.{l}.ff.up_proj.weight"])),
+                         W[f"l.{l}.ff.down_proj.weight"])
+    return P.linear(P.rms_norm(h, W["fn.weight"], 1e-5), W["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_part_between_projection_and_rotation(tmp_path, dtype):
+    register_part("qk_transform", "head_norm", HeadNorm, replace=True)
+    register_architecture("toy-headnorm", Toy4Config, toy4_spec, replace=True)
+    cfg = Toy4Config()
+    d = write_random_model(cfg, str(tmp_path / "toy4"), seed=21,
+                           dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    _, w = P.read_model(d)
+    assert "l.0.attn.q_norm.weight" in w and "l.1.attn.k_norm.weight" in w      # the transform's tensors, by name
+    eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=8, num_pages=40, num_state_slots=4,
+                                                                          poison_freed_pages=True))
+    assert eng.program is None and not eng.use_graphs           # the model's own part: through the parts, unrecorded
+    reqs = TT.make_requests(cfg.vocab_size, (29, 7, 44, 18), seed=5)
+    ref = {r: plain_forward4(cfg, w, t) for r, t in reqs.items()}
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=4)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy4 {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
