@@ -3,9 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
 
-One "step" is one decode step of the whole batch: every request brings its last
-token, the engine runs it against the paged cache, and the next token is chosen
-greedily on the device.  Requests start from a 512-token prompt (uniform random
+One "step" is one decode step of the whole batch through the generation loop
+(``Runtime.step``): every request brings its last token, the engine runs it
+against the paged cache, and the next token is chosen greedily on the device.  Requests start from a 512-token prompt (uniform random
 ids), as the reference measures decoding after a prompt
 (infernum-examples/examples/bench.rs:1049-1110).  The line printed at the end also
 holds the prefill of one 2,048-token prompt, decoding at batch 1 and 64, and the
@@ -72,40 +72,51 @@ def prefill_flops(cfg, T) -> float:
 
 
 class DecodeRun:
-    """B requests, each prefilled with a prompt, then decoded greedily step by step."""
+    """B requests through the generation loop itself (scheduler, step function, sampler: ``Runtime``): their
+    prompts go in in portions, then every call of ``step`` is one decode step of the whole batch, greedy, the
+    tokens chosen on the device (the loop launches a step while the tokens of the one before are still there)."""
 
-    def __init__(self, engine, batch: int, prompt_len: int, seed: int = 0):
+    def __init__(self, engine, batch: int, prompt_len: int, new_tokens: int, seed: int = 0):
         import torch
-        from infernum_amd.engine import StepEntry
+        from infernum_amd import BatchConfig, GenerateOptions, Runtime
+        from infernum_amd.engine.scheduler import SequencePhase
+        cc = engine.cache.config
+        chunk = min(2048, engine.rt.max_tokens_per_step - batch)
+        bc = BatchConfig(max_batch_size=batch, max_prefill_tokens=chunk, block_size=cc.page_size,
+                         num_blocks=cc.num_pages, max_tokens_per_step=chunk + batch)
         self.engine, self.batch = engine, batch
+        self.rt = Runtime(engine, None, bc)
         g = torch.Generator().manual_seed(seed)
         V = engine.spec.vocab_size
-        self.ids = [f"b{batch}_{i}" for i in range(batch)]
-        self.ctx = [0] * batch
-        last = []
-        for i, rid in enumerate(self.ids):
-            prompt = torch.randint(0, V, (prompt_len,), generator=g).tolist()
-            logits = None
-            for p in range(0, prompt_len, 2048):
-                chunk = prompt[p:p + 2048]
-                want = [len(chunk) - 1] if p + len(chunk) == prompt_len else []
-                logits = engine.step([StepEntry(rid, chunk, want)])
-            last.append(int(torch.argmax(logits[0])))
-            self.ctx[i] = prompt_len
-        self.last = last
+        self.seqs = [self.rt.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(),
+                                    GenerateOptions(max_new_tokens=new_tokens)) for _ in range(batch)]
+        while any(s.phase != SequencePhase.DECODE for s in self.seqs):
+            self.rt.step()
         sync()
 
+    @property
+    def ctx(self):
+        return [s.num_tokens for s in self.seqs]
+
     def step(self):
-        self.last = self.engine.decode_greedy(self.ids, self.last)
-        self.ctx = [c + 1 for c in self.ctx]
+        plan = self.rt.step()
+        assert len(plan.decode) == self.batch and not plan.prefill, "a decode step of the whole batch"
 
     def close(self):
-        for rid in self.ids:
-            self.engine.end(rid)
+        for s in self.seqs:
+            self.rt.scheduler.cancel(s)
+        self.rt.run()
+        sync()
+
+
+def prefill_steps(batch: int, prompt_len: int) -> int:
+    """Steps the prompts of a batch take to go in (portions of 2,048 tokens): the requests that went in first
+    decode meanwhile, so every request is given that many tokens more to generate."""
+    return -(-batch * prompt_len // 2048) + 8
 
 
 def time_decode(engine, batch, steps, warmup, prompt_len=PROMPT_LEN):
-    run = DecodeRun(engine, batch, prompt_len)
+    run = DecodeRun(engine, batch, prompt_len, new_tokens=warmup + steps + prefill_steps(batch, prompt_len) + 8)
     for _ in range(warmup):
         run.step()
     sync()
@@ -238,7 +249,8 @@ def long_contexts(a) -> int:
     batch, longest = 8, 32768
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens_per_step=16384,
                                 cache_config=CacheConfig(page_size=PAGE_SIZE, num_state_slots=batch + 1,
-                                                         num_pages=batch * (longest + 64 + PAGE_SIZE) // PAGE_SIZE + 8))
+                                                         num_pages=batch * (longest + 64 + prefill_steps(batch, longest)
+                                                                            + 2 * PAGE_SIZE) // PAGE_SIZE + 8))
     out = {"metric": "long contexts, Llama-3-8B shape", "dtype": "bf16", "data": "synthetic", "batch": batch, "decode": {},
            "prefill": {}}
     for ctx_len in (16384, 32768):
@@ -315,7 +327,8 @@ def main() -> int:
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
     max_batch = 1 if a.prefill_only else max(a.batch, 1 if a.no_points else 64)
-    tokens_needed = max(max_batch * (a.prompt_len + a.steps + a.warmup + PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
+    tokens_needed = max(max_batch * (a.prompt_len + a.steps + a.warmup + prefill_steps(max_batch, a.prompt_len)
+                                     + 2 * PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
     t_load = time.perf_counter()
     engine = Engine.from_config(cfg, seed=0, dtype=dtype,
                                 cache_config=CacheConfig(page_size=PAGE_SIZE,

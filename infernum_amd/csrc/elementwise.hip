@@ -567,3 +567,79 @@ extern "C" int ia_copy_pages(void* pool, size_t page_bytes, int num_pages, const
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// token_ids[i] = source[index[i]] where index[i] >= 0 (left as it is elsewhere): the tokens that the last step
+// chose on the device go into the next step's batch without a round trip to the host.
+__global__ __launch_bounds__(256) void gather_tokens_kernel(int* __restrict__ token_ids, const int* __restrict__ source,
+                                                            const int* __restrict__ index, int n, int source_len) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int j = index[i];
+  if (j >= 0 && j < source_len) token_ids[i] = source[j];
+}
+
+extern "C" int ia_gather_tokens(int* token_ids, const int* source, const int* index, int n, int source_len,
+                                hipStream_t stream) {
+  if (n < 0 || source_len < 0) return IA_ERR_BAD_ARG;
+  if (n == 0) return IA_OK;
+  if (!token_ids || !source || !index) return IA_ERR_BAD_ARG;
+  gather_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(token_ids, source, index, n, source_len);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ---- small arrays between pinned host memory and the device by kernels of the compute stream
+// (a copy by the DMA engines is ordered with the stream's kernels through signals between queues, which costs
+// a step of single tokens a tenth of a millisecond; a kernel that reads or writes the pinned memory itself does not)
+//
+// dst[i] = src[i] for i < n (4-byte words, src in pinned host memory); then, with nd > 0, the words
+// dst[token_off + r], r < nd, whose index src[index_off + r] is j >= 0 become source[j]: the tokens that the
+// last step chose on the device.
+__global__ __launch_bounds__(256) void words_from_host_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src,
+                                                              int n, int token_off, int nd,
+                                                              const int* __restrict__ source, int source_len,
+                                                              int index_off) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  uint32_t v = src[i];
+  const int r = i - token_off;
+  if (r >= 0 && r < nd) {
+    const int j = (int)src[index_off + r];
+    if (j >= 0 && j < source_len) v = (uint32_t)source[j];
+  }
+  dst[i] = v;
+}
+
+__global__ __launch_bounds__(256) void words_to_host_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src,
+                                                            int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+// host_src: pinned host memory (hipHostMalloc) of at least max(n, index_off + nd) words
+extern "C" int ia_words_from_host(void* dst, const void* host_src, int n, int token_off, int nd, const int* source,
+                                  int source_len, int index_off, hipStream_t stream) {
+  if (n < 0 || nd < 0 || (nd > 0 && (!source || token_off < 0 || token_off + nd > n || index_off < 0))) return IA_ERR_BAD_ARG;
+  if (n == 0) return IA_OK;
+  if (!dst || !host_src) return IA_ERR_BAD_ARG;
+  void* dev_view = nullptr;
+  hipError_t e = hipHostGetDevicePointer(&dev_view, const_cast<void*>(host_src), 0);
+  if (e != hipSuccess) return (int)e;
+  words_from_host_kernel<<<(n + 255) / 256, 256, 0, stream>>>((uint32_t*)dst, (const uint32_t*)dev_view, n, token_off, nd,
+                                                             source, source_len, index_off);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// host_dst: pinned host memory of at least n words; src on the device
+extern "C" int ia_words_to_host(void* host_dst, const void* src, int n, hipStream_t stream) {
+  if (n < 0) return IA_ERR_BAD_ARG;
+  if (n == 0) return IA_OK;
+  if (!host_dst || !src) return IA_ERR_BAD_ARG;
+  void* dev_view = nullptr;
+  hipError_t e = hipHostGetDevicePointer(&dev_view, host_dst, 0);
+  if (e != hipSuccess) return (int)e;
+  words_to_host_kernel<<<(n + 255) / 256, 256, 0, stream>>>((uint32_t*)dev_view, (const uint32_t*)src, n);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}

@@ -51,6 +51,7 @@ class PackedStep:
     num_tiles: int
     num_logit_rows: int
     tile_rows: int = 0                   # height of the row tiles that were packed (0: none)
+    order: Sequence[int] = ()            # row r of the batch is entry order[r] of the step
 
     def context(self, dev: torch.Tensor) -> StepContext:
         """The step as the parts see it, over ``dev``, the device copy of ``host``."""
@@ -139,4 +140,4 @@ def pack_step(cache: CacheManager, entries: Sequence[StepEntry], bt_width: Optio
     host = np.frombuffer(buf, dtype=np.int32)
     batch = [entries[i] for i in order]
     return PackedStep(host, offsets, sizes, [(n, c) for c in cols], batch, [q_lens_in[i] for i in order], ctx_lens,
-                      num_decode, num_tiles, num_rows, int(tile_rows))
+                      num_decode, num_tiles, num_rows, int(tile_rows), order)

@@ -16,9 +16,11 @@ from __future__ import annotations
 import os
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache import CacheConfig, CacheManager
+from ..kernels.staging import PinnedUpload
 from ..models.model import DecoderModel
 from ..parts.base import Runtime
 
@@ -72,6 +74,7 @@ class Engine:
         self._graph_pool = None
         self.graph_replays = 0
         self.max_recorded_steps = MAX_RECORDED_STEPS
+        self._staging = PinnedUpload(self.rt.device) if self.rt.device.type == "cuda" else None
         # "native": the step's launches are made by the host library from one call where every part of the
         # model has a native description (engine/program.py); "parts": by the parts' own forward, one Python
         # call per launch.  The same launches either way.
@@ -143,8 +146,17 @@ class Engine:
         """True when the pools or the state slots cannot hold this step's new tokens."""
         return not self.cache.step_fits([e.request for e in entries], [len(e.tokens) for e in entries])
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Run one batch; returns logits [sum(len(want)), vocab] fp32 in the order of entries and of ``want``."""
+    supports_device_tokens = True
+
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[tuple] = None,
+             borrow_logits: bool = False) -> torch.Tensor:
+        """Run one batch; returns logits [sum(len(want)), vocab] fp32 in the order of entries and of ``want``.
+
+        ``device_tokens`` = (tokens, index): int32 tokens on the device (what the last step's sampling left
+        there) and, per entry, the place among them of the entry's single token, or -1 for an entry whose
+        tokens are given; the batch takes those tokens on the device, and the host never sees them before.
+        ``borrow_logits``: the caller uses the logits before the next step and does not keep them (a recorded
+        step's logits are the recording's own and are written again by the next replay)."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         V = self.spec.vocab_size
         if not entries:
@@ -164,11 +176,15 @@ class Engine:
             if not cache.reserve_step(reqs, q_lens, arrays):
                 raise OutOfPages("the pages this step was checked for are gone")   # step_fits said they were there
             reserved = True
+            if device_tokens is not None:
+                for e, j in zip(entries, device_tokens[1]):
+                    if j >= 0 and len(e.tokens) != 1:
+                        raise StepError(f"request {e.request!r}: a token from the device stands for exactly one token")
             if all(n == 1 for n in q_lens):
-                logits = self._decode_step(entries)
+                logits = self._decode_step(entries, device_tokens, borrow_logits)
             else:
                 packed = pack_step(cache, entries, tile_rows=self._tile_rows)
-                ctx = packed.context(torch.from_numpy(packed.host).to(self.rt.device))
+                ctx = packed.context(self._stage(packed, device_tokens))
                 logits = self._forward(ctx)
         except BaseException:
             # the step did not run to its end: requests that came with it leave again, the others give back
@@ -189,7 +205,23 @@ class Engine:
                 return self.program.run(ctx)
         return self.model.forward(ctx, self.views)
 
-    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _stage(self, packed, device_tokens: Optional[tuple], out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The step's int32 arrays on the device (in ``out`` when given), by way of pinned memory and a kernel of
+        the stream; single tokens that the last step chose on the device go into the token ids there."""
+        if self._staging is None:
+            from ..kernels.api import KernelError
+            raise KernelError("no GPU is visible: infernum_amd runs on a gfx950 GPU only (there is no CPU fallback)")
+        rows = source = None
+        if device_tokens is not None:
+            source, index = device_tokens
+            nd = packed.num_decode                          # requests that bring one token are the first rows
+            rows = np.fromiter((index[i] for i in packed.order[:nd]), dtype=np.int32, count=nd)
+            if nd == 0 or int(rows.max()) < 0:
+                rows = source = None
+        return self._staging.upload(packed.host, out=out, token_off=packed.offsets[0], token_rows=rows, source=source)
+
+    def _decode_step(self, entries: Sequence[StepEntry], device_tokens: Optional[tuple] = None,
+                     borrow_logits: bool = False) -> torch.Tensor:
         """Every request brings one token.  Block tables are widened to a power of two of pages, and the
         kernels are told that width as the longest length, so that a shape's launches are the same from
         step to step, recorded or not."""
@@ -201,13 +233,13 @@ class Engine:
         g = self._graphs.get(key)
         if g is not None:
             self._graphs[key] = self._graphs.pop(key)       # most recently used last
-            g.inputs.copy_(torch.from_numpy(packed.host))
+            self._stage(packed, device_tokens, out=g.inputs)
             g.graph.replay()
             self.graph_replays += 1
-            return g.logits.clone()
+            return g.logits if borrow_logits else g.logits.clone()
         seen = self._shape_seen.get(key, 0)
         self._shape_seen[key] = seen + 1
-        inputs = torch.from_numpy(packed.host).to(self.rt.device)
+        inputs = self._stage(packed, device_tokens)
         ctx = packed.context(inputs)
         ctx.max_total_len = max(limit, ctx.max_total_len)
         if not self.use_graphs or seen < 1:
@@ -226,7 +258,7 @@ class Engine:
         self._graphs[key] = _DecodeGraph(inputs, graph, logits)
         graph.replay()
         self.graph_replays += 1
-        return logits.clone()
+        return logits if borrow_logits else logits.clone()
 
     def decode_greedy(self, requests: Sequence[Hashable], tokens: Sequence[int]) -> List[int]:
         """One decode step for requests that each bring one token; returns each one's next token (argmax)."""

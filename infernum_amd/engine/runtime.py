@@ -57,6 +57,17 @@ class Runtime:
         self.sampler = sampler
         self.steps = 0
         self.tokens_run = 0
+        # One step ahead: a step is launched with the tokens of the step before it still on the device, and the
+        # host reads a step's tokens while the next step runs.  Needs an engine that takes tokens from the device
+        # and a sampler that leaves them there; requests whose choice looks at their own history (a repetition
+        # penalty) are served one step at a time.
+        self.look_ahead = (os.environ.get("INFERNUM_LOOK_AHEAD", "1") != "0"
+                           and getattr(engine, "supports_device_tokens", False)
+                           and hasattr(self.sampler, "select_on_device")
+                           and getattr(getattr(engine, "rt", None), "device", None) is not None
+                           and engine.rt.device.type == "cuda")
+        self._inflight = None                 # (plan, tokens on the device, row of each request, download)
+        self._download = None
 
     # ---- building ---------------------------------------------------------------------
     @classmethod
@@ -79,7 +90,11 @@ class Runtime:
         return self.scheduler.add_request(input_ids, options, token_tx)
 
     def step(self) -> SchedulerOutput:
-        """One iteration: schedule, run the batch, choose tokens, update (engine.rs:191-237)."""
+        """One iteration: schedule, run the batch, choose tokens, update (engine.rs:191-237).  With look-ahead
+        the tokens of the step launched here reach the requests during the next call."""
+        if self.look_ahead and self._all_can_wait():
+            return self._step_ahead()
+        self._deliver()
         plan = self.scheduler.step(self.engine.cache)
         if plan.is_empty():
             return plan
@@ -114,6 +129,75 @@ class Runtime:
                 self.scheduler.on_prefill_done(t, None)
         return plan
 
+    # ---- one step ahead ------------------------------------------------------------------
+    def _all_can_wait(self) -> bool:
+        needs = self.sampler.needs_history
+        return not any(needs(s.options.sampling) for s in self.scheduler.running) and \
+            not any(needs(s.options.sampling) for s in self.scheduler.waiting)
+
+    def _deliver(self) -> None:
+        """The tokens of the step in flight, if any, go to their requests."""
+        flight, self._inflight = self._inflight, None
+        if flight is None:
+            return
+        plan, handle = flight[0], flight[3]
+        tokens = self._download.wait(handle)
+        k = 0
+        for t in plan.decode:
+            self.scheduler.on_decode_done(t, tokens[k])
+            k += 1
+        for t in plan.prefill:
+            if t.completes:
+                self.scheduler.on_prefill_done(t, tokens[k])
+                k += 1
+
+    def _step_ahead(self) -> SchedulerOutput:
+        plan = self.scheduler.step(self.engine.cache)
+        if plan.is_empty():
+            self._deliver()
+            return plan
+        before = self._inflight
+        row_before = before[2] if before is not None else {}
+        entries: List[StepEntry] = []
+        rows: List[RowRequest] = []
+        index: List[int] = []
+        row_of = {}
+        for t in plan.decode:
+            s = t.seq
+            if s.pending:                         # its last token is where the step in flight leaves it
+                entries.append(StepEntry(s.id, [0], [0]))
+                index.append(row_before[s.id])
+            else:
+                entries.append(StepEntry(s.id, [s.generated_ids[-1]], [0]))
+                index.append(-1)
+            row_of[s.id] = len(rows)
+            rows.append(self._row(s))
+        for t in plan.prefill:
+            entries.append(StepEntry(t.seq.id, t.token_ids, [len(t.token_ids) - 1] if t.completes else []))
+            index.append(-1)
+            if t.completes:
+                row_of[t.seq.id] = len(rows)
+                rows.append(self._row(t.seq))
+        try:
+            feed = (before[1], index) if before is not None and any(j >= 0 for j in index) else None
+            logits = self.engine.step(entries, device_tokens=feed, borrow_logits=True)
+            chosen = self.sampler.select_on_device(logits, rows)
+        except Exception as e:                    # the requests of this batch end with an error event
+            for t in list(plan.decode) + list(plan.prefill):
+                self.scheduler._fail(t.seq, f"{type(e).__name__}: {e}")
+            self._deliver()
+            raise
+        self.steps += 1
+        self.tokens_run += plan.num_tokens
+        self.scheduler.on_launched(plan)
+        if self._download is None:
+            from ..kernels.staging import TokenDownload
+            self._download = TokenDownload(self.engine.rt.device)
+        handle = self._download.start(chosen)
+        self._deliver()                           # the step before: its tokens while this one runs
+        self._inflight = (plan, chosen, row_of, handle)
+        return plan
+
     @staticmethod
     def _row(s: SequenceState) -> RowRequest:
         sp = s.options.sampling
@@ -126,7 +210,7 @@ class Runtime:
             hist = s.generated_ids[-n:]
             if len(hist) < n:
                 hist = s.prompt_ids[len(s.prompt_ids) - min(n - len(hist), len(s.prompt_ids)):] + hist
-        return RowRequest(sp, len(s.generated_ids), hist)
+        return RowRequest(sp, len(s.generated_ids) + s.pending, hist)
 
     def run(self, until: Optional[Callable[[], bool]] = None) -> None:
         """Step until nothing waits or runs (or until ``until()`` is true)."""
@@ -134,6 +218,8 @@ class Runtime:
             if until is not None and until():
                 return
             self.step()
+        if until is None or self.scheduler.is_idle():
+            self._deliver()
         self.scheduler.reap(self.engine.cache)
 
     # ---- whole generations ---------------------------------------------------------------

@@ -106,13 +106,15 @@ class SequenceState:
     finish_reason: Optional[FinishReason] = None
     error: Optional[str] = None
     times_set_back: int = 0
+    pending: int = 0            # tokens chosen on the device in a step whose result the host has not seen yet
 
     def all_tokens(self) -> List[int]:
+        """The tokens the host knows (a pending one is not among them)."""
         return self.prompt_ids + self.generated_ids
 
     @property
     def num_tokens(self) -> int:
-        return len(self.prompt_ids) + len(self.generated_ids)
+        return len(self.prompt_ids) + len(self.generated_ids) + self.pending
 
     def send(self, event: GenerationEvent) -> bool:
         return True if self.token_tx is None else bool(self.token_tx(event))
@@ -197,10 +199,13 @@ class Scheduler:
         out = SchedulerOutput()
         # finished requests give back what they hold (scheduler.rs:289-305)
         out.finished.extend(self.reap(cache))
-        running, waiting = list(self.running), list(self.waiting)
+        # a request whose last token is still on the device keeps what it holds and does nothing more
+        running = [s for s in self.running if not self._awaits_last_token(s)]
+        waiting = list(self.waiting)
         if not running and not waiting:
             return out
         nr, nw = len(running), len(waiting)
+        max_batch = cfg.max_batch_size - (len(self.running) - nr)
         rid = (ctypes.c_int64 * max(nr, 1))(*[cache.request_id(s.id) if cache.has(s.id) else -1 for s in running])
         phase = (ctypes.c_int * max(nr, 1))(*[2 if s.phase == SequencePhase.DECODE else 1 for s in running])
         tokens = (ctypes.c_int64 * max(nr, 1))(*[s.num_tokens for s in running])
@@ -208,7 +213,7 @@ class Scheduler:
         cap = 3 * nr + 2 * nw + 4
         actions = (ctypes.c_int * (4 * cap))()
         n = native.lib().ia_sched_step(cache.native_handle(), nr, rid, phase, tokens, nw, wait_tokens,
-                                       cfg.max_batch_size, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
+                                       max_batch, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
                                        actions, cap)
         if n < 0:
             cache._fail()
@@ -248,25 +253,44 @@ class Scheduler:
                 raise RuntimeError(f"unknown scheduling action {kind}")
         return out
 
+    def _awaits_last_token(self, seq: SequenceState) -> bool:
+        if not seq.pending or seq.phase == SequencePhase.FINISHED:
+            return False
+        return (len(seq.generated_ids) + seq.pending >= seq.options.max_new_tokens
+                or (self.max_seq_len is not None and seq.num_tokens >= self.max_seq_len))
+
+    # ---- while the model runs: the step is launched, its tokens are not here yet ------
+    def on_launched(self, plan: SchedulerOutput) -> None:
+        """The step of ``plan`` was launched and leaves its chosen tokens on the device: every request that gets
+        a token from it counts one token more from now on; ``on_decode_done`` / ``on_prefill_done`` bring it."""
+        for t in plan.decode:
+            t.seq.pending += 1
+        for t in plan.prefill:
+            if t.completes:
+                t.seq.phase = SequencePhase.DECODE
+                t.seq.pending += 1
+
     # ---- after the model has run ------------------------------------------------------
     def on_prefill_done(self, task: PrefillTask, token: Optional[int]) -> None:
         """The portion is in the cache; ``token`` is the one chosen after a portion that completes."""
-        if task.seq.phase == SequencePhase.FINISHED:
-            return
         if task.completes:
             if token is None:
                 raise ValueError("a completed prompt needs its next token")
-            task.seq.phase = SequencePhase.DECODE
+            if task.seq.phase == SequencePhase.PREFILL:
+                task.seq.phase = SequencePhase.DECODE
             self.handle_new_token(task.seq, token)
 
     def on_decode_done(self, task: DecodeTask, token: int) -> None:
-        if task.seq.phase != SequencePhase.FINISHED:
-            self.handle_new_token(task.seq, token)
+        self.handle_new_token(task.seq, token)
 
     def handle_new_token(self, seq: SequenceState, token: int) -> None:
         """infernum-runtime/src/engine.rs:445-481: the end-of-sequence token stops and is
         not emitted; a receiver that went away cancels; max_new_tokens ends with LENGTH."""
         token = int(token)
+        if seq.pending:
+            seq.pending -= 1                      # the token that was on the device
+        if seq.phase == SequencePhase.FINISHED:
+            return
         if seq.options.eos_token_id is not None and token == seq.options.eos_token_id:
             self._finish(seq, FinishReason.STOP)
             return
@@ -297,6 +321,8 @@ class Scheduler:
         return seq
 
     def _finish(self, seq: SequenceState, reason: FinishReason) -> None:
+        if seq.phase == SequencePhase.WAITING and seq in self.waiting:
+            self.waiting.remove(seq)              # set back while its last token was still on the device
         seq.phase = SequencePhase.FINISHED
         seq.finish_reason = reason
         seq.send(GenerationEvent("finished", reason=reason))

@@ -246,6 +246,42 @@ def cast(src: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = No
     return out
 
 
+def gather_tokens(token_ids: torch.Tensor, source: torch.Tensor, index: torch.Tensor) -> None:
+    """token_ids[i] = source[index[i]] where index[i] >= 0; other places stay.  All int32 on the device."""
+    _dev(token_ids, source, index)
+    n = token_ids.numel()
+    _i32(token_ids, n, "gather_tokens token_ids")
+    _i32(index, n, "gather_tokens index")
+    _i32(source, 0, "gather_tokens source")
+    _ok(_core().ia_gather_tokens(_p(token_ids), _p(source), _p(index), n, source.numel(), _stream()), "gather_tokens")
+
+
+def words_from_host(dst: torch.Tensor, pinned: torch.Tensor, n: int, token_off: int = 0, nd: int = 0,
+                    source: Optional[torch.Tensor] = None, index_off: int = 0) -> None:
+    """dst[:n] = pinned[:n] (4-byte words; ``pinned`` in pinned host memory) by a kernel of the current stream;
+    with ``nd`` > 0 the words dst[token_off + r], r < nd, whose index pinned[index_off + r] is j >= 0 become
+    source[j] (int32 on the device)."""
+    _need(dst.is_cuda and dst.is_contiguous() and dst.element_size() == 4 and dst.numel() >= n,
+          "words_from_host: a contiguous device tensor of 4-byte elements, at least n long")
+    _need(pinned.is_pinned() and pinned.element_size() == 4 and pinned.numel() >= max(n, index_off + nd),
+          "words_from_host: the source must be pinned host memory of 4-byte elements, long enough")
+    if nd:
+        _i32(source, 0, "words_from_host tokens")
+    _ok(_core().ia_words_from_host(_p(dst), ctypes.c_void_p(pinned.data_ptr()), int(n), int(token_off), int(nd),
+                                   _p(source), source.numel() if source is not None else 0, int(index_off), _stream()),
+        "words_from_host")
+
+
+def words_to_host(pinned: torch.Tensor, src: torch.Tensor) -> None:
+    """pinned[:n] = src (4-byte words) by a kernel of the current stream; an event recorded after it tells the
+    host when the words are there."""
+    n = src.numel()
+    _need(src.is_cuda and src.is_contiguous() and src.element_size() == 4, "words_to_host: a device tensor of 4-byte elements")
+    _need(pinned.is_pinned() and pinned.element_size() == 4 and pinned.numel() >= n,
+          "words_to_host: the target must be pinned host memory of 4-byte elements, long enough")
+    _ok(_core().ia_words_to_host(ctypes.c_void_p(pinned.data_ptr()), _p(src), n, _stream()), "words_to_host")
+
+
 def copy_pages(pool: torch.Tensor, src_pages: torch.Tensor, dst_pages: torch.Tensor) -> None:
     """pool[dst_pages[i]] = pool[src_pages[i]] for a pool [num_pages, ...]; pairs with a page outside the pool
     are left out.  The targets must differ from each other and from every source."""
@@ -633,7 +669,7 @@ def attention_mfma_available(d: int) -> bool:
 # standard error when the process ends (``profile_report`` gives it at any time).  The reference's switch of the
 # same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
 # are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
-_PROFILED = ("cast", "copy_pages", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
+_PROFILED = ("cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
              "gemm_library", "gemm_skinny", "attention_generic", "attention_decode", "attention_decode_rotating",
              "attention_prefill", "argmax", "repetition_penalty", "sample")
 _profile_on = False

@@ -37,20 +37,40 @@ class RowRequest:
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
+        self._staging = None
+
+    def _to_device(self, host: np.ndarray) -> torch.Tensor:
+        """A small host array to the device without waiting for what the GPU still has to do."""
+        if torch.device(self.device).type != "cuda":
+            return torch.from_numpy(host).to(self.device)
+        if self._staging is None:
+            from ..kernels.staging import PinnedUpload
+            self._staging = PinnedUpload(torch.device(self.device), buffers=8)
+        return self._staging.upload(host)
+
+    @staticmethod
+    def needs_history(sampling: Optional[SamplingParams]) -> bool:
+        """Whether a request's choice looks at the tokens it has generated (the repetition penalty does)."""
+        return sampling is not None and abs(sampling.repetition_penalty - 1.0) > 1.1920929e-07 \
+            and sampling.repetition_penalty_window > 0
 
     def select(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> List[int]:
         """logits fp32 [R, V] on the device (left unchanged); one token per row."""
+        return self.select_on_device(logits, rows).tolist()
+
+    def select_on_device(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> torch.Tensor:
+        """The same, with the tokens left on the device: int32 [R]."""
         R, V = logits.shape
         if R != len(rows):
             raise ValueError(f"{R} rows of logits for {len(rows)} requests")
-        if R == 0:
-            return []
-        sampled = [i for i, r in enumerate(rows) if r.sampling is not None]
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        if R == 0:
+            return out
+        sampled = [i for i, r in enumerate(rows) if r.sampling is not None]
         if len(sampled) < R:
             K.argmax(logits, out)
         if not sampled:
-            return out.tolist()
+            return out
         S = len(sampled)
         params = [rows[i].sampling for i in sampled]
         penalised = any(abs(p.repetition_penalty - 1.0) > 1.1920929e-07 for p in params)
@@ -60,13 +80,13 @@ class Sampler:
             nums[0, s], nums[1, s] = p.temperature, p.top_p
             nums[2, s] = token_uniform(p.seed, rows[i].generated_before)
             nums[3, s] = p.repetition_penalty
-        dev_nums = torch.from_numpy(nums).to(logits.device)
+        dev_nums = self._to_device(nums)
         if S == R and not penalised and logits.is_contiguous():
             work_logits = logits                     # nothing changes the logits: no copy
             idx = None
         else:
             # sampled rows are worked on in a copy: the penalty changes logits in place
-            idx = torch.tensor(sampled, dtype=torch.long, device=logits.device) if S < R else None
+            idx = self._to_device(np.asarray(sampled, dtype=np.int32)).long() if S < R else None
             work_logits = (logits.index_select(0, idx) if idx is not None else logits.clone()).contiguous()
         if penalised:
             tails = []
@@ -79,10 +99,10 @@ class Sampler:
             for s, t in enumerate(tails):
                 ints[s * W:s * W + len(t)] = t
                 ints[S * W + s] = len(t)
-            dev_ints = torch.from_numpy(ints).to(logits.device)
+            dev_ints = self._to_device(ints)
             K.repetition_penalty(work_logits, dev_ints[:S * W].view(S, W), dev_ints[S * W:], dev_nums[3])
         picked = out if idx is None else torch.empty(S, dtype=torch.int32, device=logits.device)
         K.sample(work_logits, torch.empty_like(work_logits), dev_nums[0], dev_nums[1], dev_nums[2], picked)
         if idx is not None:
             out.index_copy_(0, idx, picked)
-        return out.tolist()
+        return out

@@ -71,7 +71,8 @@ def test_sampled_B_portions_mixed_with_decoding(folders):
     rt = _runtime(d, "float32", block_size=8, num_blocks=24, max_batch_size=3, max_prefill_tokens=8,
                   max_tokens_per_step=16)
     sizes, real_step = [], rt.engine.step
-    rt.engine.step = lambda entries: (sizes.append(sorted(len(e.tokens) for e in entries)), real_step(entries))[1]
+    rt.engine.step = lambda entries, **kw: (sizes.append(sorted(len(e.tokens) for e in entries)),
+                                            real_step(entries, **kw))[1]
     got = rt.generate_batch(prompts, [GenerateOptions(max_new_tokens=12, sampling=s) for s in sp])
     assert any(e[0] == 1 and e[-1] > 1 for e in sizes), f"no step mixed decoded tokens with a portion: {sizes}"
     assert max(sum(e) for e in sizes) <= 16 and max(max(e) for e in sizes) <= 8
@@ -110,10 +111,10 @@ def _record_logits(rt):
     """Wraps the engine's step function: (request, place) -> the logits row that came back for it."""
     seen, real_step = {}, rt.engine.step
 
-    def step(entries):
+    def step(entries, **kw):
         before = {e.request: (rt.engine.cache.num_tokens(e.request) if rt.engine.cache.has(e.request) else 0)
                   for e in entries}
-        logits = real_step(entries)
+        logits = real_step(entries, **kw)
         rows = logits.detach().double().cpu()
         k = 0
         for e in entries:
@@ -218,3 +219,48 @@ def test_bench_command_line(folders):
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert "12 tokens in" in proc.stdout and "tok/s" in proc.stdout and "prefill 40 tokens" in proc.stdout
     assert "Model loaded: 3 layers, 128 hidden, dtype=f32" in proc.stderr
+
+
+@pytest.mark.parametrize("num_blocks", [64, 13])
+def test_one_step_ahead_changes_no_token(folders, num_blocks):
+    """With look-ahead a step is launched while the tokens of the step before it are still on the device; the
+    requests get the same tokens as when every step waits for its tokens: greedy and sampled requests, one that
+    stops at an end-of-sequence token (its row in the step launched meanwhile is wasted, not wrong), one of a
+    single new token, prompts in portions, and (13 pages) requests set back with a token still on the way."""
+    from infernum_amd import GenerateOptions, SamplingParams
+    d, cfg, w = folders["B"]
+    g = torch.Generator().manual_seed(12)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (9, 17, 6, 12, 5)]
+    probe = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=5, max_prefill_tokens=8)
+    probe.look_ahead = False
+    free_run = probe.generate(prompts[1], GenerateOptions(max_new_tokens=16))
+    eos = free_run[9]                                          # request 1 stops where this token first comes
+    opts = [GenerateOptions(max_new_tokens=16),
+            GenerateOptions(max_new_tokens=16, eos_token_id=eos),
+            GenerateOptions(max_new_tokens=14, sampling=SamplingParams(temperature=0.8, top_p=0.9, seed=3,
+                                                                       repetition_penalty=1.0)),
+            GenerateOptions(max_new_tokens=1),
+            GenerateOptions(max_new_tokens=15, sampling=SamplingParams(temperature=1.1, top_p=1.0, seed=5,
+                                                                       repetition_penalty=1.0))]
+    results = {}
+    for ahead in (False, True):
+        rt = _runtime(d, "float32", block_size=4, num_blocks=num_blocks, max_batch_size=5, max_prefill_tokens=8)
+        assert rt.look_ahead
+        rt.look_ahead = ahead
+        with_device_tokens, real_step = [], rt.engine.step
+        rt.engine.step = lambda entries, **kw: (with_device_tokens.append(kw.get("device_tokens") is not None),
+                                                real_step(entries, **kw))[1]
+        seqs = [rt.submit(p, o) for p, o in zip(prompts, opts)]
+        n_back = 0
+        while not rt.scheduler.is_idle():
+            n_back += len(rt.step().set_back)
+        rt.run()
+        assert all(s.error is None and s.pending == 0 for s in seqs)
+        results[ahead] = [(list(s.generated_ids), s.finish_reason) for s in seqs]
+        assert any(with_device_tokens) == ahead
+        assert (n_back > 0) == (num_blocks == 13), f"{n_back} set back with {num_blocks} pages"
+        rt.scheduler.reap(rt.engine.cache)
+        rt.engine.cache.check()
+        assert rt.engine.cache.free_pages() == num_blocks
+    assert results[True] == results[False]
+    assert results[True][1][0] == free_run[:free_run.index(eos)] and len(results[True][3][0]) == 1

@@ -274,3 +274,63 @@ def test_generate_batch_and_no_kv_cache():
     assert eng.cache.free_pages() == 64
     with pytest.raises(GenerationError, match="tokenizer"):
         rt.generate("some text", o)
+
+
+def test_tokens_still_on_the_device_count_and_arrive_later():
+    """A step is launched and its tokens are not on the host yet (``on_launched``): the requests count one token
+    more, a request whose last token that is does nothing further but keeps its pages, and the token's arrival
+    finishes it; a request that was set back meanwhile and finishes on arrival leaves the queue."""
+    from infernum_amd.cache import CacheConfig, CacheManager
+    from infernum_amd.engine.scheduler import BatchConfig, FinishReason, Scheduler, SequencePhase
+    from infernum_amd.parts import CacheSpec
+    from infernum_amd.sampling import GenerateOptions
+    cache = CacheManager([(CacheSpec("full", 1, 8), None)], [None], CacheConfig(page_size=4, num_pages=16, num_state_slots=4))
+    sch = Scheduler(BatchConfig(max_batch_size=2, max_prefill_tokens=8, block_size=4, num_blocks=16, max_tokens_per_step=16))
+    a = sch.add_request([1, 2, 3], GenerateOptions(max_new_tokens=2))
+    b = sch.add_request([4, 5, 6, 7, 8], GenerateOptions(max_new_tokens=3))
+    c = sch.add_request([9], GenerateOptions(max_new_tokens=1))
+
+    def launch(plan):
+        for t in plan.prefill:
+            if not cache.has(t.seq.id):
+                cache.admit(t.seq.id)
+            assert cache.reserve(t.seq.id, len(t.token_ids))
+            cache.commit(t.seq.id, len(t.token_ids))
+        for t in plan.decode:
+            assert cache.reserve(t.seq.id, 1)
+            cache.commit(t.seq.id, 1)
+        sch.on_launched(plan)
+
+    p1 = sch.step(cache)
+    assert [t.seq for t in p1.prefill] == [a, b] and all(t.completes for t in p1.prefill) and sch.num_waiting() == 1
+    launch(p1)
+    assert a.pending == b.pending == 1 and a.num_tokens == 4 and a.phase == SequencePhase.DECODE and a.generated_ids == []
+    p2 = sch.step(cache)                                      # decided with the first tokens still on the device
+    assert [t.seq for t in p2.decode] == [a, b] and not p2.prefill
+    launch(p2)
+    for t in p1.prefill:
+        sch.on_prefill_done(t, 50)
+    assert a.generated_ids == [50] and a.pending == 1 and a.phase == SequencePhase.DECODE
+    p3 = sch.step(cache)                                      # a waits for its last token: only b moves, c cannot come in
+    assert [t.seq for t in p3.decode] == [b] and not p3.prefill and sch.num_waiting() == 1 and cache.has(a.id)
+    launch(p3)
+    for t in p2.decode:
+        sch.on_decode_done(t, 51)
+    assert a.phase == SequencePhase.FINISHED and a.finish_reason == FinishReason.LENGTH and a.generated_ids == [50, 51]
+    assert b.generated_ids == [50, 51] and b.pending == 1
+    p4 = sch.step(cache)                                      # a is reaped, c is admitted beside b, which waits
+    assert not cache.has(a.id) and [t.seq for t in p4.prefill] == [c] and not p4.decode
+    launch(p4)
+    for t in p3.decode:
+        sch.on_decode_done(t, 52)
+    assert b.phase == SequencePhase.FINISHED and b.generated_ids == [50, 51, 52] and b.pending == 0
+    # a request set back with a token on the way, which then turns out to be its end
+    b2 = sch.add_request([4, 5], GenerateOptions(max_new_tokens=5, eos_token_id=77))
+    b2.pending, b2.phase = 1, SequencePhase.WAITING           # as a set-back leaves it
+    sch.handle_new_token(b2, 77)
+    assert b2.phase == SequencePhase.FINISHED and b2.finish_reason == FinishReason.STOP and b2 not in sch.waiting
+    for t in p4.prefill:
+        sch.on_prefill_done(t, 9)
+    assert c.phase == SequencePhase.FINISHED and c.generated_ids == [9]
+    sch.step(cache)
+    assert sch.is_idle() and cache.free_pages() == 16
