@@ -624,7 +624,9 @@ int ia_cache_pack_step(void* h, int n, const int64_t* reqs, const int* q_lens, c
 // returns to the front of the queue; a request that is alone and still does not fit fails.
 //
 // Running requests come in the order of admission: rid (their number in the cache, -1 when they hold
-// nothing yet), phase (1 = prompt, 2 = decoding) and tokens (prompt and generated).  The queue comes head
+// nothing yet), phase (1 = prompt, 2 = decoding, 3 = done but for a token that is still on its way: it keeps
+// what it holds, does nothing, is never set back, and will give everything back soon, so a request that cannot
+// move because of it waits instead of failing or setting others back) and tokens (prompt and generated).  The queue comes head
 // first.  Actions are records of four ints (kind, index, a, b):
 //   1 decode   index = running request
 //   2 portion  index = running request, a = tokens already stored, b = tokens of the portion
@@ -671,6 +673,22 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
     return false;
   };
   auto drop_from_live = [&](int s) { live.erase(std::find(live.begin(), live.end(), s)); };
+  // the request admitted last among those that can be set back (-1: none), and whether one is on its way out
+  auto last_movable = [&]() {
+    for (size_t k = live.size(); k-- > 0;)
+      if (run_phase[live[k]] != 3) return live[k];
+    return -1;
+  };
+  auto movable_count = [&]() {
+    int n = 0;
+    for (int s : live) n += run_phase[s] != 3;
+    return n;
+  };
+  auto any_leaving = [&]() {
+    for (int s : live)
+      if (run_phase[s] == 3) return true;
+    return false;
+  };
   std::vector<int> freed;                      // (group, page) pairs of everything released in this step
   auto release = [&](int s) {
     if (rid[(size_t)s] >= 0 && c->admitted(rid[(size_t)s])) {
@@ -702,8 +720,9 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
       ++i;
       continue;
     }
-    const int victim = live.back();
-    if (victim == s && live.size() == 1) {
+    if (any_leaving()) { ++i; continue; }     // pages come back when the leaving requests' tokens are in: wait
+    const int victim = last_movable();
+    if (victim == s && movable_count() == 1) {
       acts.push_back({4, s, 1, 0});
       drop_from_live(s);
       release(s);
@@ -723,9 +742,9 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
     int64_t n = std::min<int64_t>(std::min<int64_t>(run_tokens[s] - cached, max_prefill), budget);
     n = std::min<int64_t>(n, tokens_that_fit(r));
     if (n <= 0) {
-      if (!planned()) {
-        const int victim = live.back();           // nobody can move: the last admitted request makes room
-        if (victim == s && live.size() == 1) {
+      if (!planned() && !any_leaving()) {
+        const int victim = last_movable();        // nobody can move: the last admitted request makes room
+        if (victim == s && movable_count() == 1) {
           acts.push_back({4, s, 2, 0});
           drop_from_live(s);
           release(s);

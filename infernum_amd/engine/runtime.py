@@ -31,6 +31,18 @@ class GenerationError(RuntimeError):
     pass
 
 
+class _TokensAtHand:
+    """The tokens of an engine that keeps them where the host reads them anyway (stand-ins on the CPU)."""
+
+    @staticmethod
+    def start(tokens):
+        return tokens
+
+    @staticmethod
+    def wait(handle) -> List[int]:
+        return [int(t) for t in handle.tolist()]
+
+
 class Runtime:
     def __init__(self, engine: Any, tokenizer: Any = None, batch_config: Optional[BatchConfig] = None,
                  max_seq_len: Optional[int] = None, sampler: Any = None):
@@ -63,9 +75,7 @@ class Runtime:
         # penalty) are served one step at a time.
         self.look_ahead = (os.environ.get("INFERNUM_LOOK_AHEAD", "1") != "0"
                            and getattr(engine, "supports_device_tokens", False)
-                           and hasattr(self.sampler, "select_on_device")
-                           and getattr(getattr(engine, "rt", None), "device", None) is not None
-                           and engine.rt.device.type == "cuda")
+                           and hasattr(self.sampler, "select_on_device") and hasattr(self.sampler, "needs_history"))
         self._inflight = None                 # (plan, tokens on the device, row of each request, download)
         self._download = None
 
@@ -191,8 +201,12 @@ class Runtime:
         self.tokens_run += plan.num_tokens
         self.scheduler.on_launched(plan)
         if self._download is None:
-            from ..kernels.staging import TokenDownload
-            self._download = TokenDownload(self.engine.rt.device)
+            device = getattr(getattr(self.engine, "rt", None), "device", None)
+            if device is not None and device.type == "cuda":
+                from ..kernels.staging import TokenDownload
+                self._download = TokenDownload(device)
+            else:
+                self._download = _TokensAtHand()
         handle = self._download.start(chosen)
         self._deliver()                           # the step before: its tokens while this one runs
         self._inflight = (plan, chosen, row_of, handle)

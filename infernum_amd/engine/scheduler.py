@@ -199,21 +199,20 @@ class Scheduler:
         out = SchedulerOutput()
         # finished requests give back what they hold (scheduler.rs:289-305)
         out.finished.extend(self.reap(cache))
-        # a request whose last token is still on the device keeps what it holds and does nothing more
-        running = [s for s in self.running if not self._awaits_last_token(s)]
-        waiting = list(self.waiting)
+        running, waiting = list(self.running), list(self.waiting)
         if not running and not waiting:
             return out
         nr, nw = len(running), len(waiting)
-        max_batch = cfg.max_batch_size - (len(self.running) - nr)
         rid = (ctypes.c_int64 * max(nr, 1))(*[cache.request_id(s.id) if cache.has(s.id) else -1 for s in running])
-        phase = (ctypes.c_int * max(nr, 1))(*[2 if s.phase == SequencePhase.DECODE else 1 for s in running])
+        # 3: a request whose last token is still on the device keeps what it holds and does nothing more
+        phase = (ctypes.c_int * max(nr, 1))(*[3 if self._awaits_last_token(s) else
+                                              (2 if s.phase == SequencePhase.DECODE else 1) for s in running])
         tokens = (ctypes.c_int64 * max(nr, 1))(*[s.num_tokens for s in running])
         wait_tokens = (ctypes.c_int64 * max(nw, 1))(*[s.num_tokens for s in waiting])
         cap = 3 * nr + 2 * nw + 4
         actions = (ctypes.c_int * (4 * cap))()
         n = native.lib().ia_sched_step(cache.native_handle(), nr, rid, phase, tokens, nw, wait_tokens,
-                                       max_batch, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
+                                       cfg.max_batch_size, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
                                        actions, cap)
         if n < 0:
             cache._fail()

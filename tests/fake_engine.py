@@ -27,9 +27,16 @@ class FakeEngine:
         self.history = {}
         self.steps = []            # per step: list of (request, number of tokens, wanted places)
 
-    def step(self, entries):
+    supports_device_tokens = True
+
+    def step(self, entries, device_tokens=None, borrow_logits=False):
+        """``device_tokens`` = (tokens of the last step, where the engine left them; per entry the place of its
+        single token among them, or -1): as the real engine, which takes such tokens on the device."""
         rows = []
         log = []
+        if device_tokens is not None:
+            source, index = device_tokens
+            entries = [type(e)(e.request, [int(source[j])], e.want) if j >= 0 else e for e, j in zip(entries, index)]
         for e in entries:
             need = self.cache.pages_needed(e.request, len(e.tokens))
             if any(n > g.allocator.num_free for n, g in zip(need, self.cache.groups)):
@@ -57,6 +64,13 @@ class FakeEngine:
 
 class CpuSampler:
     """Greedy by argmax (first maximum); sampled rows by a plain inverse CDF of softmax(x / T)."""
+
+    @staticmethod
+    def needs_history(sampling):
+        return False
+
+    def select_on_device(self, logits, rows):
+        return torch.tensor(self.select(logits, rows), dtype=torch.int32)
 
     def select(self, logits, rows):
         from infernum_amd.sampling import token_uniform

@@ -26,11 +26,16 @@ class PlainScheduler(Scheduler):
             for i, n in enumerate(need):
                 promised[i] += n
 
+        # requests that are done but for a token still on its way: they hold their pages, do nothing, are never
+        # set back; who cannot move because of them waits
+        leaving = [s for s in self.running if self._awaits_last_token(s)]
+        movable = lambda: [s for s in self.running if s not in leaving]        # noqa: E731
+
         # 2. one token for every decoding request
         i = 0
         while i < len(self.running):
             seq = self.running[i]
-            if seq.phase != SequencePhase.DECODE:
+            if seq.phase != SequencePhase.DECODE or seq in leaving:
                 i += 1
                 continue
             need = cache.pages_needed(seq.id, 1)
@@ -40,8 +45,11 @@ class PlainScheduler(Scheduler):
                 out.decode.append(DecodeTask(seq))
                 i += 1
                 continue
-            victim = self.running[-1]
-            if victim is seq and len(self.running) == 1:
+            if leaving:
+                i += 1
+                continue
+            victim = movable()[-1]
+            if victim is seq and len(movable()) == 1:
                 self._fail(seq, f"the page pool is too small for a request of {seq.num_tokens + 1} tokens")
                 self.running.remove(seq)
                 cache.release(seq.id)
@@ -65,10 +73,10 @@ class PlainScheduler(Scheduler):
             n = min(n, cache.tokens_that_fit(seq.id, promised) if cache.has(seq.id)
                     else cache.tokens_that_fit(None, promised))
             if n <= 0:
-                if out.is_empty():
+                if out.is_empty() and not leaving:
                     # nobody can move: the last admitted request makes room
-                    victim = self.running[-1]
-                    if victim is seq and len(self.running) == 1:
+                    victim = movable()[-1]
+                    if victim is seq and len(movable()) == 1:
                         self._fail(seq, f"the page pool is too small for a request of {seq.num_tokens} tokens")
                         self.running.remove(seq)
                         if cache.has(seq.id):

@@ -8,11 +8,16 @@ from infernum_amd.engine import BatchConfig, FinishReason, GenerationError, Runt
 from infernum_amd.sampling import GenerateOptions, SamplingParams
 
 
-def runtime(page_size=4, num_pages=16, max_batch=4, chunk=512, budget=64, slots=8, max_seq_len=None, vocab=50):
+def runtime(page_size=4, num_pages=16, max_batch=4, chunk=512, budget=64, slots=8, max_seq_len=None, vocab=50,
+            look_ahead=False):
+    """``look_ahead``: a step is launched while the tokens of the step before it are still where the engine left
+    them (the stand-in engine plays along); False: every step waits for its tokens."""
     eng = FakeEngine(vocab, page_size, num_pages, slots)
     bc = BatchConfig(max_batch_size=max_batch, max_prefill_tokens=chunk, block_size=page_size, num_blocks=num_pages,
                      max_tokens_per_step=budget)
-    return Runtime(eng, None, bc, max_seq_len=max_seq_len, sampler=CpuSampler()), eng
+    rt = Runtime(eng, None, bc, max_seq_len=max_seq_len, sampler=CpuSampler())
+    rt.look_ahead = look_ahead
+    return rt, eng
 
 
 GREEDY = GenerateOptions(max_new_tokens=5)
@@ -227,12 +232,13 @@ def test_a_long_prompt_takes_what_is_free_and_waits_for_the_rest():
 
 
 # ---- everything together, random ---------------------------------------------------------------------------
+@pytest.mark.parametrize("look_ahead", [False, True])
 @pytest.mark.parametrize("seed", range(5))
-def test_random_load_generates_what_each_request_generates_alone(seed):
+def test_random_load_generates_what_each_request_generates_alone(seed, look_ahead):
     rng = random.Random(seed)
     ps = rng.choice((2, 4, 8))
     rt, eng = runtime(page_size=ps, num_pages=rng.choice((12, 20, 40)), max_batch=rng.choice((2, 3, 5)),
-                      chunk=rng.choice((3, 8, 64)), budget=rng.choice((8, 16, 64)), slots=5)
+                      chunk=rng.choice((3, 8, 64)), budget=rng.choice((8, 16, 64)), slots=5, look_ahead=look_ahead)
     pool_tokens = ps * eng.cache.groups[0].allocator.num_pages
     jobs, seqs = [], []
     for i in range(14):
@@ -256,6 +262,7 @@ def test_random_load_generates_what_each_request_generates_alone(seed):
         eng.cache.check()
         steps += 1
         assert steps < 5000, "the loop does not end"
+    rt.run()                                      # the tokens of the last step, if they are still on their way
     rt.scheduler.reap(eng.cache)
     for s, (p, o) in zip(seqs, jobs):
         assert s.error is None
@@ -334,3 +341,27 @@ def test_tokens_still_on_the_device_count_and_arrive_later():
     assert c.phase == SequencePhase.FINISHED and c.generated_ids == [9]
     sch.step(cache)
     assert sch.is_idle() and cache.free_pages() == 16
+
+
+def test_others_wait_for_the_pages_of_a_request_whose_last_token_is_on_its_way():
+    """One step ahead, a request that has launched its last step holds pages and does nothing more.  A request
+    that needs a page then is neither failed as alone in a pool too small nor set back: it waits a step, until
+    the token has come and the pages are free."""
+    rt, eng = runtime(page_size=2, num_pages=6, max_batch=2, look_ahead=True)
+    a = rt.submit([1, 2, 3, 4], GenerateOptions(max_new_tokens=2))         # 2 pages, a third for its second token
+    b = rt.submit([6, 7, 8, 9, 1], GenerateOptions(max_new_tokens=6))   # 3 pages, a fourth after a step
+    plans = []
+    while not rt.scheduler.is_idle():
+        plans.append(rt.step())
+        eng.cache.check()
+        assert len(plans) < 50
+    rt.run()
+    assert a.error is None and b.error is None
+    assert a.generated_ids == reference_generation([1, 2, 3, 4], GenerateOptions(max_new_tokens=2))
+    assert b.generated_ids == reference_generation([6, 7, 8, 9, 1], GenerateOptions(max_new_tokens=6))
+    assert a.times_set_back == 0 and b.times_set_back == 0
+    # the step after a's last launch has nothing for b to run with: every page is held until a's token is here
+    third = plans[2]
+    assert not third.decode and not third.prefill and not third.set_back and not third.finished
+    assert [t.seq for t in plans[3].decode] == [b] and plans[3].finished == [a]
+    assert eng.cache.free_pages() == 6

@@ -12,7 +12,7 @@ from infernum_amd.sampling import GenerateOptions, SamplingParams
 from plain_scheduler import PlainScheduler
 
 
-def pair(seed):
+def pair(seed, look_ahead=False):
     rng = random.Random(seed)
     ps = rng.choice((2, 4, 8))
     kw = dict(page_size=ps, num_pages=rng.choice((6, 12, 20, 40)), num_state_slots=5)
@@ -25,6 +25,8 @@ def pair(seed):
     for plain in (False, True):
         eng = FakeEngine(50, needs=list(needs), **kw)
         rt = Runtime(eng, None, bc, sampler=CpuSampler())
+        assert rt.look_ahead                      # the stand-in engine takes tokens "from the device" too
+        rt.look_ahead = look_ahead
         if plain:
             rt.scheduler = PlainScheduler(bc)
         out.append((rt, eng))
@@ -36,9 +38,11 @@ def digest(plan):
             [s.id for s in plan.set_back], [(s.id, s.error) for s in plan.finished])
 
 
+@pytest.mark.parametrize("look_ahead", [False, True])
 @pytest.mark.parametrize("seed", range(12))
-def test_native_decisions_equal_plain_decisions(seed):
-    rng, (rt_a, eng_a), (rt_b, eng_b) = pair(seed)
+def test_native_decisions_equal_plain_decisions(seed, look_ahead):
+    """``look_ahead``: a step is decided while the tokens of the step before it are not known yet."""
+    rng, (rt_a, eng_a), (rt_b, eng_b) = pair(seed, look_ahead)
     pool_tokens = eng_a.cache.page_size * eng_a.cache.groups[0].allocator.num_pages
     jobs = []
     for i in range(16):
@@ -66,8 +70,13 @@ def test_native_decisions_equal_plain_decisions(seed):
         steps += 1
         assert steps < 5000, "the loop does not end"
     assert rt_b.scheduler.is_idle()
+    rt_a.run(), rt_b.run()                        # the tokens of the last step, if they are still on their way
     if seed in (1, 3, 4, 8, 10):
         assert set_backs >= 5, "these loads are meant to run out of pages"
+    from fake_engine import reference_generation
+    for (p, o), a in zip(jobs, seqs_a):
+        if a.error is None:
+            assert a.generated_ids == reference_generation(p, o), "a request's tokens depend on its own history only"
     for a, b in zip(seqs_a, seqs_b):
         assert (a.generated_ids, a.error, a.finish_reason, a.times_set_back) == \
                (b.generated_ids, b.error, b.finish_reason, b.times_set_back)
