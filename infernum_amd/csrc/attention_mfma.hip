@@ -25,6 +25,7 @@
 // zeroed (values) or masked (scores): a stale or poisoned page never leaks in.
 // A key that is needed but has no page in the block table gives NaN, not a fault.
 #include "common.h"
+#include <type_traits>
 
 #ifndef IA_HEAD_DIM
 #error "compile with -DIA_HEAD_DIM=<head size>"
@@ -501,6 +502,12 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
 // ia_attn_prefill).  Keys and values go through LDS in tiles of 64 keys (32 above a head size of 128), loaded
 // once per workgroup and read by all its waves; the loads of the next tile are in flight while the matrix
 // cores work on this one.
+// paired: the workgroup of tile k of a request takes rows 32 k .. 32 k + 31 and, from the other end of the
+// request's new tokens, the block of 32 rows that is k-th from last (waves 0, 1 and waves 2, 3): under the
+// causal mask a block of rows costs as many rounds as it has keys before it, so every workgroup of a request
+// then has the same work, where tiles of 64 consecutive rows give the last tile of a prompt from its start
+// as much as all others wait for.  A wave skips the rounds beyond its own rows' keys, and its rows meet the
+// same tiles of keys in the same order either way: the same bits.
 //   S^T[key, col] = K[key, :] . Q[col, :]       v_mfma_f32_16x16x32_bf16 over 32 head dims a step
 //   O^T[dim, col] += V^T[dim, key] P^T[key, col] one v_mfma_f32_16x16x32_bf16 over the 32 keys of a tile
 // The accumulators of the two S^T tiles of 16 keys leave lane (col, qd) with the keys 4 qd .. 4 qd + 3 and
@@ -520,13 +527,16 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
     const int* __restrict__ seq_starts, const int* __restrict__ seq_ctx, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, float scale_log2,
-    int window) {
+    int window, int paired) {
   __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KT][PF_KROW];
   __shared__ __attribute__((aligned(16))) uint16_t vs[2][PF_SUBS][HD][PF_VROW];
   __shared__ int s_poison;
   constexpr int PF_THREADS = 4 * HGW * 64;
   const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, qd = lane >> 4;
-  const int wave = (tid >> 6) & 3, hgw = tid >> 8;      // group of 16 rows, group of CT heads
+  // hgw: the group of CT heads; wave: the group of 16 rows.  The waves of a workgroup go to the four SIMDs in turn,
+  // so the row groups are turned by the head group: every SIMD then has waves of all row groups, and the waves that
+  // run out of keys early (the rows of the near end in a paired launch) leave no SIMD empty.
+  const int hgw = tid >> 8, wave = ((tid >> 6) + hgw * (4 / HGW)) & 3;
   // Workgroups start in the order of their number: all heads of the first tile, then of the next (the
   // host lists the tiles with the most keys first, so that the long ones do not start last), and the
   // key/value heads of one tile go to different dies, each of which then keeps its head's keys in its L2.
@@ -536,8 +546,21 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
   const int G = nh / nkv, HC = (G + CT * HGW - 1) / (CT * HGW);
   const int g = by / HC, hc = by - g * HC;
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
-  const int rows_here = (qlen - row0) < 64 ? (qlen - row0) : 64;      // rows of this workgroup (>= 1)
-  const int rb = row0 + wave * 16;                                     // first row of this wave
+  // rows of this workgroup: first_row .. (one stretch of 64, or two of 32) .. last_row
+  int rb, first_row, last_row;                                         // rb: first row of this wave
+  bool wave_live;
+  if (paired) {
+    const int halves = (qlen + 31) >> 5, ha = row0 >> 6, hb = halves - 1 - ha;      // hb >= ha
+    rb = (wave < 2 ? ha : hb) * 32 + (wave & 1) * 16;
+    wave_live = rb < qlen && (wave < 2 || hb > ha);
+    first_row = ha * 32;
+    last_row = (hb * 32 + 32 < qlen ? hb * 32 + 32 : qlen) - 1;
+  } else {
+    rb = row0 + wave * 16;
+    wave_live = rb < qlen;
+    first_row = row0;
+    last_row = (row0 + 64 < qlen ? row0 + 64 : qlen) - 1;
+  }
   if (tid == 0) s_poison = 0;
 
   // ---- queries of this wave: CT heads x 16 rows, as B operands (col = row j of head c)
@@ -554,10 +577,10 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     const int hj = (hc * HGW + hgw) * CT + c;
-    const bool ok = hj < G && row < qlen;
+    const bool ok = hj < G && row < qlen && wave_live;
     pos[c] = ok ? ctx + row : -1;
     lo[c] = (window > 0 && pos[c] - window + 1 > 0) ? pos[c] - window + 1 : 0;
-    const uint16_t* qrow = q + (size_t)(qstart + (ok ? row : row0)) * q_row_stride + (size_t)(g * G + (ok ? hj : 0)) * HD;
+    const uint16_t* qrow = q + (size_t)(qstart + (ok ? row : first_row)) * q_row_stride + (size_t)(g * G + (ok ? hj : 0)) * HD;
 #pragma unroll
     for (int st = 0; st < NS32; ++st) {
       const bool real = ok && !(HALF_LAST && st == NS32 - 1 && qd >= 2);
@@ -572,20 +595,21 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
   const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
 
   // ---- keys the workgroup needs: those its rows may see
-  const int key_hi = ctx + row0 + rows_here - 1;
-  const int key_lo = (window > 0 && ctx + row0 - window + 1 > 0) ? ctx + row0 - window + 1 : 0;
+  const int key_hi = ctx + last_row;
+  const int key_lo = (window > 0 && ctx + first_row - window + 1 > 0) ? ctx + first_row - window + 1 : 0;
   const int wave_hi = ctx + rb + 15;                                    // last key any row of this wave sees
   const int wave_lo = (window > 0 && ctx + rb - window + 1 > 0) ? ctx + rb - window + 1 : 0;
   const int wave_lo_last = (window > 0 && ctx + rb + 15 - window + 1 > 0) ? ctx + rb + 15 - window + 1 : 0;
-  const bool wave_live = rb < qlen;
   const int* bt = block_tables + (size_t)sidx * bt_stride;
   const int t_begin = key_lo / PF_KT, t_end = key_hi / PF_KT;          // inclusive
 
   // staging: K tile = 32 keys x HD/8 pieces of 16 bytes; V^T tile = HD dims x 8 quads of 4 keys (8 bytes)
   constexpr int KPIECES = PF_KT * (HD / 8), KPT = (KPIECES + PF_THREADS - 1) / (PF_THREADS);
   constexpr int VPIECES = HD * PF_QPT, VPT = (VPIECES + PF_THREADS - 1) / (PF_THREADS);
-  uint4 kreg[KPT];
-  uint2 vreg[VPT];
+  // two sets of registers: the loads of a tile are issued two rounds before the tile is used and wait in
+  // registers for a round, then in LDS for another, so that a round is never shorter than a load takes
+  uint4 kregs[2][KPT];
+  uint2 vregs[2][VPT];
   bool bad = false;
   // Page numbers are read one tile ahead of the keys and values they lead to, so that a tile's loads
   // do not wait for the block table: pgk[i] for the key row of K piece i, pgv for this thread's quad of V.
@@ -625,7 +649,9 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     for (int i = 0; i < KPT; ++i) pgk[i] = bt[page_index(clampk(t0 + k_row[i]))];
     pgv = bt[page_index(clampk(t0 + v_quad * 4))];        // clamping stays within the quad's page when it is needed
   };
-  auto load_tile = [&](int t) {
+  auto load_tile = [&](int t, auto set_c) {
+    uint4* const kreg = kregs[decltype(set_c)::value];
+    uint2* const vreg = vregs[decltype(set_c)::value];
     const int t0 = t * PF_KT;
     const int key0 = t0 + v_quad * 4;
     if (t0 >= key_lo && t0 + PF_KT - 1 <= key_hi) {
@@ -672,7 +698,9 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
       vreg[i] = make_uint2(v.x & mx, v.y & my);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int buf, auto set_c) {
+    const uint4* const kreg = kregs[decltype(set_c)::value];
+    const uint2* const vreg = vregs[decltype(set_c)::value];
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int pc = tid + i * PF_THREADS;
@@ -689,17 +717,24 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     }
   };
 
+  // Tile t lies in register set and LDS buffer (t - t_begin) & 1.
+  using set0 = std::integral_constant<int, 0>;
+  using set1 = std::integral_constant<int, 1>;
   load_pages(t_begin);
-  load_tile(t_begin);
-  if (t_begin < t_end) load_pages(t_begin + 1);
-  store_tile(0);
+  load_tile(t_begin, set0{});
+  if (t_begin < t_end) {
+    load_pages(t_begin + 1);
+    load_tile(t_begin + 1, set1{});                   // waits for its page numbers: once a workgroup
+    if (t_begin + 2 <= t_end) load_pages(t_begin + 2);
+  }
+  store_tile(0, set0{});
   __syncthreads();
-  for (int t = t_begin; t <= t_end; ++t) {
-    const int buf = (t - t_begin) & 1;
-    const bool more = t < t_end;
-    if (more) {
-      load_tile(t + 1);                        // with the page numbers read a round ago
-      if (t + 2 <= t_end) load_pages(t + 2);
+  auto round = [&](int t, auto set_c) {
+    constexpr int buf = decltype(set_c)::value;
+    using other = std::integral_constant<int, buf ^ 1>;
+    if (t + 2 <= t_end) {
+      load_tile(t + 2, set_c);                 // this set's tile is in LDS since the last round; page numbers a round old
+      if (t + 3 <= t_end) load_pages(t + 3);
     }
 #pragma unroll
     for (int sub = 0; sub < PF_SUBS; ++sub) {
@@ -742,16 +777,27 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
               sv[kt * 4 + r] = ok ? sv[kt * 4 + r] : -INFINITY;
             }
         }
-        // the scale is positive: the maximum is taken of the raw scores and scaled once
-        float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, IA_WAVE));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE)) * scale_log2;
         // The reference point of the exponentials follows the running maximum lazily: it moves only when the
         // maximum has grown by more than 2^PF_LAZY, so probabilities stay below 2^PF_LAZY (exact in fp32 and in
-        // the relative rounding of bf16) and the accumulators are rescaled rarely.
-        const bool move = tmax > m[c] + PF_LAZY;           // also the first tile (m = -inf) and never for -inf
-        const float m_new = move ? tmax : m[c];
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        // the relative rounding of bf16) and the accumulators are rescaled rarely.  A column's maximum lies in one
+        // of its four lanes, so a column has to move exactly when one of its lanes sees such a score among its own
+        // eight keys: the lanes look at their own keys only, and the maximum over the lanes of a column (two
+        // exchanges through LDS) is worked out only in the rounds in which some column of the wave moves: the
+        // first ones of a row, and few after them.  (The scale is positive: the maximum is taken of the raw
+        // scores and scaled once.)
+        const float lmax = scale_log2 * fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                                              fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+        if (__any(lmax > m[c] + PF_LAZY)) {                  // never for -inf; always in a column's first tile
+          float tmax = fmaxf(lmax, __shfl_xor(lmax, 16, IA_WAVE));
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE));
+          const float m_new = (tmax > m[c] + PF_LAZY) ? tmax : m[c];
+          const float corr = __builtin_amdgcn_exp2f(m[c] - ((m_new == -INFINITY) ? 0.f : m_new));   // 1 where nothing moved
+          lacc[c] *= corr;
+#pragma unroll
+          for (int n = 0; n < NS; ++n) o[c][n] *= corr;
+          m[c] = m_new;
+        }
+        const float m_safe = (m[c] == -INFINITY) ? 0.f : m[c];
         // probabilities are rounded to bf16 by the hardware conversion (nearest even); their sum is taken by the
         // matrix cores of the same rounded values (a product with a tile of ones), so that numerator and
         // denominator of the softmax agree and the vector units are spared the additions
@@ -762,13 +808,6 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
                        __builtin_amdgcn_exp2f(fmaf(sv[2 * r + 1], scale_log2, -m_safe))};
           pk[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(e, bf16x2_t));
         }
-        if (__any(move)) {
-          const float corr = __builtin_amdgcn_exp2f(m[c] - m_safe);      // 1 for the columns that did not move
-          lacc[c] *= corr;
-#pragma unroll
-          for (int n = 0; n < NS; ++n) o[c][n] *= corr;
-        }
-        m[c] = m_new;
         pb[c] = __builtin_bit_cast(bf16x8_t, make_uint4(pk[0], pk[1], pk[2], pk[3]));
         lacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[c], lacc[c], 0, 0, 0);
       }
@@ -781,8 +820,12 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
       }
     }
     }
-    if (more) store_tile(buf ^ 1);
+    if (t < t_end) store_tile(buf ^ 1, other{});      // tile t + 1, asked for a round ago
     __syncthreads();
+  };
+  for (int t = t_begin; t <= t_end; t += 2) {
+    round(t, set0{});
+    if (t + 1 <= t_end) round(t + 1, set1{});
   }
   if (bad) s_poison = 1;      // a key that is needed has no page in the block table: the result is NaN
   __syncthreads();
@@ -897,12 +940,18 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
   return IA_OK;
 }
 
-// heads_per_workgroup: 0 lets this function choose; 1, 2 or 4 (4 up to a head size of 160) asks for that many
+// launch_shape, low byte: 0 lets this function choose; 1, 2 or 4 (4 up to a head size of 160) asks for that many
 // groups of four waves, one query head each, that share the tiles of keys and values a workgroup brings in.
+// Bit 8 (IA_PREFILL_PAIRED): a workgroup takes 32 rows from each end of its request's new tokens in place of 64
+// consecutive ones (see the kernel); tiles must then list every block of 64 rows of every request, as the
+// engine's do.  The result has the same bits whatever the shape.
+#define IA_PREFILL_PAIRED 0x100
 extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
                                int out_row_stride, const int* seq_starts, const int* seq_ctx, const int* block_tables,
                                int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
-                               float scale, int window, int heads_per_workgroup, hipStream_t stream) {
+                               float scale, int window, int launch_shape, hipStream_t stream) {
+  if (launch_shape < 0 || (launch_shape & ~(0xff | IA_PREFILL_PAIRED))) return IA_ERR_BAD_ARG;
+  const int heads_per_workgroup = launch_shape & 0xff, paired = (launch_shape & IA_PREFILL_PAIRED) ? 1 : 0;
   if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
       bt_stride <= 0 || !(scale > 0.f))
     return IA_ERR_BAD_ARG;
@@ -929,7 +978,8 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
 #define PF_LAUNCH_P(C, W, P2)                                                                                     \
   attn_prefill_kernel<C, W, P2><<<grid, 4 * W * 64, 0, stream>>>(                                                 \
       (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
-      out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window)
+      out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window, \
+      paired)
 #define PF_LAUNCH(C, W)                      \
   do {                                       \
     if ((ps & (ps - 1)) == 0) PF_LAUNCH_P(C, W, true); \

@@ -170,8 +170,8 @@ class StepProgram:
                     if nd > 0:
                         s = K.decode_splits(nd, a["nh"], a["nkv"], ctx.max_total_len)
                     if ctx.num_seqs > nd:
-                        w = K.prefill_heads_per_workgroup(a["nh"], a["nkv"], a["d"], ctx.q_lens[nd:], ctx.ctx_lens[nd:],
-                                                          a["window"], dev)
+                        w = K.prefill_launch_shape(a["nh"], a["nkv"], a["d"], ctx.q_lens[nd:], ctx.ctx_lens[nd:],
+                                                   a["window"], dev)
                         if tiles is None:
                             tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
                 got = memo[key] = (s, w)

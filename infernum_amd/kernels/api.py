@@ -553,18 +553,21 @@ def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[t
 
 
 PREFILL_TILE_ROWS = 64      # query rows of a workgroup's tile in attention_prefill
+PREFILL_PAIRED = 0x100      # in a launch shape: 32 rows from each end of a request in place of 64 consecutive ones
 
 
 def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
                       tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, d: int, scale: float,
-                      window: int, heads_per_workgroup: int = 0) -> None:
+                      window: int, heads_per_workgroup: int = 0, paired: bool = False) -> None:
     """bf16 causal attention of portions of prompts over their pages, on MFMA.
 
     Request s brings rows seq_starts[s] .. seq_starts[s+1]-1 of qkv and had seq_ctx[s] tokens cached
     before; tiles[i] = (s, first row of a block of PREFILL_TILE_ROWS among the request's rows).  ``heads_per_workgroup``:
-    0 for the kernel's own choice, or 1, 2, 4 (see :func:`prefill_heads_per_workgroup`); the result has the
-    same bits whichever is taken.
+    0 for the kernel's own choice, or 1, 2, 4; ``paired``: a workgroup takes half a block of rows from each end of
+    its request's new tokens, so that all workgroups of a request have the same work under the causal mask (every
+    block of every request must be listed then).  A value of :func:`prefill_launch_shape` may stand in
+    ``heads_per_workgroup`` for both.  The result has the same bits whatever the shape.
     """
     _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, "attention_prefill")
     _need(qkv.dtype == torch.bfloat16, "attention_prefill: bf16 only")
@@ -577,27 +580,34 @@ def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     _need(ps % 4 == 0, f"attention_prefill: page size {ps} is not a multiple of 4")
     _ok(_attn(d).ia_attn_prefill(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d, _p(seq_starts),
                                  _p(seq_ctx), _p(block_tables), block_tables.shape[1], _p(tiles), num_tiles, nh, nkv,
-                                 ps, k_pages.shape[0], ctypes.c_float(scale), int(window), int(heads_per_workgroup),
-                                 _stream()),
+                                 ps, k_pages.shape[0], ctypes.c_float(scale), int(window),
+                                 int(heads_per_workgroup) | (PREFILL_PAIRED if paired else 0), _stream()),
         "attention_prefill")
 
 
 _compute_units: Dict[int, int] = {}
 
 
-def prefill_heads_per_workgroup(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_lens: Sequence[int],
-                                window: int, device: torch.device) -> int:
-    """How many query heads should share a workgroup's tiles of keys in :func:`attention_prefill` for these
-    portions of prompts (``q_lens`` new tokens after ``ctx_lens`` cached ones each); 0: the kernel's default.
+def prefill_launch_shape(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_lens: Sequence[int],
+                         window: int, device: torch.device) -> int:
+    """The shape of the :func:`attention_prefill` launch for these portions of prompts (``q_lens`` new tokens
+    after ``ctx_lens`` cached ones each): how many query heads share a workgroup's tiles of keys (0: the kernel's
+    default), with :data:`PREFILL_PAIRED` added when a workgroup should take half its rows from each end of its
+    request.  The bits of the result do not depend on it; all figures are of the 8B shape (32 heads over 8, 128).
 
-    At head sizes 80 to 160 with three or more query heads to a key/value head the default is four.  Two
-    measure 20 to 28 % faster (8B shape: 79 against 94 us at 2,048 tokens, 135 against 176 us for 1,024 after
-    3,072) when the launch is small: when four heads a workgroup give fewer workgroups than three quarters of
-    the compute units, or no more than one a compute unit while the longest tile has 1.5 times the keys of the
-    average one (a prompt from its start), so that more, smaller workgroups fill what the long ones leave idle.
+    Four heads a workgroup (the default at head sizes 80 to 160 with three or more query heads to a key/value
+    head) read the keys least often but make few workgroups: when they would fill fewer than three quarters of
+    the compute units, two heads are taken (1,024 tokens: 34 against 49 us).  When the launch has no more
+    workgroups than compute units, every workgroup runs from start to end and the longest sets the time: under
+    the causal mask that is the last block of a prompt, with twice the rounds of the average one.  Paired rows
+    give all workgroups of a request the same work then (2,048 tokens: 66 against 89 us with four heads, 71 with
+    two unpaired; 2,048 after 2,048: 147 against 171).  With more workgroups than compute units the rounds of a
+    paired workgroup in which half its waves have run out of keys cost more than the balance gains (4,096
+    tokens: 220 against 192 us), and under a window the rows of the two ends share no keys: not paired then.
     """
-    if not (80 <= d <= 160) or nh // nkv < 3:
-        return 0
+    G = nh // nkv
+    widest = 4 if 80 <= d <= 160 else 2
+    hpw = widest if G >= 3 else (2 if G == 2 else 1)
     tiles = total = longest = 0
     for q, c in zip(q_lens, ctx_lens):
         for first in range(0, q, 64):           # a block of 64 rows sees the keys up to its last row, or a window's worth
@@ -613,12 +623,16 @@ def prefill_heads_per_workgroup(nh: int, nkv: int, d: int, q_lens: Sequence[int]
     cus = _compute_units.get(idx)
     if cus is None:
         cus = _compute_units[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
-    workgroups = tiles * nkv * ((nh // nkv + 3) // 4)
-    if 4 * workgroups < 3 * cus:
-        return 2
-    if workgroups <= cus and longest * tiles >= 1.5 * total:
-        return 2
-    return 0
+    workgroups = tiles * nkv * ((G + hpw - 1) // hpw)
+    if hpw == 4 and 4 * workgroups < 3 * cus:
+        hpw, workgroups = 2, tiles * nkv * ((G + 1) // 2)
+    if window == 0:
+        return hpw | (PREFILL_PAIRED if workgroups <= cus else 0)
+    # under a window: two heads where four would give at most one workgroup a compute unit with the longest
+    # block at 1.5 times the average (more, smaller workgroups fill what the long ones leave idle)
+    if hpw == 4 and workgroups <= cus and longest * tiles >= 1.5 * total:
+        hpw = 2
+    return hpw
 
 
 # ------------------------------------------------------------------------- sampling

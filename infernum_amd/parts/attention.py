@@ -181,11 +181,11 @@ class Attention(Mixer):
             K.attention_decode(qkv[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.positions[:nd], bt[:nd], nh, nkv,
                                d, self.scale, self.window, ctx.max_total_len)
         if ctx.num_seqs > nd:
-            key = ("prefill_heads_per_workgroup", nh, nkv, d, self.window)
+            key = ("prefill_launch_shape", nh, nkv, d, self.window)
             hpw = ctx.extras.get(key)
             if hpw is None:             # once per step for all layers of this shape
-                hpw = ctx.extras[key] = K.prefill_heads_per_workgroup(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:],
-                                                                      self.window, qkv.device)
+                hpw = ctx.extras[key] = K.prefill_launch_shape(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:],
+                                                               self.window, qkv.device)
             tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
             K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
                                 tiles, num_tiles, nh, nkv, d, self.scale, self.window, hpw)

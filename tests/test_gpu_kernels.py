@@ -573,36 +573,44 @@ def test_attention_mfma_prefill(nh, nkv, d, ps, window):
     K().attention_generic(case["q"], case["kp"], case["vp"], gen, case["token_seq"], case["positions"], case["bt"], nh,
                           nkv, d, scale, window)
     assert (out.double() - gen.double()).abs().max().item() <= 2e-2
-    # one, two or four query heads to a workgroup (four up to a head size of 160): the same bits
+    # one, two or four query heads to a workgroup (four up to a head size of 160), rows of a workgroup from one
+    # stretch or from both ends of the request: the same bits
     for hpw in (1, 2, 4):
-        other = torch.full_like(out, float("nan"))
-        if hpw == 4 and d > 160:
-            with pytest.raises(K().KernelError):
-                K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt, nh,
-                                      nkv, d, scale, window, heads_per_workgroup=hpw)
-            continue
-        K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt, nh, nkv, d,
-                              scale, window, heads_per_workgroup=hpw)
-        assert torch.equal(other, out), hpw
+        for paired in (False, True):
+            other = torch.full_like(out, float("nan"))
+            if hpw == 4 and d > 160:
+                with pytest.raises(K().KernelError):
+                    K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt,
+                                          nh, nkv, d, scale, window, heads_per_workgroup=hpw, paired=paired)
+                continue
+            K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt, nh,
+                                  nkv, d, scale, window, heads_per_workgroup=hpw, paired=paired)
+            assert torch.equal(other, out), (hpw, paired)
     with pytest.raises(K().KernelError):
         K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt, nh, nkv, d,
                               scale, window, heads_per_workgroup=3)
 
 
-def test_prefill_heads_per_workgroup():
-    """The choice for small launches at the head sizes that have four heads a workgroup by default."""
+def test_prefill_launch_shape():
+    """Heads per workgroup and pairing of rows for launches of different sizes."""
     api = K()
     dev = torch.device(DEV)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    pick = lambda q, c, d=128, nh=32, nkv=8, w=0: api.prefill_heads_per_workgroup(nh, nkv, d, q, c, w, dev)
+    P = api.PREFILL_PAIRED
+    pick = lambda q, c, d=128, nh=32, nkv=8, w=0: api.prefill_launch_shape(nh, nkv, d, q, c, w, dev)
     per_tile = 8                                 # workgroups a block of 64 rows gives with four heads each
-    few = [64 * max(1, cus // per_tile // 2)]    # half as many workgroups as compute units
-    assert pick(few, [0]) == 2
-    exactly = [64 * (cus // per_tile)]           # one a compute unit
-    assert pick(exactly, [0]) == 2               # a prompt from its start: the last block sees twice the average
-    assert pick(exactly, [3 * exactly[0]]) == 0  # after a long context all blocks are about alike
-    assert pick([4 * exactly[0]], [0]) == 0      # many workgroups a compute unit
-    assert pick(few, [0], d=64) == 0 and pick(few, [0], d=256) == 0 and pick(few, [0], nh=16) == 0
+    few = [64 * max(1, cus // per_tile // 2)]    # half as many workgroups as compute units: two heads, and
+    assert pick(few, [0]) == 2 | P               # still no more workgroups than compute units: paired
+    exactly = [64 * (cus // per_tile)]           # one workgroup a compute unit with four heads
+    assert pick(exactly, [0]) == 4 | P
+    assert pick(exactly, [3 * exactly[0]]) == 4 | P
+    assert pick([4 * exactly[0]], [0]) == 4      # many workgroups a compute unit: rows as they come
+    assert pick(few, [0], d=64) == 2 | P and pick(few, [0], d=256) == 2 | P
+    assert pick([64 * cus], [0], d=64) == 2
+    assert pick(few, [0], nh=16) == 2 | P and pick(few, [0], nh=8) == 1 | P
+    # under a window nothing is paired; two heads where four would leave one long workgroup a compute unit
+    assert pick(few, [0], w=100) == 2 and pick(exactly, [0], w=10 ** 6) == 2 and pick(exactly, [3 * exactly[0]], w=10 ** 6) == 4
+    assert pick([], []) == 0
 
 
 @pytest.mark.parametrize("splits", [None, 1, 3, 7])
