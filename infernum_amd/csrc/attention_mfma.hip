@@ -520,6 +520,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 #define PF_KROW (HD + 8)        // bf16 per key row in LDS: 16 bytes of padding spread the banks
 #define PF_VROW 40              // bf16 per dim row of V^T in LDS (32 keys + 8 of padding)
 #define PF_LAZY 6.0f            // log2 of how far the running maximum may run ahead of the reference point
+#define PF_LAZY_EXP 64.0f       // 2^PF_LAZY
 
 template <int CT, int HGW, bool POW2>
 __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
       const uint4 v = real ? *reinterpret_cast<const uint4*>(qrow + st * 32 + qd * 8) : make_uint4(0u, 0u, 0u, 0u);
       q32[c][st] = __builtin_bit_cast(bf16x8_t, v);
     }
-    m[c] = -INFINITY;
+    m[c] = ok ? -INFINITY : 0.f;       // a column without a row never asks for a reference point
     lacc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int n = 0; n < NS; ++n) o[c][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -779,34 +780,41 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
         }
         // The reference point of the exponentials follows the running maximum lazily: it moves only when the
         // maximum has grown by more than 2^PF_LAZY, so probabilities stay below 2^PF_LAZY (exact in fp32 and in
-        // the relative rounding of bf16) and the accumulators are rescaled rarely.  A column's maximum lies in one
-        // of its four lanes, so a column has to move exactly when one of its lanes sees such a score among its own
-        // eight keys: the lanes look at their own keys only, and the maximum over the lanes of a column (two
-        // exchanges through LDS) is worked out only in the rounds in which some column of the wave moves: the
-        // first ones of a row, and few after them.  (The scale is positive: the maximum is taken of the raw
-        // scores and scaled once.)
-        const float lmax = scale_log2 * fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                                              fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-        if (__any(lmax > m[c] + PF_LAZY)) {                  // never for -inf; always in a column's first tile
+        // the relative rounding of bf16) and the accumulators are rescaled rarely.  The exponentials are taken
+        // against the reference point as it stands; only when one of them comes out above 2^PF_LAZY in some lane
+        // of the wave, or a column has no reference point yet, the maximum of the scores is worked out (over a
+        // lane's eight keys, then over the four lanes of a column: two exchanges through LDS), the reference
+        // point moves, the accumulators are rescaled and the exponentials are taken again: in a row's first
+        // rounds, and in few after them.  (The scale is positive: the maximum is taken of the raw scores and
+        // scaled once.)
+        float m_safe = (m[c] == -INFINITY) ? 0.f : m[c];
+        float e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2, -m_safe));
+        const float emax = fmaxf(fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])), fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
+        if (__any(emax > PF_LAZY_EXP || m[c] == -INFINITY)) {
+          const float lmax = scale_log2 * fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                                                fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
           float tmax = fmaxf(lmax, __shfl_xor(lmax, 16, IA_WAVE));
           tmax = fmaxf(tmax, __shfl_xor(tmax, 32, IA_WAVE));
-          const float m_new = (tmax > m[c] + PF_LAZY) ? tmax : m[c];
-          const float corr = __builtin_amdgcn_exp2f(m[c] - ((m_new == -INFINITY) ? 0.f : m_new));   // 1 where nothing moved
+          const float m_new = (tmax > m[c] + PF_LAZY) ? tmax : m[c];        // never moves to -inf
+          m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+          const float corr = __builtin_amdgcn_exp2f(m[c] - m_safe);         // 1 where nothing moved, 0 at the start
           lacc[c] *= corr;
 #pragma unroll
           for (int n = 0; n < NS; ++n) o[c][n] *= corr;
           m[c] = m_new;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2, -m_safe));
         }
-        const float m_safe = (m[c] == -INFINITY) ? 0.f : m[c];
         // probabilities are rounded to bf16 by the hardware conversion (nearest even); their sum is taken by the
         // matrix cores of the same rounded values (a product with a tile of ones), so that numerator and
         // denominator of the softmax agree and the vector units are spared the additions
         uint32_t pk[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          f32x2_t e = {__builtin_amdgcn_exp2f(fmaf(sv[2 * r], scale_log2, -m_safe)),
-                       __builtin_amdgcn_exp2f(fmaf(sv[2 * r + 1], scale_log2, -m_safe))};
-          pk[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(e, bf16x2_t));
+          f32x2_t e2 = {e[2 * r], e[2 * r + 1]};
+          pk[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(e2, bf16x2_t));
         }
         pb[c] = __builtin_bit_cast(bf16x8_t, make_uint4(pk[0], pk[1], pk[2], pk[3]));
         lacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[c], lacc[c], 0, 0, 0);
