@@ -1,6 +1,6 @@
 """The engine against the plain implementation at the layer sizes of Llama-3.1-8B (width 4,096, 32 heads on 8
-key/value heads of 128, feed-forward width 14,336, the vocabulary of 128,256; two layers), under all four ways of
-cutting, in 32-bit and in bfloat16.
+key/value heads of 128, feed-forward width 14,336, the vocabulary of 128,256; two layers), and of the 13B and 1B
+shapes that the benchmarks also run, under all four ways of cutting, in 32-bit and in bfloat16.
 
 The tiny configurations cannot show what only these sizes have: inner dimensions of 4,096 and 14,336 split over
 workgroups and joined by the next kernel, four heads of 128 to a workgroup, a head of 128,256 rows.  Their
@@ -21,11 +21,23 @@ import trace_tools as TT
 
 pytestmark = pytest.mark.gpu
 
-RAW = {"model_type": "llama", "vocab_size": 128256, "hidden_size": 4096, "intermediate_size": 14336,
-       "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "rope_theta": 500000.0,
-       "max_position_embeddings": 8192, "rms_norm_eps": 1e-5,
-       "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
-                        "original_max_position_embeddings": 8192}}
+_LLAMA3 = {"rope_type": "llama3", "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
+# Two layers of each shape that the benchmarks run.  "13b": as many key/value heads as heads (one query head a
+# workgroup in the attention kernels, one used column of sixteen in the decode kernel's tiles), widths 5,120 and
+# 13,824 (54 chunks of 256 for the split products), no scaling of the rotation.  "1b": heads of 64, the head tied to
+# the embedding, a scaling factor of 32; its vocabulary is cut to 16,001 (odd) to keep the float64 model short.
+SHAPES = {
+    "8b": {"model_type": "llama", "vocab_size": 128256, "hidden_size": 4096, "intermediate_size": 14336,
+           "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "rope_theta": 500000.0,
+           "max_position_embeddings": 8192, "rms_norm_eps": 1e-5, "rope_scaling": dict(_LLAMA3, factor=8.0)},
+    "13b": {"model_type": "llama", "vocab_size": 32000, "hidden_size": 5120, "intermediate_size": 13824,
+            "num_hidden_layers": 2, "num_attention_heads": 40, "num_key_value_heads": 40, "rope_theta": 10000.0,
+            "max_position_embeddings": 4096, "rms_norm_eps": 1e-5},
+    "1b": {"model_type": "llama", "vocab_size": 16001, "hidden_size": 2048, "intermediate_size": 8192,
+           "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+           "rope_theta": 500000.0, "max_position_embeddings": 131072, "rms_norm_eps": 1e-5,
+           "tie_word_embeddings": True, "rope_scaling": dict(_LLAMA3, factor=32.0)},
+}
 LENGTHS = (200, 61, 130)
 
 
@@ -33,12 +45,13 @@ def _ratio(a: torch.Tensor, ref: torch.Tensor) -> float:
     return float((a.double() - ref).abs().max() / ref.pow(2).mean().sqrt())
 
 
-@pytest.fixture(scope="module")
-def real(tmp_path_factory):
+@pytest.fixture(scope="module", params=list(SHAPES))
+def real(request, tmp_path_factory):
+    RAW = SHAPES[request.param]
     from infernum_amd.config import LlamaConfig
     from infernum_amd.weights import write_random_model
-    d = str(tmp_path_factory.mktemp("real_sizes"))
-    cfg = LlamaConfig.from_dict(RAW, where="real sizes")
+    d = str(tmp_path_factory.mktemp("real_sizes_" + request.param))
+    cfg = LlamaConfig.from_dict(RAW, where="real sizes " + request.param)
     write_random_model(cfg, d, 5, dtype=torch.bfloat16, made_on="cuda:0", norm_init=("uniform", 0.5, 1.5))
     pcfg, w = P.read_model(d)
     reqs = TT.make_requests(RAW["vocab_size"], LENGTHS, seed=1)
@@ -50,7 +63,7 @@ def real(tmp_path_factory):
     short = min(reqs, key=lambda r: len(reqs[r]))
     e32 = _ratio(P.forward(pcfg, w, reqs[short], dtype=torch.float32), exact[short])
     ebf = max(_ratio(rounding[r], exact[r]) for r in reqs)
-    print(f"real sizes: plain fp32 against float64 {e32:.2e}; plain with bfloat16 roundings against exact {ebf:.2e}")
+    print(f"real sizes {request.param}: plain fp32 against float64 {e32:.2e}; plain with bfloat16 roundings against exact {ebf:.2e}")
     assert 1e-6 < e32 < 1e-4 and 1e-2 < ebf < 0.3, "the plain implementations disagree in a way rounding does not explain"
     return d, reqs, exact, rounding, e32, ebf
 
