@@ -264,3 +264,39 @@ def test_one_step_ahead_changes_no_token(folders, num_blocks):
         assert rt.engine.cache.free_pages() == num_blocks
     assert results[True] == results[False]
     assert results[True][1][0] == free_run[:free_run.index(eos)] and len(results[True][3][0]) == 1
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_one_step_ahead_under_random_loads(folders, seed):
+    """Random requests (greedy and sampled, some with a stop token) over pools so small that requests are set
+    back, with random limits of batch, portion and budget: in 32-bit, where a token's logits do not depend on what
+    else is in its step, one step ahead and one step at a time give every request the same tokens and endings."""
+    import random
+    from infernum_amd import GenerateOptions, SamplingParams
+    results = []
+    for ahead in (False, True):
+        rng = random.Random(1000 + seed)
+        d, cfg, w = folders[rng.choice("AB")]
+        vocab = cfg["vocab_size"]
+        ps, n_req = rng.choice((2, 4, 8, 16)), rng.randint(2, 8)
+        prompts = [[rng.randrange(vocab) for _ in range(rng.randint(1, 40))] for _ in range(n_req)]
+        opts = []
+        for _ in range(n_req):
+            sp = None if rng.random() < 0.5 else SamplingParams(temperature=rng.choice((0.3, 0.7, 1.2)),
+                                                               top_p=rng.choice((1.0, 0.9, 0.5)), seed=rng.randrange(1 << 30))
+            opts.append(GenerateOptions(max_new_tokens=rng.randint(1, 24), sampling=sp,
+                                        eos_token_id=rng.randrange(vocab) if rng.random() < 0.5 else None))
+        longest = max(len(p) + o.max_new_tokens for p, o in zip(prompts, opts))
+        pool = max(-(-longest // ps) + 1, rng.randint(3, 30))
+        rt = _runtime(d, "float32", block_size=ps, num_blocks=pool, max_batch_size=rng.choice((2, 3, 5)),
+                      max_prefill_tokens=rng.choice((3, 8, 64)), max_tokens_per_step=rng.choice((8, 16, 64)))
+        assert rt.look_ahead
+        rt.look_ahead = ahead
+        seqs = [rt.submit(p, o) for p, o in zip(prompts, opts)]
+        rt.run()
+        assert all(s.pending == 0 for s in seqs)
+        results.append([(list(s.generated_ids), s.error, s.finish_reason, len(s.generated_ids) <= o.max_new_tokens)
+                        for s, o in zip(seqs, opts)])
+        rt.engine.cache.check()
+        assert rt.engine.cache.free_pages() == pool
+    assert results[0] == results[1]
