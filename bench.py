@@ -205,7 +205,7 @@ def serve(a) -> int:
     from infernum_amd import BatchConfig, CacheConfig, Engine, GenerateOptions, LlamaConfig, Runtime
     cfg = LlamaConfig.from_dict(LLAMA_1B)
     bc = BatchConfig(max_batch_size=a.serve_batch, max_prefill_tokens=a.serve_chunk, block_size=PAGE_SIZE,
-                     num_blocks=a.serve_blocks, max_tokens_per_step=a.serve_chunk + a.serve_batch)
+                     num_blocks=a.serve_blocks, max_tokens_per_step=a.serve_budget or max(a.serve_chunk, a.serve_batch))
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16",
                                 cache_config=CacheConfig(page_size=bc.block_size, num_pages=bc.num_blocks,
                                                          num_state_slots=bc.max_batch_size),
@@ -302,6 +302,9 @@ def main() -> int:
     ap.add_argument("--serve-requests", type=int, default=128)
     ap.add_argument("--serve-batch", type=int, default=128)
     ap.add_argument("--serve-chunk", type=int, default=2048)
+    ap.add_argument("--serve-budget", type=int, default=0,
+                    help="tokens of a step, decoded ones and portions together (default: the larger of chunk and batch: a step of\n"
+                         "2,048 rows fills the library's tiles of 256, one of 2,100 pays for 2,304)")
     ap.add_argument("--serve-blocks", type=int, default=16384)
     a = ap.parse_args()
     if a.gpus != 1:
