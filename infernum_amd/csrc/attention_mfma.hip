@@ -952,14 +952,16 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
 // groups of four waves, one query head each, that share the tiles of keys and values a workgroup brings in.
 // Bit 8 (IA_PREFILL_PAIRED): a workgroup takes 32 rows from each end of its request's new tokens in place of 64
 // consecutive ones (see the kernel); tiles must then list every block of 64 rows of every request, as the
-// engine's do.  The result has the same bits whatever the shape.
+// engine's do.  Without effect under a window.  The result has the same bits whatever the shape.
 #define IA_PREFILL_PAIRED 0x100
 extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
                                int out_row_stride, const int* seq_starts, const int* seq_ctx, const int* block_tables,
                                int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
                                float scale, int window, int launch_shape, hipStream_t stream) {
   if (launch_shape < 0 || (launch_shape & ~(0xff | IA_PREFILL_PAIRED))) return IA_ERR_BAD_ARG;
-  const int heads_per_workgroup = launch_shape & 0xff, paired = (launch_shape & IA_PREFILL_PAIRED) ? 1 : 0;
+  // under a window the rows of the two ends share no keys, and the keys between them may have no page any more:
+  // rows are not paired then, whatever was asked for
+  const int heads_per_workgroup = launch_shape & 0xff, paired = ((launch_shape & IA_PREFILL_PAIRED) && window <= 0) ? 1 : 0;
   if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
       bt_stride <= 0 || !(scale > 0.f))
     return IA_ERR_BAD_ARG;

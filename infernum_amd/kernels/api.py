@@ -569,7 +569,7 @@ def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     before; tiles[i] = (s, first row of a block of PREFILL_TILE_ROWS among the request's rows).  ``heads_per_workgroup``:
     0 for the kernel's own choice, or 1, 2, 4; ``paired``: a workgroup takes half a block of rows from each end of
     its request's new tokens, so that all workgroups of a request have the same work under the causal mask (every
-    block of every request must be listed then).  A value of :func:`prefill_launch_shape` may stand in
+    block of every request must be listed then; without effect under a window).  A value of :func:`prefill_launch_shape` may stand in
     ``heads_per_workgroup`` for both.  The result has the same bits whatever the shape.
     """
     _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, "attention_prefill")
