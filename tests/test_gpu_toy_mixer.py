@@ -594,3 +594,166 @@ def test_a_part_between_projection_and_rotation(tmp_path, dtype):
         worst, rms, where = TT.error_against(got, ref)
         print(f"toy4 {dtype} {name}: {worst / rms:.2e} at {where}")
         assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+
+
+# ------------------------------------------------------------------------------------------------
+# The remaining kinds of parts as a model's own: a norm (centred, with a bias), an embedding (scaled, with a
+# learned vector per position added) and a head (with a cap on the logits) around the stock attention and
+# feed-forward.
+from infernum_amd.parts import Embedding, Head, Norm        # noqa: E402
+
+
+class CentredNorm(Norm):
+    """out = (s - mean(s)) / sqrt(var(s) + eps) * w + b with s = h + delta."""
+
+    def __init__(self, rt, size, eps):
+        super().__init__(rt)
+        self.size, self.eps = size, eps
+
+    def weights(self):
+        return {"weight": WeightSpec((self.size,), ("uniform", 0.5, 1.5), follows_compute_dtype=False),
+                "bias": WeightSpec((self.size,), ("normal", 0.1), follows_compute_dtype=False)}
+
+    def load(self, tensors):
+        self.w, self.b = tensors["weight"].float(), tensors["bias"].float()
+
+    def forward(self, h, delta, out=None, rows=None):
+        if delta is not None:
+            delta = delta.joined(torch.float32) if hasattr(delta, "joined") else delta.float()
+        if rows is not None:                               # only these rows, and h stays as it is
+            s = h.index_select(0, rows.long())
+            if delta is not None:
+                s = s + delta.index_select(0, rows.long())
+        else:
+            if delta is not None:
+                h += delta
+            s = h
+        c = s - s.mean(-1, keepdim=True)
+        y = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + self.eps) * self.w + self.b).to(self.rt.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+
+class ScaledPositionedEmbedding(Embedding):
+    """h[t] = sqrt(H) * E[id_t] + P[position_t]."""
+
+    def __init__(self, rt, vocab_size, hidden_size, max_positions):
+        super().__init__(rt)
+        self.V, self.H, self.L = vocab_size, hidden_size, max_positions
+
+    def weights(self):
+        return {"weight": WeightSpec((self.V, self.H), ("normal", 0.3)),
+                "positions": WeightSpec((self.L, self.H), ("normal", 0.2))}
+
+    def load(self, tensors):
+        self.table, self.pos = tensors["weight"], tensors["positions"]
+
+    def forward(self, ctx):
+        return (math.sqrt(self.H) * self.table[ctx.token_ids.long()].float()
+                + self.pos[ctx.positions.long()].float()).contiguous()
+
+
+class CappedHead(Head):
+    """logits = cap * tanh(W f / cap)."""
+
+    def __init__(self, rt, vocab_size, hidden_size, cap):
+        super().__init__(rt)
+        self.V, self.H, self.cap = vocab_size, hidden_size, cap
+
+    def weights(self):
+        return {"weight": WeightSpec((self.V, self.H), ("normal", 0.3))}
+
+    def load(self, tensors):
+        self.w = tensors["weight"]
+
+    def forward(self, x):
+        return self.cap * torch.tanh(x.float() @ self.w.float().t() / self.cap)
+
+
+@dataclass(frozen=True)
+class Toy5Config:
+    vocab_size: int = 53
+    hidden_size: int = 48
+    num_heads: int = 3
+    num_kv_heads: int = 1
+    intermediate_size: int = 72
+    max_positions: int = 96
+    cap: float = 5.0
+    eps: float = 1e-4
+    model_type: str = "toy-dressed"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return Toy5Config(**{k: v for k, v in raw.items() if k in Toy5Config.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy5_spec(cfg: Toy5Config) -> ModelSpec:
+    H, d = cfg.hidden_size, cfg.hidden_size // cfg.num_heads
+    norm = lambda prefix: PartSpec("centred", {"size": H, "eps": cfg.eps}, prefix)
+    layers = [LayerSpec("prenorm",
+                        PartSpec("attention", {"hidden_size": H, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
+                                               "head_dim": d, "init_std": 0.1,
+                                               "position": {"kind": "none", "params": {}}}, f"l.{i}.attn."),
+                        PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size, "init_std": 0.1},
+                                 f"l.{i}.ff."),
+                        norm(f"l.{i}.n1."), norm(f"l.{i}.n2.")) for i in range(2)]
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("scaled_positioned", {"vocab_size": cfg.vocab_size, "hidden_size": H,
+                                                              "max_positions": cfg.max_positions}, "emb."),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn."),
+                     head=PartSpec("capped", {"vocab_size": cfg.vocab_size, "hidden_size": H, "cap": cfg.cap}, "head."))
+
+
+def plain_forward5(cfg: Toy5Config, w, ids):
+    W = {k: v.double() for k, v in w.items()}
+    H, nh, nkv = cfg.hidden_size, cfg.num_heads, cfg.num_kv_heads
+    d, T = H // nh, len(ids)
+
+    def centred(x, p):
+        c = x - x.mean(-1, keepdim=True)
+        return c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + cfg.eps) * W[p + "weight"] + W[p + "bias"]
+
+    h = math.sqrt(H) * P.embedding(W["emb.weight"], ids) + W["emb.positions"][:T]
+    for l in range(2):
+        p = f"l.{l}.attn."
+        n = centred(h, f"l.{l}.n1.")
+        q = P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d)
+        k = P.linear(n, W[p + "k_proj.weight"]).reshape(T, nkv, d)
+        v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, nkv, d)
+        h = h + P.linear(P.causal_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, H), W[p + "o_proj.weight"])
+        m = centred(h, f"l.{l}.n2.")
+        h = h + P.linear(P.swiglu(P.linear(m, W[f"l.{l}.ff.gate_proj.weight"]), P.linear(m, W[f"l.{l}.ff.up_proj.weight"])),
+                         W[f"l.{l}.ff.down_proj.weight"])
+    return cfg.cap * torch.tanh(P.linear(centred(h, "fn."), W["head.weight"]) / cfg.cap)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_an_embedding_and_a_head_of_the_models_own(tmp_path, dtype):
+    register_part("norm", "centred", CentredNorm, replace=True)
+    register_part("embedding", "scaled_positioned", ScaledPositionedEmbedding, replace=True)
+    register_part("head", "capped", CappedHead, replace=True)
+    register_architecture("toy-dressed", Toy5Config, toy5_spec, replace=True)
+    cfg = Toy5Config()
+    d = write_random_model(cfg, str(tmp_path / "toy5"), seed=33,
+                           dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    _, w = P.read_model(d)
+    assert {"emb.positions", "fn.bias", "l.1.n2.bias", "head.weight"} <= set(w)
+    eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4,
+                                                                          poison_freed_pages=True))
+    assert eng.program is None and not eng.use_graphs           # parts of the model's own: through the parts, unrecorded
+    reqs = TT.make_requests(cfg.vocab_size, (37, 5, 52, 20), seed=8)
+    ref = {r: plain_forward5(cfg, w, t) for r, t in reqs.items()}
+    assert max(float(v.abs().max()) for v in ref.values()) <= cfg.cap
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=2)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy5 {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
