@@ -218,6 +218,8 @@ class Engine:
             rows = np.fromiter((index[i] for i in packed.order[:nd]), dtype=np.int32, count=nd)
             if nd == 0 or int(rows.max()) < 0:
                 rows = source = None
+            elif int(rows.max()) >= source.numel():
+                raise StepError(f"a token is to come from place {int(rows.max())} of the last step's {source.numel()} choices")
         return self._staging.upload(packed.host, out=out, token_off=packed.offsets[0], token_rows=rows, source=source)
 
     def _decode_step(self, entries: Sequence[StepEntry], device_tokens: Optional[tuple] = None,
@@ -244,12 +246,13 @@ class Engine:
         ctx.max_total_len = max(limit, ctx.max_total_len)
         if not self.use_graphs or seen < 1:
             return self._forward(ctx)
-        # second time this shape comes: record it (kernels were loaded by the first, eager run)
+        # second time this shape comes: record it (kernels were loaded by the first, eager run).  The device
+        # is idle before a recording is dropped: a replay of it may still be queued (the host runs a step ahead)
+        torch.cuda.synchronize(self.rt.device)
         while len(self._graphs) >= self.max_recorded_steps:
             oldest = next(iter(self._graphs))
             del self._graphs[oldest]                        # its memory returns to the graphs' pool
             self._shape_seen.pop(oldest, None)
-        torch.cuda.synchronize(self.rt.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self._graph_pool):
             logits = self._forward(ctx)

@@ -142,6 +142,33 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     return out
 
 
+def causal_attention_blocked(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                             window: Optional[int] = None, round_to: Optional[torch.dtype] = None,
+                             q_positions: Optional[torch.Tensor] = None, block: int = 512) -> torch.Tensor:
+    """What :func:`causal_attention` computes (the same formulas and citations), one head and a block of query
+    rows at a time, so that sequences of thousands of tokens take seconds; ``test_plain_pins`` holds the two
+    together.  ``q_positions`` [Tq]: q holds the queries of these places only (default: of every place)."""
+    Tq, nh, d = q.shape
+    nkv = k.shape[1]
+    pos = torch.arange(Tq) if q_positions is None else torch.as_tensor(q_positions, dtype=torch.long)
+    out = torch.zeros_like(q)
+    for h in range(nh):
+        g = h * nkv // nh
+        for r0 in range(0, Tq, block):
+            p = pos[r0:r0 + block]
+            hi = int(p.max()) + 1
+            lo = 0 if not window else max(0, int(p.min()) - window + 1)
+            s = (q[r0:r0 + block, h, :] @ k[lo:hi, g, :].t()) * scale          # [rows, keys lo .. hi-1]
+            j = torch.arange(lo, hi)[None, :]
+            seen = j <= p[:, None]
+            if window:
+                seen &= j >= (p[:, None] - window + 1)
+            s = s.masked_fill(~seen, float("-inf"))
+            w = rounded(torch.exp(s - s.max(dim=1, keepdim=True).values), round_to)
+            out[r0:r0 + block, h, :] = (w @ v[lo:hi, g, :]) / w.sum(dim=1, keepdim=True)
+    return out
+
+
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """gate / (1 + exp(-gate)) * up.  infernum-cuda/kernels/silu.cu:36-40."""
     return gate / (1.0 + torch.exp(-gate)) * up
@@ -159,9 +186,15 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
 
 
 def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: Sequence[int], dtype=torch.float64,
-            round_to: Optional[torch.dtype] = None) -> torch.Tensor:
+            round_to: Optional[torch.dtype] = None, blocked: bool = False,
+            rows: Optional[Sequence[int]] = None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.  Order of operations:
     infernum-llama/src/graph_builder.rs:442-536.
+
+    ``blocked``: attention by :func:`causal_attention_blocked` (long sequences).  ``rows``: logits at these
+    places only, [len(rows), V]: the last layer works out its queries, its feed-forward and the head for them
+    alone (its keys and values still come from every token), which is what makes a sequence of tens of
+    thousands of tokens affordable when only its end is compared.
 
     ``round_to`` (torch.bfloat16) rounds every activation that an engine serving in that type stores between
     two operations: the outputs of norms, projections, the rotation, attention (and its exponentials), the
@@ -179,15 +212,25 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: Sequence[int], dtype=tor
     freqs = rope_frequencies(d, theta, cfg.get("rope_scaling"), dtype=dtype)
     T = len(ids)
     pos = torch.arange(T)
+    keep = None if rows is None else torch.as_tensor(list(rows), dtype=torch.long)
+    L = cfg["num_hidden_layers"]
     h = embedding(W["model.embed_tokens.weight"], ids)
-    for i in range(cfg["num_hidden_layers"]):
+    for i in range(L):
         p = f"model.layers.{i}."
         n = r(rms_norm(h, W[p + "input_layernorm.weight"], eps))
-        q = r(linear(n, W[p + "self_attn.q_proj.weight"])).reshape(T, nh, d)
         k = r(linear(n, W[p + "self_attn.k_proj.weight"])).reshape(T, nkv, d)
         v = r(linear(n, W[p + "self_attn.v_proj.weight"])).reshape(T, nkv, d)
-        q, k = r(rope(q, pos, freqs)), r(rope(k, pos, freqs))
-        a = r(causal_attention(q, k, v, 1.0 / math.sqrt(d), layer_window(cfg, i), round_to)).reshape(T, nh * d)
+        k = r(rope(k, pos, freqs))
+        q_pos = pos
+        if keep is not None and i == L - 1:         # from here on only the wanted places
+            n, h, q_pos = n[keep], h[keep], keep
+        q = r(linear(n, W[p + "self_attn.q_proj.weight"])).reshape(len(q_pos), nh, d)
+        q = r(rope(q, q_pos, freqs))
+        if blocked or len(q_pos) != T:
+            a = causal_attention_blocked(q, k, v, 1.0 / math.sqrt(d), layer_window(cfg, i), round_to, q_pos)
+        else:
+            a = causal_attention(q, k, v, 1.0 / math.sqrt(d), layer_window(cfg, i), round_to)
+        a = r(a).reshape(len(q_pos), nh * d)
         h = h + r(linear(a, W[p + "self_attn.o_proj.weight"]))
         m = r(rms_norm(h, W[p + "post_attention_layernorm.weight"], eps))
         act = r(swiglu(r(linear(m, W[p + "mlp.gate_proj.weight"])), r(linear(m, W[p + "mlp.up_proj.weight"]))))

@@ -456,9 +456,12 @@ def test_rope_from_partial_sums():
 
 
 # ------------------------------------------------------------------- attention
-def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
+def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None, loud=(), q_lift=0.0):
     """Random queries/keys/values of several requests laid out into shuffled pages.
-    Returns everything the kernels need plus the dense tensors for the reference."""
+    Returns everything the kernels need plus the dense tensors for the reference.
+    ``loud``: (request, key, value) sets the first component of that key (every head) to the value, and
+    ``q_lift`` is added to the first component of every query head: the key's score is about
+    q_lift * value * scale above the others for every query that sees it."""
     g = torch.Generator().manual_seed(seed)
     B = len(lens)
     pages_per = [-(-L // ps) for L in lens]
@@ -471,6 +474,8 @@ def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
     if scale_one is not None:                      # make one far key stand out
         b, j, factor = scale_one
         kd[b][j] *= factor
+    for b, j, value in loud:
+        kd[b][j][:, 0] = value
     kp = torch.zeros(num_pages, nkv, ps, d)
     vp = torch.zeros(num_pages, nkv, d, ps)
     it = iter(perm)
@@ -483,6 +488,8 @@ def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None):
             vp[p, :, :, :n] = vd[b][i * ps:i * ps + n].permute(1, 2, 0)
     N = sum(q_lens)
     q = torch.randn(N, nh * d, generator=g)
+    if q_lift:
+        q[:, ::d] += q_lift
     token_seq = torch.cat([torch.full((ql,), b, dtype=torch.int32) for b, ql in enumerate(q_lens)])
     positions = torch.cat([torch.arange(L - ql, L, dtype=torch.int32) for L, ql in zip(lens, q_lens)])
     to = lambda t: t.to(dtype).to(DEV)
@@ -589,6 +596,47 @@ def test_attention_mfma_prefill(nh, nkv, d, ps, window):
     with pytest.raises(K().KernelError):
         K().attention_prefill(case["q"], case["kp"], case["vp"], other, starts, ctx, case["bt"], tiles, nt, nh, nkv, d,
                               scale, window, heads_per_workgroup=3)
+
+
+@pytest.mark.parametrize("ctx0", [0, 200])
+@pytest.mark.parametrize("nh,nkv,d,ps", [(8, 2, 128, 16), (4, 2, 64, 8), (6, 1, 48, 4)])
+def test_attention_mfma_prefill_reference_point_moves_in_late_tiles(nh, nkv, d, ps, ctx0):
+    """The prefill kernel takes its exponentials against a reference point that it moves only when a score
+    comes out far above it.  Key 300 of 700 has some 2^29 times the weight of everything before it and key
+    520 some 2^58 times that: every row that sees them moves its point in its fifth and in its ninth tile of
+    keys, with sums of dozens of keys in its accumulators that have to be scaled down; rows of one tile see
+    the loud keys, rows of others do not.  Once for a whole prompt, once for a portion after 200 cached tokens
+    (whose first rows come before the first loud key); a second, short request rides along."""
+    L = 700
+    lens, q_lens = [L, 90], [L - ctx0, 90]
+    scale = 1.0 / math.sqrt(d)
+    lift = 6.0
+    case = _paged_case(nh, nkv, d, ps, lens, q_lens, torch.bfloat16, seed=11 + d, q_lift=lift,
+                       loud=[(0, 300, 20.0 / (lift * scale)), (0, 520, 60.0 / (lift * scale))])
+    N = case["N"]
+    starts = torch.tensor([0, q_lens[0], N], dtype=torch.int32, device=DEV)
+    ctx = torch.tensor([ctx0, 0], dtype=torch.int32, device=DEV)
+    tiles, nt = _prefill_tiles(q_lens)
+    want = _ref_attention(case, nh, nkv, d, scale, 0)
+    # the plain result itself says that the loud keys carry the rows behind them
+    v = case["vd"][0].double().cpu()
+    row = lambda p: want[p - ctx0].reshape(nh, d)[0]
+    assert (row(400) - v[300, 0]).abs().max() < 1e-3 and (row(699) - v[520, 0]).abs().max() < 1e-3
+    assert (row(299) - v[300, 0]).abs().max() > 0.1
+    gen = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K().attention_generic(case["q"], case["kp"], case["vp"], gen, case["token_seq"], case["positions"], case["bt"], nh,
+                          nkv, d, scale, 0)
+    assert (gen.double().cpu() - want).abs().max().item() <= 2e-2
+    first = None
+    for hpw in (1, 2, 4):
+        for paired in (False, True):
+            out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+            K().attention_prefill(case["q"], case["kp"], case["vp"], out, starts, ctx, case["bt"], tiles, nt, nh, nkv,
+                                  d, scale, 0, heads_per_workgroup=hpw, paired=paired)
+            err = (out.double().cpu() - want).abs().max().item()
+            assert err <= 2e-2, (hpw, paired, err)
+            first = out if first is None else first
+            assert torch.equal(out, first), (hpw, paired)
 
 
 def test_prefill_launch_shape():

@@ -123,6 +123,33 @@ def test_attention_window():
     assert not torch.allclose(out[t], full[t], atol=1e-6)
 
 
+def test_blocked_attention_is_the_attention_row_by_row():
+    """The form for long sequences (a head and a block of rows at a time) against the loop over tokens: whole,
+    under a window that cuts inside a block, with rounded exponentials, and for a few places only."""
+    q, k, v = (torch.randn(75, n, 8, dtype=torch.float64) for n in (6, 2, 2))
+    for window in (None, 9, 40):
+        for round_to in (None, torch.bfloat16):
+            want = P.causal_attention(q, k, v, 0.3, window, round_to)
+            for block in (7, 32, 512):
+                got = P.causal_attention_blocked(q, k, v, 0.3, window, round_to, block=block)
+                assert torch.allclose(got, want, atol=1e-12), (window, round_to, block)
+            rows = torch.tensor([3, 74, 20, 21])
+            some = P.causal_attention_blocked(q[rows], k, v, 0.3, window, round_to, q_positions=rows, block=3)
+            assert torch.allclose(some, want[rows], atol=1e-12)
+
+
+def test_whole_model_blocked_and_at_chosen_places(tmp_path):
+    import tiny_models as TM
+    for name in ("A", "C"):
+        cfg, w = P.read_model(TM.write_tiny(name, str(tmp_path / name)))
+        ids = [int(t) for t in torch.randint(0, cfg["vocab_size"], (45,))]
+        full = P.forward(cfg, w, ids)
+        assert torch.allclose(P.forward(cfg, w, ids, blocked=True), full, atol=1e-10)
+        assert torch.allclose(P.forward(cfg, w, ids, rows=[44, 7, 30]), full[[44, 7, 30]], atol=1e-10)
+        assert torch.allclose(P.forward(cfg, w, ids, rows=[0, 5], round_to=torch.bfloat16),
+                              P.forward(cfg, w, ids, round_to=torch.bfloat16)[[0, 5]], atol=1e-10)
+
+
 def test_swiglu_equals_library():
     g, u = torch.randn(4, 10, dtype=torch.float64), torch.randn(4, 10, dtype=torch.float64)
     assert torch.allclose(P.swiglu(g, u), torch.nn.functional.silu(g) * u, atol=1e-12)
