@@ -116,8 +116,8 @@ def test_long_prompts_whole_in_portions_and_with_a_decoded_tail(name, dtype, tmp
 @pytest.mark.parametrize("name", ["A", "W"])
 def test_a_dozen_tokens_decoded_after_33000(name, dtype, tmp_path_factory):
     """Pages of 16 tokens: 2,064 entries in a block table, more than the decode kernel keeps in LDS; the keys of
-    the one request are split over dozens of workgroups.  W: the window group's first 1,900 pages have long been
-    given back and the pool is so small that they were used again.  The plain model works out its last layer at
+    the one request are split over dozens of workgroups.  W: the window group has long given back the pages of
+    the first 31,000 tokens.  The plain model works out its last layer at
     the twelve places only."""
     from infernum_amd.engine import StepEntry
     from infernum_amd.kernels import api
