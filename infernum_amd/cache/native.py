@@ -48,21 +48,15 @@ _SIGNATURES = {
     "ia_cache_commit_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int)]),
     "ia_cache_unreserve_step": (c_int, [c_void_p, c_int, POINTER(c_int64)]),
     "ia_cache_check": (c_int, [c_void_p]),
-    # the native program of a step (csrc/step_program.cpp)
-    "ia_program_create": (c_void_p, [POINTER(c_int), c_int, c_void_p]),
+    # the interpreter of a step's program (csrc/step_program.cpp)
+    "ia_program_create": (c_void_p, []),
     "ia_program_destroy": (None, [c_void_p]),
     "ia_program_error": (c_char_p, [c_void_p]),
-    "ia_program_set_rotation": (None, [c_void_p, c_int]),
-    "ia_program_set_functions": (c_int, [c_void_p, POINTER(c_void_p), c_int]),
-    "ia_program_add_norm": (c_int, [c_void_p, c_void_p, c_int, c_float, c_int]),
-    "ia_program_add_attention": (c_int, [c_void_p, POINTER(c_int), c_int, c_float, POINTER(c_void_p), c_int,
-                                         POINTER(c_int)]),
-    "ia_program_add_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
-    "ia_program_set_head": (c_int, [c_void_p, c_void_p]),
-    "ia_program_finish": (c_size_t, [c_void_p, c_int]),
-    "ia_program_set_arena": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),
-    "ia_program_run": (c_int, [c_void_p, POINTER(c_int), c_int, POINTER(c_void_p), c_int, POINTER(c_int), POINTER(c_int),
-                               POINTER(c_int), c_int, c_void_p, c_void_p]),
+    "ia_program_num_ops": (c_int, [c_void_p]),
+    "ia_program_last_launches": (ctypes.c_longlong, [c_void_p]),
+    "ia_program_add_op": (c_int, [c_void_p, c_void_p, c_char_p, POINTER(c_int64), c_int, POINTER(c_int64), c_int, c_int]),
+    "ia_program_finish": (c_int, [c_void_p, c_int, c_int]),
+    "ia_program_run": (c_int, [c_void_p, POINTER(c_int64), c_int, POINTER(c_void_p), c_int, c_void_p]),
     "ia_cache_token_slots": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, POINTER(c_int32)]),
     "ia_cache_pack_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int), POINTER(c_int32), POINTER(c_int),
                                    POINTER(c_int32), c_int, c_int, POINTER(c_int32), c_int]),

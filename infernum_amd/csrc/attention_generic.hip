@@ -117,3 +117,7 @@ extern "C" int ia_attention_generic(const void* q, int q_row_stride, const void*
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_attention_generic)

@@ -1009,3 +1009,9 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_attn_decode)
+IA_OP(ia_attn_decode_fused)
+IA_OP(ia_attn_prefill)

@@ -44,7 +44,7 @@ CORE_SOURCES = [
     "sampling.hip",
     "peaks.hip",
 ]
-HEADERS = ["common.h", "no_alloc.h"]
+HEADERS = ["common.h", "no_alloc.h", "op_call.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
 HOST_SOURCES = ["host_core.cpp", "step_program.cpp"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
@@ -121,7 +121,7 @@ def _existing(files: Sequence[str]) -> List[str]:
 
 def _fingerprint(sources: Sequence[str], defines: Sequence[str], host: bool = False) -> str:
     h = hashlib.sha256()
-    for f in list(sources) + ([] if host else _existing(HEADERS)):
+    for f in list(sources) + _existing(HEADERS):
         with open(os.path.join(CSRC_DIR, f), "rb") as fh:
             h.update(f.encode())
             h.update(fh.read())

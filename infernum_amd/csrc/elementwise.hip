@@ -643,3 +643,12 @@ extern "C" int ia_words_to_host(void* host_dst, const void* src, int n, hipStrea
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_embed)
+IA_OP(ia_add_rmsnorm)
+IA_OP(ia_residual_add)
+IA_OP(ia_rope_kv_append)
+IA_OP(ia_swiglu)
+IA_OP(ia_cast)

@@ -103,3 +103,7 @@ extern "C" int ia_gemm_generic(const void* A, const void* W, void* C, int in_dty
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_gemm_generic)

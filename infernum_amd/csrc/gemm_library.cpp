@@ -163,3 +163,7 @@ extern "C" int ia_gemm_lt_plans() {
   std::lock_guard<std::mutex> lock(g_mu);
   return (int)g_plans.size();
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_gemm_lt)

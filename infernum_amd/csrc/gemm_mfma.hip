@@ -281,3 +281,7 @@ extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
   if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4, 1>(x, w, c, M, N, K, stream);
   return IA_ERR_BAD_ARG;
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_gemm_mfma)

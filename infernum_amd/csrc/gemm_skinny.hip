@@ -297,6 +297,22 @@ extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dty
   return launch_join<uint16_t>(workspace, (uint16_t*)C, M, N, splits, epilogue, stream);
 }
 
+// The same product for any number of rows, 128 at a time (a result in fp32 from bf16 operands has no other
+// kernel here: the head of a step that wants the logits of many places).  The workspace serves every piece in turn.
+extern "C" int ia_gemm_skinny_rows(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
+                                   float* workspace, size_t workspace_floats, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
+  if (out_dtype != IA_F32 && out_dtype != IA_BF16) return IA_ERR_BAD_ARG;
+  const size_t out_bytes = out_dtype == IA_F32 ? 4 : 2;
+  for (int m0 = 0; m0 < M; m0 += 128) {
+    const int m = M - m0 < 128 ? M - m0 : 128;
+    const int rc = ia_gemm_skinny((const char*)X + (size_t)m0 * K * 2, W, (char*)C + (size_t)m0 * N * out_bytes, out_dtype,
+                                  m, N, K, SK_EPI_NONE, workspace, workspace_floats, stream);
+    if (rc != IA_OK) return rc;
+  }
+  return IA_OK;
+}
+
 // ---- the same product for callers that cannot allocate: the workspace is an array of this library ----------
 #include <mutex>
 #include "no_alloc.h"
@@ -346,3 +362,8 @@ extern "C" int ia_gemm_skinny_no_alloc(const void* X, const void* W, void* C, in
   if (rc != IA_OK) return rc;
   return ia_gemm_skinny(X, W, C, out_dtype, M, N, K, epilogue, ws, IA_SKINNY_SCRATCH_FLOATS, stream);
 }
+
+// ---- the launchers of this file as operations of a step's program (see op_call.h) ----
+#include "op_call.h"
+IA_OP(ia_gemm_skinny)
+IA_OP(ia_gemm_skinny_rows)

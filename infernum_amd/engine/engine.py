@@ -75,16 +75,17 @@ class Engine:
         self.graph_replays = 0
         self.max_recorded_steps = MAX_RECORDED_STEPS
         self._staging = PinnedUpload(self.rt.device) if self.rt.device.type == "cuda" else None
-        # "native": the step's launches are made by the host library from one call where every part of the
-        # model has a native description (engine/program.py); "parts": by the parts' own forward, one Python
-        # call per launch.  The same launches either way.
+        # "native": the step's launches are made by the host library from one call, from the program that the
+        # model's parts wrote (engine/program.py; a part without launchers of its own is called back); "parts":
+        # by the parts' own forward, one Python call per launch (the twin that tests hold the program to, and
+        # the way of INFERNUM_PROFILE=1).  The same launches either way.
         executor = executor or os.environ.get("INFERNUM_EXECUTOR", "native")
         if executor not in ("native", "parts"):
             raise ValueError(f"executor must be 'native' or 'parts', got {executor!r}")
         self.program = None
         if executor == "native" and self.rt.device.type == "cuda":
             from .program import build
-            self.program = build(model, self.views, self.rt.max_tokens_per_step)
+            self.program = build(model, self.views, len(self.cache.groups), self.rt.max_tokens_per_step)
 
     # ---- building ------------------------------------------------------------------
     @staticmethod

@@ -424,6 +424,23 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
+def gemm_skinny_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T for any M through :func:`gemm_skinny`'s kernel, 128 rows at a time (an fp32
+    result from bf16 operands has no other kernel: the head of a step that wants the logits of many places)."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] == K,
+          "gemm_skinny_rows: bf16 operands [M, K] and [N, K]")
+    _need(M >= 1 and gemm_skinny_supported(1, N, K), f"gemm_skinny_rows: M={M} N={N} K={K} not supported (K % 8 == 0)")
+    _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (M, N), f"gemm_skinny_rows: out must be contiguous [{M}, {N}]")
+    splits = gemm_skinny_splits(N, K)
+    ws = torch.empty((splits, min(M, SKINNY_MAX_M), N), dtype=torch.float32, device=a.device) if splits > 1 else None
+    _ok(_core().ia_gemm_skinny_rows(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, _p(ws),
+                                    ctypes.c_size_t(ws.numel() if ws is not None else 0), _stream()), "gemm_skinny_rows")
+    return out
+
+
 # ------------------------------------------------------------------------ attention
 def _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, what):
     _dev(qkv, k_pages, v_pages, out, block_tables)
@@ -687,7 +704,7 @@ def attention_mfma_available(d: int) -> bool:
 # same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
 # are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
 _PROFILED = ("cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
-             "gemm_library", "gemm_skinny", "attention_generic", "attention_decode", "attention_decode_rotating",
+             "gemm_library", "gemm_skinny", "gemm_skinny_rows", "attention_generic", "attention_decode", "attention_decode_rotating",
              "attention_prefill", "argmax", "repetition_penalty", "sample")
 _profile_on = False
 _profile_open: List[Tuple[str, "torch.cuda.Event", "torch.cuda.Event"]] = []

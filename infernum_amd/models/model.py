@@ -101,6 +101,31 @@ class DecoderModel:
                 needs.append((m.cache_spec(), m.state_spec()))
         return needs
 
+    # ---- the step as a program ------------------------------------------------------
+    def native(self, program, views: List[CacheView]) -> None:
+        """Every part writes its operations into ``program`` (engine/program.StepProgram), in the order in which
+        ``_forward`` below calls the parts' ``forward``."""
+        self.embedding.native(program, None)
+        for e, view in zip(self.spec.schedule, views):
+            self.blocks[e.layer].native(program, view)
+        if self.final_norm is not None:
+            self.final_norm.native(program, None, rows=True)
+        else:
+            pending, H, dt = program.pending, self.spec.hidden_size, self.rt.dtype
+
+            def wanted_rows(ctx: StepContext) -> None:
+                from ..kernels import api as K
+                n, rows = ctx.num_tokens, ctx.logit_rows
+                if rows.numel() == 0:
+                    return
+                h, delta = program.h.view(torch.float32, n, H), program.read(pending, n)
+                if delta is not None:
+                    K.residual_add(h, delta.joined(dt) if isinstance(delta, K.SplitSum) else delta)
+                program.x.view(dt, rows.numel(), H).copy_(h.index_select(0, rows.long()))
+            program.python(wanted_rows, "wanted rows")
+            program.pending = None
+        self.head.native(program, None)
+
     # ---- one step --------------------------------------------------------------
     def forward(self, ctx: StepContext, views: List[CacheView]) -> torch.Tensor:
         """Runs the tokens of ``ctx`` and returns fp32 logits [R, V] at ctx.logit_rows."""

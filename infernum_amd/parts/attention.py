@@ -24,7 +24,7 @@ import torch
 from ..kernels import api as K
 from .base import (CacheSpec, CacheView, Mixer, PartSpec, Runtime, StepContext, WeightSpec, make_part,
                    register_part)
-from .linear import linear, measure_routes_for
+from .linear import emit_linear, linear, measure_routes_for
 
 
 # Steps of up to this many single tokens rotate inside the attention kernel (8B shape: 1.5 % faster at 1 and 8
@@ -158,16 +158,99 @@ class Attention(Mixer):
         self.attend(q, out, ctx, cache)
         return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
-    def native(self, program, view: CacheView) -> bool:
-        from . import rope
-        if type(self) is not Attention or type(self.position) not in (rope.RotaryEmbedding, rope.NoPositionEncoding):
-            return False                      # a subclass may do something else in forward
-        if self.qk_transform is not None:
-            return False                      # a part of the model's own between projection and rotation
+    def native(self, program, view: CacheView) -> None:
+        """The launches of ``forward`` and ``attend``, each with the steps it is for: steps of up to
+        ROTATE_IN_ATTENTION_UP_TO single tokens take the kernel that rotates, writes the pages and attends in one
+        launch; all others the rotary kernel, then the kernel for single tokens on the first rows and the one for
+        portions of prompts on the rest (or the plain kernel on all rows)."""
+        if type(self).forward is not Attention.forward or type(self).attend is not Attention.attend:
+            return super().native(program, view)              # a subclass that computes something else
+        from ..engine.program import NEVER, STREAM, Guard
         if view is None or view.k_pages is None or view.v_pages is None:
-            return False
-        program.add_attention(self, view)
-        return True
+            raise K.KernelError("attention needs pages of the cache")
+        nh, nkv, d, window, rt = self.nh, self.nkv, self.d, self.window, self.rt
+        k, v, g, writable = view.k_pages, view.v_pages, view.group, view.writable
+        ps, num_pages = int(k.shape[2]), int(k.shape[0])
+        inv_freq = self.position.inv_freq
+        rot = self.position.rotary_dim if inv_freq is not None else 0
+        f64 = int(inv_freq is not None and inv_freq.dtype == torch.float64)
+        w = self.w_qkv if writable else self.w_qkv[: nh * d]     # another run's keys and values: only queries are made
+        row, T, N = int(w.shape[0]), program.T, program.N
+        act, scale = program.act_code, float(self.scale)
+        mfma = self.use_mfma and ps % 4 == 0
+        program.keep(k, v, inv_freq, w)
+        bt, bt_cols = program.block_table(g), program.bt_cols(g)
+        slots = program.slots(g) if writable else None
+        out = program.buffer("attention.out", T * nh * d * program.act_bytes)
+        fused = NEVER
+        if mfma and self.rotate_in_attention and self.qk_transform is None:
+            fused = Guard.between(program.NPT, 0, 0) & Guard.between(N, 1, ROTATE_IN_ATTENTION_UP_TO)
+        separate = ~fused
+        if mfma:
+            lib = K._attn(d)
+            records = T + 1024      # requests x parts of their keys: what fills the GPU, or the requests themselves
+            part_o = program.buffer("attention.part_o", records * nh * d * 4)
+            part_ml = program.buffer("attention.part_ml", records * nh * 2 * 4)
+            dev = rt.device
+
+            def parts_of_the_keys(ctx: StepContext) -> int:
+                nd = ctx.num_decode
+                if nd == 0:
+                    return 1
+                if ctx.block_tables[g].shape[1] * ps < ctx.max_total_len:
+                    raise K.KernelError("attention: the block tables are narrower than the longest request")
+                n = K.decode_splits(nd, nh, nkv, ctx.max_total_len)
+                if nd * n > records:
+                    raise K.KernelError("attention: the parts of the keys do not fit the program's arena")
+                return n
+
+            def launch_shape(ctx: StepContext) -> int:
+                nd = ctx.num_decode
+                if ctx.num_seqs == nd:
+                    return 0
+                return K.prefill_launch_shape(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:], window, dev)
+            splits = program.scalar(("attention: parts of the keys", nh, nkv, g, ps), parts_of_the_keys)
+            shape = program.scalar(("attention: launch shape", nh, nkv, d, window), launch_shape)
+            tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
+        qkv = emit_linear(program, program.x, N, w, rt.dtype, None, self.qk_transform is None, "attention.qkv",
+                          "attention.qkv")
+        if self.qk_transform is not None:
+            where, transform, kv_heads = qkv.tensor(), self.qk_transform, (nkv if writable else 0)
+
+            def between_projection_and_rotation(ctx: StepContext) -> None:
+                t = where.view(rt.dtype, ctx.num_tokens, row)
+                y = transform.forward(t, nh, kv_heads, d, ctx)
+                if y.data_ptr() != t.data_ptr():
+                    t.copy_(y)
+            program.python(between_projection_and_rotation, type(transform).__name__)
+        for alt in qkv.alts:
+            src, code, parts = alt.where, (K.DTYPE_CODE[torch.float32] if alt.splits else act), (alt.splits or 1)
+            if mfma:
+                program.op(lib, "ia_attn_decode_fused",
+                           [src, code, parts, N, row, slots, inv_freq, f64, rot, k, v, out, nh * d, part_o, part_ml,
+                            program.positions, bt, bt_cols, N, nh, nkv, ps, num_pages, scale, window, splits, STREAM],
+                           alt.when & fused)
+            q, q_stride = src, row
+            if alt.splits:                   # partial sums: the rotated queries get a tensor of their own
+                q, q_stride = program.buffer("attention.q", T * nh * d * program.act_bytes), nh * d
+            program.op("core", "ia_rope_kv_append",
+                       [src, code, parts, N, q, q_stride, act, program.positions, slots, inv_freq, f64,
+                        k if writable else None, v if writable else None, N, row, nh, nkv, d, rot,
+                        ps if writable else 0, num_pages if writable else 0, int(writable), STREAM], alt.when & separate)
+            if not mfma:
+                program.op("core", "ia_attention_generic",
+                           [q, q_stride, k, v, out, nh * d, act, program.token_seq, program.positions, bt, bt_cols, N, nh,
+                            nkv, d, ps, num_pages, scale, window, STREAM], alt.when & separate)
+                continue
+            program.op(lib, "ia_attn_decode",
+                       [q, q_stride, k, v, out, nh * d, part_o, part_ml, program.positions, bt, bt_cols, program.ND, nh,
+                        nkv, ps, num_pages, scale, window, splits, STREAM],
+                       alt.when & separate & Guard.between(program.ND, 1))
+            program.op(lib, "ia_attn_prefill",
+                       [q, q_stride, k, v, out, nh * d, program.seq_starts, program.seq_ctx, bt, bt_cols, tiles, num_tiles,
+                        nh, nkv, ps, num_pages, scale, window, shape, STREAM],
+                       alt.when & separate & Guard.between(program.NP, 1))
+        program.pending = emit_linear(program, out, N, self.w_o, rt.dtype, None, True, "attention.mix", "attention.o")
 
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d

@@ -251,10 +251,12 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Take the tensors of ``weights`` (by local name), already on the device."""
 
-    def native(self, program: Any, view: Optional["CacheView"], **kw: Any) -> bool:
-        """Add this part to the native program of a step (``engine.program.StepProgram``) as the operation that
-        makes the launches of ``forward``; False when it has none (the model then runs through the parts)."""
-        return False
+    def native(self, program: Any, view: Optional["CacheView"], **kw: Any) -> None:
+        """Write this part into the program of a step (``engine.program.StepProgram``): the operations that
+        make the launches of ``forward``, reading and leaving the program's registers as ``forward`` reads its
+        arguments and returns its result.  Every category has a default that calls back into ``forward``; a
+        part with launchers of its own writes them instead (``program.op``)."""
+        raise NotImplementedError(f"{type(self).__name__} has no category that a program knows")
 
     def step_needs(self) -> Dict[str, Any]:
         """Arrays that the part wants packed with every step beyond those every step has.  Known:
@@ -271,6 +273,25 @@ class Norm(Part):
         ``delta`` is what a mixer or a feed-forward returned: a tensor [N, H] in the compute dtype, or
         a ``kernels.api.SplitSum`` (fp32 partial sums [S, N, H] that are added here)."""
         raise NotImplementedError
+
+    def native(self, program: Any, view: Optional["CacheView"] = None, rows: bool = False) -> None:
+        """Reads ``program.h`` and ``program.pending``, leaves the normalised rows in ``program.x`` (of the wanted
+        rows only with ``rows``).  This default calls ``forward``."""
+        pending, H, dt = program.pending, program.hidden_size, self.rt.dtype
+
+        def call(ctx: "StepContext") -> None:
+            n = ctx.num_tokens
+            h = program.h.view(torch.float32, n, H)
+            picked = ctx.logit_rows if rows else None
+            n_out = int(picked.numel()) if rows else n
+            if n_out == 0:
+                return
+            out = program.x.view(dt, n_out, H)
+            y = self.forward(h, program.read(pending, n), out=out, rows=picked)
+            if y.data_ptr() != out.data_ptr():
+                out.copy_(y)
+        program.python(call, type(self).__name__)
+        program.pending = None
 
 
 class PositionEncoding(Part):
@@ -306,6 +327,10 @@ class Mixer(Part):
         next norm joins); reads and writes its cache view."""
         raise NotImplementedError
 
+    def native(self, program: Any, view: Optional["CacheView"]) -> None:
+        """Reads ``program.x``, leaves its result as ``program.pending``.  This default calls ``forward``."""
+        _call_forward(self, program, "mixer.out", lambda x, ctx: self.forward(x, ctx, view))
+
 
 class FeedForward(Part):
     category = "feed_forward"
@@ -313,6 +338,10 @@ class FeedForward(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext) -> Any:
         """x [N, H] in the compute dtype -> [N, H] (a tensor, or a SplitSum that the next norm joins)."""
         raise NotImplementedError
+
+    def native(self, program: Any, view: Optional["CacheView"] = None) -> None:
+        """Reads ``program.x``, leaves its result as ``program.pending``.  This default calls ``forward``."""
+        _call_forward(self, program, "feed_forward.out", lambda x, ctx: self.forward(x, ctx))
 
 
 class Embedding(Part):
@@ -322,6 +351,13 @@ class Embedding(Part):
         """-> the residual stream h [N, H] in fp32."""
         raise NotImplementedError
 
+    def native(self, program: Any, view: Optional["CacheView"] = None) -> None:
+        """Fills ``program.h``.  This default calls ``forward``."""
+        H = program.hidden_size
+        program.python(lambda ctx: program.h.view(torch.float32, ctx.num_tokens, H).copy_(self.forward(ctx)),
+                       type(self).__name__)
+        program.pending = None
+
 
 class Head(Part):
     category = "head"
@@ -329,6 +365,16 @@ class Head(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x [R, H] -> logits [R, V] fp32."""
         raise NotImplementedError
+
+    def native(self, program: Any, view: Optional["CacheView"] = None) -> None:
+        """Reads the wanted rows from ``program.x``, fills the step's logits.  This default calls ``forward``."""
+        H, dt = program.hidden_size, self.rt.dtype
+
+        def call(ctx: "StepContext") -> None:
+            R = int(ctx.logit_rows.numel())
+            if R:
+                program.step_logits().copy_(self.forward(program.x.view(dt, R, H)))
+        program.python(call, type(self).__name__)
 
 
 class Block:
@@ -355,10 +401,36 @@ class Block:
                 cache: CacheView) -> torch.Tensor:
         raise NotImplementedError
 
-    def native(self, program: Any, view: CacheView) -> bool:
-        """Add the arrangement's parts to the native program in the order ``forward`` runs them; False when
-        the arrangement or one of its parts has no native description."""
-        return False
+    def native(self, program: Any, view: CacheView) -> None:
+        """Write the arrangement into a step's program: its parts' operations in the order ``forward`` runs them
+        (each part's ``native``).  This default calls ``forward`` for the whole layer."""
+        pending, H, dt = program.pending, program.hidden_size, self.rt.dtype
+        buf, value = program.store("block.out", H)
+
+        def call(ctx: StepContext) -> None:
+            n = ctx.num_tokens
+            out = self.forward(program.h.view(torch.float32, n, H), program.read(pending, n), ctx, view)
+            _put(buf.view(dt, n, H), out, dt)
+        program.python(call, type(self).__name__)
+        program.pending = value
+
+
+def _put(dst: torch.Tensor, y: Any, dtype: torch.dtype) -> None:
+    """What a part's ``forward`` returned (a tensor or partial sums), into a buffer of the program."""
+    if hasattr(y, "joined"):
+        y = y.joined(dtype)
+    dst.copy_(y)
+
+
+def _call_forward(part: Part, program: Any, key: str, forward: Callable[[torch.Tensor, StepContext], Any]) -> None:
+    H, dt = program.hidden_size, part.rt.dtype
+    buf, value = program.store(key, H)
+
+    def call(ctx: StepContext) -> None:
+        n = ctx.num_tokens
+        _put(buf.view(dt, n, H), forward(program.x.view(dt, n, H), ctx), dt)
+    program.python(call, type(part).__name__)
+    program.pending = value
 
 
 # -------------------------------------------------------------------- registry

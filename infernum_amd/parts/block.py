@@ -24,12 +24,13 @@ class PreNormBlock(Block):
         n = self.feed_forward_norm.forward(h, a)
         return self.feed_forward.forward(n, ctx)
 
-    def native(self, program, view: CacheView) -> bool:
-        if type(self) is not PreNormBlock or self.extra or None in (self.feed_forward, self.mixer_norm,
-                                                                    self.feed_forward_norm):
-            return False
-        return (self.mixer_norm.native(program, None) and self.mixer.native(program, view)
-                and self.feed_forward_norm.native(program, None) and self.feed_forward.native(program, None))
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not PreNormBlock.forward:
+            return super().native(program, view)
+        self.mixer_norm.native(program, None)
+        self.mixer.native(program, view)
+        self.feed_forward_norm.native(program, None)
+        self.feed_forward.native(program, None)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -15,7 +15,7 @@ import torch
 
 from ..kernels import api as K
 from .base import Embedding, Head, Runtime, StepContext, WeightSpec, register_part
-from .linear import linear
+from .linear import emit_linear, linear
 
 
 class TokenEmbedding(Embedding):
@@ -36,8 +36,13 @@ class TokenEmbedding(Embedding):
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
         return K.embed(self.table, ctx.token_ids, h)
 
-    def native(self, program, view) -> bool:
-        return type(self) is TokenEmbedding       # the program reads ``table`` itself
+    def native(self, program, view=None) -> None:
+        if type(self).forward is not TokenEmbedding.forward:
+            return super().native(program, view)
+        from ..engine.program import STREAM
+        program.op("core", "ia_embed", [self.table, K.DTYPE_CODE[self.table.dtype], program.token_ids, program.h,
+                                        program.N, self.hidden_size, self.vocab_size, STREAM])
+        program.pending = None
 
 
 class LinearHead(Head):
@@ -59,11 +64,10 @@ class LinearHead(Head):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
 
-    def native(self, program, view) -> bool:
-        if type(self) is not LinearHead:
-            return False
-        program.set_head(self.weight)
-        return True
+    def native(self, program, view=None) -> None:
+        if type(self).forward is not LinearHead.forward:
+            return super().native(program, view)
+        emit_linear(program, program.x, program.R, self.weight, torch.float32, None, False, program.logits, "head")
 
 
 register_part("embedding", "token", TokenEmbedding)

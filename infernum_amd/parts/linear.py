@@ -5,17 +5,19 @@ is what a product that streams the weight once wants); the reference transposes
 them on the host instead (infernum-cuda/src/inner/weights/generic_impl.rs:107-131)
 and calls cuBLAS (infernum-cuda/src/inner/cuda/ops/matmul.rs:68-117).
 
+Which kernel a product goes to is decided in ONE place, :func:`plan`: a short list of routes, each for some
+blocks of sixteen rows.  :func:`linear` runs the route of the rows at hand; :func:`emit_linear` writes every
+route into a step's program with its condition, so both make the same launches.
+
 fp32: the hand-written fp32 kernel, always (no reduced-precision matrix mode).
-bf16: up to 128 rows the hand-written MFMA kernel that streams the weight once or the library's
-product, whichever was measured faster for the weight's shape (up to 16 rows always the former; without a
-measurement up to 64 rows the former, to 128 for weights that are not wide); above that the library product (hipBLASLt, called directly with its choice of
-an algorithm kept per shape), as the reference uses its library there; an fp32
-result of many rows comes 128 rows at a time from the hand-written kernel.
-``set_prefill_gemm("mfma")`` (or INFERNUM_PREFILL_GEMM=mfma in the environment)
-sends the many-row bf16 products to the hand-written LDS-tiled MFMA kernel
-instead, where it takes the size (K in steps of 64); it is correct at every size
-but slower than the library so far, hence not the default.  ``"torch"`` sends
-them to the same library through ``torch.mm``, which costs more on the host.
+bf16: up to 128 rows the hand-written MFMA kernel that streams the weight once, or the library's product
+(hipBLASLt, called directly with its choice of an algorithm kept per shape) where that is known to be faster for
+the weight's shape (:data:`KNOWN_ROUTES`, a table that is part of the source, so that two runs of one model make
+the same launches; ``INFERNUM_GEMM_ROUTE=measured`` times both when a model loads instead, ``static`` keeps to
+the rule of sizes); above 128 rows the library, as the reference uses its library there; an fp32 result of many
+rows comes 128 rows at a time from the hand-written kernel.  ``set_prefill_gemm("mfma")`` (or
+INFERNUM_PREFILL_GEMM=mfma) sends the many-row bf16 products to the hand-written LDS-tiled MFMA kernel instead,
+where it takes the size (K in steps of 64).
 
 ``epilogue="swiglu"`` returns silu(y[:, :N/2]) * y[:, N/2:]; the decode kernel
 does it while it joins its partial sums, the other paths in a kernel of its own.
@@ -25,35 +27,50 @@ does it while it joins its partial sums, the other paths in a kernel of its own.
 from __future__ import annotations
 
 import os
-from typing import Optional, Union
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Tuple, Union
 
 import torch
 
 from ..kernels import api as K
 from ..kernels.api import SplitSum
 
+ALL_BLOCKS = 0x1FF          # bit b < 8: 16 b + 1 .. 16 b + 16 rows; bit 8: more than 128 rows
+_UP_TO_128 = 0xFF
 
-# The weight-streaming kernel takes up to 128 rows.  Up to 64 rows it is the faster one for every weight; from 65
+# The weight-streaming kernel takes up to 128 rows.  Up to 64 rows it is the faster one for most weights; from 65
 # to 128 rows for weights of fewer than 16,384 rows (8B shapes at 128 rows: 23 against 25 us for QKV, 15 against
 # 25 for the output projection, 38 against 75 for down), while the library is ahead on wider ones (gate+up 60
-# against 76 us).
+# against 76 us).  This rule stands for shapes that the table below does not hold.
 SKINNY_ROWS_ANY_WIDTH = 64
 SKINNY_WIDE = 16384
 
-# Which of the two the rows from 17 to 128 really go to is measured, once per shape of a weight and use
-# (``measure_route``): the rule above stands where nothing was measured.  The library's kernels are ahead for
-# some shapes already at 32 rows (Llama-2-13B's QKV and gate+up products at 64 rows: 35 against 52 and 61 against
-# 82 us) and behind for others (the 8B shape's down projection: 38 against 34), and no rule of sizes tells which.
-ROUTES = ("measured", "static")
-_route = os.environ.get("INFERNUM_GEMM_ROUTE", "measured")
+# (N, K, epilogue, keep_split) of a weight and its use -> the blocks of sixteen rows (bit b: 16 b + 1 .. 16 b + 16)
+# that go to the library, for 17 to 128 rows.  Measured with ``measure_route`` on an MI355X, three times over, a
+# bit kept where most runs agreed; the shapes are those of the Llama 1B, 8B, 13B and 70B layers.  The library's
+# kernels are ahead for some shapes already at 32 rows and behind for others at 128, and no rule of sizes tells.
+KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
+    (3072, 2048, None, True): 0, (2048, 2048, None, True): 0, (16384, 2048, "swiglu", False): 0b11110010,
+    (2048, 8192, None, True): 0,
+    (6144, 4096, None, True): 0, (4096, 4096, None, True): 0, (28672, 4096, "swiglu", False): 0b11110000,
+    (4096, 14336, None, True): 0,
+    (15360, 5120, None, True): 0b11111110, (5120, 5120, None, True): 0b01010010,
+    (27648, 5120, "swiglu", False): 0b11101010, (5120, 13824, None, True): 0b01001110,
+    (10240, 8192, None, True): 0b11101110, (8192, 8192, None, True): 0b01011110,
+    (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
+}
+
+ROUTES = ("table", "measured", "static")
+_route = os.environ.get("INFERNUM_GEMM_ROUTE", "table")
 if _route not in ROUTES:
     raise ValueError(f"INFERNUM_GEMM_ROUTE={_route!r}: one of {ROUTES}")
-_library_rows: dict = {}         # (N, K, epilogue, keep_split) -> bit b set: 16 b + 1 .. 16 b + 16 rows go to the library
+_measured: Dict[Tuple[int, int, Optional[str], bool], int] = {}
 
 
 def set_gemm_route(name: str) -> str:
-    """"measured": engines made from now on time both products for their weights' shapes; "static": the rule
-    of sizes.  Returns the previous choice."""
+    """"table": the routes that are part of the source, then the rule of sizes; "measured": parts loaded from now
+    on time both products for their weights' shapes (once a process); "static": the rule of sizes alone.  Engines
+    that are built already keep the launches they were built with.  Returns the previous choice."""
     global _route
     if name not in ROUTES:
         raise ValueError(f"gemm route {name!r}: one of {ROUTES}")
@@ -61,20 +78,24 @@ def set_gemm_route(name: str) -> str:
     return previous
 
 
+def gemm_routes() -> Dict[str, Any]:
+    """What decides the routes now, for a benchmark's record: the mode and, when measured, the outcomes."""
+    return {"route": _route, "measured": {f"{n}x{k}{'+' + e if e else ''}{'/split' if s else ''}": m
+                                          for (n, k, e, s), m in sorted(_measured.items(), key=str)}}
+
+
 def library_rows(N: int, K_: int, epilogue: Optional[str], keep_split: bool) -> int:
-    """The measured choice for a weight [N, K_] in this use as a mask over blocks of 16 rows (bit b: 16 b + 1 to
-    16 b + 16 rows go to the library), or -1 where nothing was measured."""
-    return _library_rows.get((N, K_, epilogue, bool(keep_split)), -1) if _route == "measured" else -1
-
-
-def _skinny_rows(M: int, N: int, Kdim: int, out_dtype: torch.dtype, epilogue: Optional[str], keep_split: bool) -> bool:
-    """Whether a bf16 product of M rows goes to the weight-streaming kernel (sizes it takes assumed)."""
-    if out_dtype != torch.bfloat16:
-        return True
-    mask = library_rows(N, Kdim, epilogue, keep_split)
-    if mask >= 0:
-        return not (mask >> ((M - 1) // 16)) & 1
-    return M <= SKINNY_ROWS_ANY_WIDTH or N < SKINNY_WIDE
+    """The blocks of sixteen rows (bit b: 16 b + 1 to 16 b + 16, b = 1 .. 7) of a bf16 product with this weight
+    and use that go to the library rather than to the weight-streaming kernel."""
+    key = (N, K_, epilogue, bool(keep_split))
+    mask = -1
+    if _route == "measured":
+        mask = _measured.get(key, -1)
+    elif _route == "table":
+        mask = KNOWN_ROUTES.get(key, -1)
+    if mask < 0:
+        mask = 0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1)
+    return mask & 0xFE             # up to 16 rows the weight-streaming kernel, always
 
 
 def measure_routes_for(rt, uses) -> None:
@@ -93,8 +114,8 @@ def measure_route(w: torch.Tensor, epilogue: Optional[str], keep_split: bool, ma
     Once per shape and use in a process.  Returns the mask of :func:`library_rows`."""
     N, Kdim = w.shape
     key = (N, Kdim, epilogue, bool(keep_split))
-    if key in _library_rows:
-        return _library_rows[key]
+    if key in _measured:
+        return _measured[key]
     mask = 0
     if w.is_cuda and w.dtype == torch.bfloat16 and K.gemm_skinny_supported(1, N, Kdim) and _prefill_gemm == "library":
         def timed(fn) -> float:
@@ -126,20 +147,19 @@ def measure_route(w: torch.Tensor, epilogue: Optional[str], keep_split: bool, ma
                 if timed(library) < margin * timed(own):
                     mask |= 1 << block
         except K.KernelError:
-            mask = 0                                  # a shape that one of them refuses: the rule of sizes
-            _library_rows[key] = -1
-            return -1
-    _library_rows[key] = mask
+            mask = -1                                 # a shape that one of them refuses: the rule of sizes
+    _measured[key] = mask
     return mask
 
-PREFILL_GEMMS = ("library", "mfma", "torch")
+
+PREFILL_GEMMS = ("library", "mfma")
 _prefill_gemm = os.environ.get("INFERNUM_PREFILL_GEMM", "library")
 if _prefill_gemm not in PREFILL_GEMMS:
     raise ValueError(f"INFERNUM_PREFILL_GEMM={_prefill_gemm!r}: one of {PREFILL_GEMMS}")
 
 
 def set_prefill_gemm(name: str) -> str:
-    """Chooses the bf16 product for more than 64 rows; returns the previous choice."""
+    """Chooses the bf16 product for more than 128 rows; returns the previous choice."""
     global _prefill_gemm
     if name not in PREFILL_GEMMS:
         raise ValueError(f"prefill gemm {name!r}: one of {PREFILL_GEMMS}")
@@ -151,6 +171,78 @@ def prefill_gemm() -> str:
     return _prefill_gemm
 
 
+# ------------------------------------------------------------------------------ the one place that decides
+@dataclass(frozen=True)
+class Route:
+    """Rows (a mask over blocks of sixteen, see ALL_BLOCKS) -> the kernel that takes them.  Kinds: "generic"
+    (fp32 multiply-adds in a fixed order), "skinny" (the weight-streaming kernel, its parts joined, the
+    activation in its epilogue), "skinny_split" (the same with its partial sums left for the next kernel),
+    "skinny_rows" (128 rows at a time), "library" (hipBLASLt; ``fallback`` names the kernel for a shape it
+    refuses), "mfma" (the LDS-tiled kernel)."""
+
+    blocks: int
+    kind: str
+    fallback: Optional[str] = None
+
+
+_MANY_ROWS = 65536         # the LDS-tiled kernel addresses rows with 32 bits: its fitness is judged at this many
+
+
+def plan(N: int, Kdim: int, dtype: torch.dtype, out_dtype: torch.dtype, epilogue: Optional[str], keep_split: bool,
+         kernels: str = "auto") -> List[Route]:
+    """The routes of x [M, Kdim] (``dtype``) times a weight [N, Kdim] for every M >= 1, in the order they are tried."""
+    if epilogue not in (None, "swiglu"):
+        raise K.KernelError(f"linear: unknown epilogue {epilogue!r}")
+    if dtype not in (torch.float32, torch.bfloat16):
+        raise K.KernelError(f"linear: dtype {dtype} is not supported")
+    if kernels == "generic" or dtype == torch.float32:
+        return [Route(ALL_BLOCKS, "generic")]
+    tiled_fits = K.gemm_mfma_supported(_MANY_ROWS, N, Kdim)
+    many = Route(0, "mfma") if (_prefill_gemm == "mfma" and tiled_fits) else \
+        Route(0, "library", fallback="mfma" if tiled_fits else "generic")
+    if not K.gemm_skinny_supported(1, N, Kdim):
+        return [Route(ALL_BLOCKS, many.kind, many.fallback)] if out_dtype == torch.bfloat16 else [Route(ALL_BLOCKS, "generic")]
+    own = "skinny_split" if (keep_split and epilogue is None and K.gemm_skinny_splits(N, Kdim) > 1) else "skinny"
+    if out_dtype != torch.bfloat16:
+        if epilogue is not None:
+            raise K.KernelError("linear: an fp32 result from bf16 operands has no activation here")
+        return [Route(_UP_TO_128, own), Route(ALL_BLOCKS & ~_UP_TO_128, "skinny_rows")]
+    to_library = library_rows(N, Kdim, epilogue, keep_split) if _prefill_gemm == "library" else \
+        (0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1))
+    routes = [Route(_UP_TO_128 & ~to_library, own),
+              Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback)]
+    return [r for r in routes if r.blocks]
+
+
+def route_of(routes: List[Route], M: int) -> Route:
+    bit = 1 << min((M - 1) // 16, 8)
+    for r in routes:
+        if r.blocks & bit:
+            return r
+    raise K.KernelError(f"linear: no route for {M} rows")
+
+
+def _run(kind: str, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, epilogue: Optional[str],
+         fallback: Optional[str] = None):
+    M, N = x.shape[0], w.shape[0]
+    if kind == "skinny":
+        return K.gemm_skinny(x, w, epilogue=epilogue, out_dtype=out_dtype), True
+    if kind == "skinny_split":
+        return K.gemm_skinny(x, w, keep_split=True), True
+    if kind == "skinny_rows":
+        return K.gemm_skinny_rows(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device)), True
+    if kind == "generic":
+        return K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device)), False
+    if kind == "mfma":
+        return K.gemm_mfma(x, w), False
+    if kind == "library":
+        try:
+            return K.gemm_library(x, w), False
+        except K.KernelUnsupported:             # the library has no algorithm for this shape
+            return _run(fallback or "generic", x, w, out_dtype, None)
+    raise K.KernelError(f"linear: unknown route {kind!r}")
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            epilogue: Optional[str] = None, keep_split: bool = False,
            kernels: str = "auto") -> Union[torch.Tensor, SplitSum]:
@@ -158,41 +250,79 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     M, Kdim = x.shape
     N = w.shape[0]
     out_dtype = out_dtype or x.dtype
-    n_out = N // 2 if epilogue == "swiglu" else N
     if M == 0:
-        return torch.empty((0, n_out), dtype=out_dtype, device=x.device)
-    if kernels == "generic":
-        if x.dtype not in (torch.float32, torch.bfloat16):
-            raise K.KernelError(f"linear: dtype {x.dtype} is not supported")
-        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
-    elif x.dtype == torch.bfloat16 and K.gemm_skinny_supported(M, N, Kdim) and x.is_contiguous() and \
-            _skinny_rows(M, N, Kdim, out_dtype, epilogue, keep_split):
-        return K.gemm_skinny(x, w, epilogue=epilogue, keep_split=keep_split, out_dtype=out_dtype)
-    elif x.dtype == torch.float32:
-        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
-    elif x.dtype != torch.bfloat16:
-        raise K.KernelError(f"linear: dtype {x.dtype} is not supported")
-    elif out_dtype == torch.bfloat16:
-        if _prefill_gemm == "mfma" and x.is_contiguous() and K.gemm_mfma_supported(M, N, Kdim):
-            y = K.gemm_mfma(x, w)
-        elif _prefill_gemm == "torch" or not x.is_contiguous():
-            y = torch.mm(x, w.t())                  # library product, fp32 accumulation
-        else:
-            try:
-                y = K.gemm_library(x, w)
-            except K.KernelUnsupported:             # the library has no algorithm for this shape
-                y = K.gemm_mfma(x, w) if K.gemm_mfma_supported(M, N, Kdim) else \
-                    K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
-    elif K.gemm_skinny_supported(1, N, Kdim) and x.is_contiguous():
-        # fp32 result from bf16 operands, many rows: 128 rows at a time through the skinny kernel
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        for m0 in range(0, M, K.SKINNY_MAX_M):
-            m1 = min(M, m0 + K.SKINNY_MAX_M)
-            K.gemm_skinny(x[m0:m1], w, out=y[m0:m1])
-    else:
-        y = K.gemm_generic(x, w, torch.empty((M, N), dtype=out_dtype, device=x.device))
-    if epilogue == "swiglu":
-        return K.swiglu(y, torch.empty((M, n_out), dtype=y.dtype, device=y.device))
-    if epilogue is not None:
-        raise K.KernelError(f"linear: unknown epilogue {epilogue!r}")
+        return torch.empty((0, N // 2 if epilogue == "swiglu" else N), dtype=out_dtype, device=x.device)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    route = route_of(plan(N, Kdim, x.dtype, out_dtype, epilogue, keep_split, kernels), M)
+    y, activated = _run(route.kind, x, w, out_dtype, epilogue, route.fallback)
+    if epilogue == "swiglu" and not activated:
+        return K.swiglu(y, torch.empty((M, N // 2), dtype=y.dtype, device=y.device))
     return y
+
+
+# ------------------------------------------------------------------- the same routes, written into a program
+def emit_linear(program, x: Any, M: Any, w: torch.Tensor, out_dtype: torch.dtype, epilogue: Optional[str],
+                keep_split: bool, out: Any, key: str, when: Any = None):
+    """Writes the launches of :func:`linear` for ``x`` (an address: a Buffer, a tensor, a StepPtr) of ``M`` rows
+    (a number of the step) into ``program``, one route after the other, each for its rows.  ``out``: a key (the
+    result gets a buffer of that name) or a StepPtr (the step's logits); ``key`` names the scratch memory.
+    Returns the ``Value`` that stands for the result."""
+    from ..engine import program as P
+    rt = program.rt
+    when = P.ALWAYS if when is None else when
+    N, Kdim = w.shape
+    T = program.T
+    routes = plan(N, Kdim, rt.dtype, out_dtype, epilogue, keep_split, rt.kernels)
+    n_out = N // 2 if epilogue == "swiglu" else N
+    out_bytes = 4 if out_dtype == torch.float32 else 2
+    splits = K.gemm_skinny_splits(N, Kdim) if any(r.kind.startswith("skinny") for r in routes) else 1
+    small = min(T, K.SKINNY_MAX_M)
+    if isinstance(out, str):
+        size = T * n_out * out_bytes
+        if any(r.kind == "skinny_split" for r in routes):
+            size = max(size, splits * small * N * 4)
+        out = program.buffer(out, size)
+    code, in_code = K.DTYPE_CODE[out_dtype], K.DTYPE_CODE[rt.dtype]
+    program.keep(w)
+    alts = []
+    for r in routes:
+        g = when & P.Guard.blocks(M, r.blocks)
+        if g.never:
+            continue
+        if r.kind == "skinny_split":
+            program.op("core", "ia_gemm_skinny", [x, w, None, 0, M, N, Kdim, 0, out, M * (splits * N), P.STREAM], g)
+            alts.append(P.Alt(g, out, splits, torch.float32))
+            continue
+        if r.kind == "skinny":
+            ws = program.buffer(key + ".parts", splits * small * N * 4) if splits > 1 else None
+            program.op("core", "ia_gemm_skinny", [x, w, out, code, M, N, Kdim, K.EPILOGUE[epilogue], ws,
+                                                   M * (splits * N) if splits > 1 else 0, P.STREAM], g)
+        elif r.kind == "skinny_rows":
+            ws = program.buffer(key + ".parts", splits * small * N * 4) if splits > 1 else None
+            program.op("core", "ia_gemm_skinny_rows", [x, w, out, code, M, N, Kdim, ws,
+                                                        splits * small * N if splits > 1 else 0, P.STREAM], g)
+        else:
+            # a product that leaves the whole matrix: into scratch first when an activation follows
+            y = program.buffer(key + ".product", T * N * out_bytes) if epilogue == "swiglu" else out
+            _emit_whole(program, r.kind, x, w, y, M, N, Kdim, in_code, code, g, False)
+            if r.fallback:
+                _emit_whole(program, r.fallback, x, w, y, M, N, Kdim, in_code, code, g, True)
+            if epilogue == "swiglu":
+                program.op("core", "ia_swiglu", [y, out, code, M, N // 2, P.STREAM], g)
+        alts.append(P.Alt(g, out, 0, out_dtype))
+    return P.Value(n_out, alts)
+
+
+def _emit_whole(program, kind, x, w, y, M, N, Kdim, in_code, out_code, when, if_unsupported) -> None:
+    from ..engine import program as P
+    if kind == "generic":
+        program.op("core", "ia_gemm_generic", [x, w, y, in_code, out_code, M, N, Kdim, Kdim, Kdim, N, P.STREAM],
+                   when, if_unsupported)
+    elif kind == "mfma":
+        program.op("core", "ia_gemm_mfma", [x, w, y, M, N, Kdim, 0, P.STREAM], when, if_unsupported)
+    elif kind == "library":
+        ws = K.library_workspace(program.rt.device)
+        program.op("blaslt", "ia_gemm_lt", [x, w, y, M, N, Kdim, in_code, ws, ws.numel(), P.STREAM], when, if_unsupported)
+    else:
+        raise K.KernelError(f"linear: {kind!r} does not leave a whole matrix")

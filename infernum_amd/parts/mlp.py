@@ -10,7 +10,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import FeedForward, Runtime, StepContext, WeightSpec, register_part
-from .linear import linear, measure_routes_for
+from .linear import emit_linear, linear, measure_routes_for
 
 
 class SwiGLUFeedForward(FeedForward):
@@ -40,12 +40,13 @@ class SwiGLUFeedForward(FeedForward):
         act = linear(x, self.w_gate_up, epilogue="swiglu", kernels=self.rt.kernels)
         return linear(act, self.w_down, keep_split=True, kernels=self.rt.kernels)
 
-
-    def native(self, program, view) -> bool:
-        if type(self) is not SwiGLUFeedForward:
-            return False
-        program.add_swiglu(self.w_gate_up, self.w_down)
-        return True
+    def native(self, program, view=None) -> None:
+        if type(self).forward is not SwiGLUFeedForward.forward:
+            return super().native(program, view)
+        dt = self.rt.dtype
+        act = emit_linear(program, program.x, program.N, self.w_gate_up, dt, "swiglu", False, "swiglu.act", "swiglu.gate_up")
+        program.pending = emit_linear(program, act.tensor(), program.N, self.w_down, dt, None, True, "swiglu.out",
+                                      "swiglu.down")
 
 
 register_part("feed_forward", "swiglu", SwiGLUFeedForward)

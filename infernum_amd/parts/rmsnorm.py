@@ -39,11 +39,24 @@ class RMSNorm(Norm):
         return K.add_rmsnorm(h, delta, self.weight, self.eps, out, rows)
 
 
-    def native(self, program, view, final: bool = False) -> bool:
-        if type(self) is not RMSNorm:
-            return False
-        program.add_norm(self.weight, self.eps, final=final)
-        return True
+    def native(self, program, view=None, rows: bool = False) -> None:
+        """One launch per form the pending delta can have (none, a tensor, partial sums of a split product)."""
+        if type(self).forward is not RMSNorm.forward:
+            return super().native(program, view, rows)          # a subclass that computes something else
+        from ..engine.program import ALWAYS, STREAM, Guard
+        base = Guard.between(program.R, 1) if rows else ALWAYS
+        for alt in (program.pending.alts if program.pending is not None else [None]):
+            delta, code, splits, when = None, program.act_code, 1, base
+            if alt is not None:
+                if not alt.splits and alt.dtype != self.rt.dtype:
+                    raise K.KernelError("add_rmsnorm: the delta must have the activations' dtype")
+                delta, when = alt.where, base & alt.when
+                code, splits = (K.DTYPE_CODE[torch.float32], alt.splits) if alt.splits else (program.act_code, 1)
+            program.op("core", "ia_add_rmsnorm",
+                       [program.h, delta, code, splits, program.N, program.act_code, self.weight,
+                        K.DTYPE_CODE[self.weight.dtype], program.x, program.logit_rows if rows else None,
+                        program.R if rows else program.N, self.size, float(self.eps), STREAM], when)
+        program.pending = None
 
 
 register_part("norm", "rmsnorm", RMSNorm)

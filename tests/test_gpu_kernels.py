@@ -413,20 +413,53 @@ def test_gemm_library_refuses_what_it_cannot_do():
         api.gemm_library(_rand(80, 128)[:, :64], _rand(32, 64))                                    # not contiguous
 
 
-def test_linear_by_the_library_directly_and_through_torch():
+def test_linear_by_the_library_and_by_the_tiled_kernel():
     import importlib
     L = importlib.import_module("infernum_amd.parts.linear")
     x, w = _rand(200, 256, dtype=torch.bfloat16, seed=3), _rand(330, 256, dtype=torch.bfloat16, scale=0.1, seed=4)
     assert L.prefill_gemm() == "library"
+    assert [r.kind for r in L.plan(330, 256, torch.bfloat16, torch.bfloat16, None, False)] == ["skinny", "library"]
     direct = L.linear(x, w)
-    previous = L.set_prefill_gemm("torch")
+    previous = L.set_prefill_gemm("mfma")
     try:
-        through = L.linear(x, w)
+        assert [r.kind for r in L.plan(330, 256, torch.bfloat16, torch.bfloat16, None, False)] == ["skinny", "mfma"]
+        tiled = L.linear(x, w)
     finally:
         L.set_prefill_gemm(previous)
     want = x.double() @ w.double().t()
     bound = 2e-5 * 16 * 0.1 + 2.0 ** -8 * want.abs()
-    assert bool(((direct.double() - want).abs() <= bound).all()) and bool(((through.double() - want).abs() <= bound).all())
+    assert bool(((direct.double() - want).abs() <= bound).all()) and bool(((tiled.double() - want).abs() <= bound).all())
+    with pytest.raises(ValueError):
+        L.set_prefill_gemm("torch")
+
+
+def test_linear_fp32_result_of_many_rows_from_bf16_operands():
+    """The head of a step that wants many rows: 128 rows at a time through the weight-streaming kernel."""
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    x, w = _rand(300, 96, dtype=torch.bfloat16, seed=5), _rand(1000, 96, dtype=torch.bfloat16, scale=0.1, seed=6)
+    assert [r.kind for r in L.plan(1000, 96, torch.bfloat16, torch.float32, None, False)] == ["skinny", "skinny_rows"]
+    y = L.linear(x, w, out_dtype=torch.float32)
+    want = x.double() @ w.double().t()
+    assert y.dtype == torch.float32 and (y.double() - want).abs().max().item() <= 2e-5 * 10 * 0.1
+    for m in (1, 128, 129, 256, 257):
+        assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
+
+
+def test_known_routes_send_rows_to_the_library_where_the_table_says():
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    key = (15360, 5120, None, True)
+    assert L.KNOWN_ROUTES[key] == 0b11111110
+    kinds = lambda: {m: L.route_of(L.plan(15360, 5120, torch.bfloat16, torch.bfloat16, None, True), m).kind
+                     for m in (1, 16, 17, 64, 128, 129)}
+    assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "library", 64: "library", 128: "library", 129: "library"}
+    previous = L.set_gemm_route("static")
+    try:
+        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "skinny_split", 64: "skinny_split",
+                           128: "skinny_split", 129: "library"}
+    finally:
+        L.set_gemm_route(previous)
 
 
 def test_rope_from_partial_sums():

@@ -174,6 +174,14 @@ def test_toy_model_is_registered_built_loaded_and_stepped(toy, dtype):
         assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
         eng.cache.check()
         assert eng.cache.slots.num_free == 4 and all(g.allocator.num_free == 48 for g in eng.cache.groups)
+    # the step ran as one program: the stock parts' launches made by the host library, the mixer of this file
+    # called back in its place among them; the parts' own forward, call by call from Python, gives the same bits
+    assert eng.program is not None and eng.program.num_ops > 30
+    twin = Engine.from_pretrained(d, dtype=dtype, executor="parts",
+                                  cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4))
+    assert twin.program is None
+    a, b = TT.run_steps(eng, TT.trace_portions(reqs)), TT.run_steps(twin, TT.trace_portions(reqs))
+    assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
 
 
 def test_state_slot_is_zeroed_when_taken_again(toy):
@@ -583,7 +591,7 @@ def test_a_part_between_projection_and_rotation(tmp_path, dtype):
     assert "l.0.attn.q_norm.weight" in w and "l.1.attn.k_norm.weight" in w      # the transform's tensors, by name
     eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=8, num_pages=40, num_state_slots=4,
                                                                           poison_freed_pages=True))
-    assert eng.program is None and not eng.use_graphs           # the model's own part: through the parts, unrecorded
+    assert eng.program is not None and not eng.use_graphs       # the model's own part is called back from the program; unrecorded
     reqs = TT.make_requests(cfg.vocab_size, (29, 7, 44, 18), seed=5)
     ref = {r: plain_forward4(cfg, w, t) for r, t in reqs.items()}
     tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
@@ -745,7 +753,7 @@ def test_a_norm_an_embedding_and_a_head_of_the_models_own(tmp_path, dtype):
     assert {"emb.positions", "fn.bias", "l.1.n2.bias", "head.weight"} <= set(w)
     eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4,
                                                                           poison_freed_pages=True))
-    assert eng.program is None and not eng.use_graphs           # parts of the model's own: through the parts, unrecorded
+    assert eng.program is not None and not eng.use_graphs       # the model's own parts are called back from the program; unrecorded
     reqs = TT.make_requests(cfg.vocab_size, (37, 5, 52, 20), seed=8)
     ref = {r: plain_forward5(cfg, w, t) for r, t in reqs.items()}
     assert max(float(v.abs().max()) for v in ref.values()) <= cfg.cap
