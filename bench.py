@@ -199,7 +199,10 @@ LLAMA_1B = dict(
 
 def serve(a) -> int:
     """Continuous batching of 128 requests on the Llama-3.2-1B shape: prompts of 64 to 2,048 tokens, 32 to 512
-    new tokens each (uniform, seeded), greedy, context 4,096.  Prints one JSON line of its own."""
+    new tokens each (uniform, seeded), greedy, context 4,096.  Prints one JSON line of its own: tokens a second
+    (generated, of prompts, together) and the run's place against the roofline (portions of prompts and decoded
+    tokens share steps, so they are priced together, step by step; the reference prices prefill and decode apart,
+    performance.md:9-41, infernum-examples/examples/bench.rs:1031-1110, where they run apart)."""
     import random
     import torch
     from infernum_amd import BatchConfig, CacheConfig, Engine, GenerateOptions, LlamaConfig, Runtime
@@ -220,10 +223,34 @@ def serve(a) -> int:
     t0 = time.perf_counter()
     seqs = [rt.submit(p, GenerateOptions(max_new_tokens=n)) for p, n in jobs]
     steps = set_back = 0
+    # what every step has to do at the least: read every weight once and the keys and values of its requests; two
+    # flops per weight and token (the head on the rows that want logits), four per query, key and head dimension
+    per_layers, head = matmul_params(cfg)
+    kv_bytes_per_token = 2 * cfg.num_kv_heads * cfg.head_dim * cfg.num_hidden_layers * 2
+    attn_flops_per_pair = 4.0 * cfg.num_attention_heads * cfg.head_dim * cfg.num_hidden_layers
+    total_bytes = total_flops = bound_s = 0.0
+    cache = engine.cache
     while not rt.scheduler.is_idle():
         plan = rt.step()
         steps += 1
         set_back += len(plan.set_back)
+        if plan.is_empty():
+            continue
+        keys = pairs = 0.0
+        for t in plan.decode:
+            keys += t.seq.num_tokens
+            pairs += t.seq.num_tokens
+        for t in plan.prefill:
+            n = len(t.token_ids)
+            after = cache.num_tokens(t.seq.id) if cache.has(t.seq.id) else n
+            keys += after
+            pairs += n * after - n * (n - 1) / 2.0
+        rows = len(plan.decode) + sum(1 for t in plan.prefill if t.completes)
+        step_bytes = (per_layers + head) * 2.0 + keys * kv_bytes_per_token
+        step_flops = 2.0 * per_layers * plan.num_tokens + 2.0 * head * rows + attn_flops_per_pair * pairs
+        total_bytes += step_bytes
+        total_flops += step_flops
+        bound_s += max(step_bytes / (HBM_PEAK_GBS * 1e9), step_flops / (PEAK_TFLOPS["bf16"] * 1e12))
     sync()
     dt = time.perf_counter() - t0
     gen = sum(len(s.generated_ids) for s in seqs)
@@ -231,7 +258,14 @@ def serve(a) -> int:
     assert all(s.error is None and len(s.generated_ids) == n for s, (_, n) in zip(seqs, jobs))
     print(json.dumps({"metric": "continuous batching, Llama-3.2-1B shape", "requests": len(jobs),
                       "generated_tokens": gen, "prompt_tokens": prompt, "seconds": round(dt, 3),
-                      "generated_tok_per_s": round(gen / dt, 1), "all_tok_per_s": round((gen + prompt) / dt, 1),
+                      "generated_tok_per_s": round(gen / dt, 1), "prompt_tok_per_s": round(prompt / dt, 1),
+                      "all_tok_per_s": round((gen + prompt) / dt, 1),
+                      "roofline": {"bound": "per step the larger of bytes / HBM peak and flops / bf16 peak, summed",
+                                   "bound_seconds": round(bound_s, 4), "frac": round(bound_s / dt, 4),
+                                   "gb_read_at_least": round(total_bytes / 1e9, 1),
+                                   "hbm_frac": round(total_bytes / dt / (HBM_PEAK_GBS * 1e9), 4),
+                                   "tflop": round(total_flops / 1e12, 1),
+                                   "flops_frac": round(total_flops / dt / (PEAK_TFLOPS["bf16"] * 1e12), 4)},
                       "steps": steps, "ms_per_step": round(dt / steps * 1e3, 3), "set_back": set_back,
                       "graph_replays": engine.graph_replays, "max_batch": bc.max_batch_size,
                       "chunk": bc.max_prefill_tokens, "num_blocks": bc.num_blocks, "dtype": "bf16",
@@ -345,6 +379,8 @@ def main() -> int:
         print(json.dumps({"prefill": time_prefill(engine, cfg, a.dtype, repeats=max(3, a.warmup))}))
         return 0
 
+    import importlib
+    gemm_route = importlib.import_module("infernum_amd.parts.linear").gemm_routes()["route"]
     # ---- the timed K steps at the headline batch ---------------------------------
     dt, ctx_mid = time_decode(engine, a.batch, a.steps, a.warmup, a.prompt_len)
     ms_per_step = dt / a.steps * 1e3
@@ -359,7 +395,7 @@ def main() -> int:
             "hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads, "num_kv_heads": cfg.num_kv_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LEN, "page_size": PAGE_SIZE,
-            "parallelism": "none", "sampling": "greedy",
+            "parallelism": "none", "sampling": "greedy", "gemm_route": gemm_route,
             "rope": "llama3(8,1,4,8192) theta 5e5" if a.shape == "8b" else "theta 1e4",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -58,9 +58,9 @@ class Engine:
         self.model = model
         self.rt: Runtime = model.rt
         self.spec = model.spec
-        self.cache = CacheManager(model.cache_needs(), [e.cache_of for e in model.spec.schedule], cache_config,
+        self.cache = CacheManager(model.cache_needs(), model.cache_sources(), cache_config,
                                   dtype=self.rt.dtype, device=self.rt.device)
-        self.views = self.cache.views()
+        self.views = model.entry_views(self.cache.views())          # one per schedule entry
         # row tiles that parts asked for: one height is laid out with the step's arrays, further ones are
         # made when a part asks (StepContext.row_tiles)
         heights = sorted(model.step_needs().get("row_tiles", ()))

@@ -62,6 +62,9 @@ class Runtime:
         if limit is not None and batch_config.max_tokens_per_step > limit:
             raise ValueError(f"max_tokens_per_step {batch_config.max_tokens_per_step} is above the engine's {limit}")
         self.batch_config = batch_config
+        if max_seq_len is None:
+            # the model's own bound (max_position_embeddings; infernum-llama/src/config.rs:44-45, ModelConfig.max_seq_len)
+            max_seq_len = getattr(getattr(engine, "spec", None), "max_position", 0) or None
         self.scheduler = Scheduler(batch_config, max_seq_len=max_seq_len)
         if sampler is None:
             from ..sampling.sampler import Sampler
@@ -78,6 +81,7 @@ class Runtime:
                            and hasattr(self.sampler, "select_on_device") and hasattr(self.sampler, "needs_history"))
         self._inflight = None                 # (plan, tokens on the device, row of each request, download)
         self._download = None
+        self._recomputed = 0                  # requests served without the cache so far (their names)
 
     # ---- building ---------------------------------------------------------------------
     @classmethod
@@ -282,24 +286,33 @@ class Runtime:
 
     def _prepare(self, prompt: Prompt, options: Optional[GenerateOptions]):
         options = options or GenerateOptions()
+        if options.eos_token_id is None:
+            # the model's end-of-sequence token stands in for every request that names none
+            # (infernum-runtime/src/runtime.rs:127-134); ``submit`` takes the options as they are
+            eos = getattr(getattr(self.engine, "spec", None), "eos_token_id", None)
+            options = GenerateOptions(options.max_new_tokens, eos, options.sampling, options.use_kv_cache)
         if isinstance(prompt, str):
             if self.tokenizer is None:
                 raise GenerationError("a text prompt needs a tokenizer (tokenizer.json in the model folder); "
                                       "pass token ids instead")
-            ids = self.tokenizer.encode(prompt, add_bos=True)
-            if options.eos_token_id is None:
-                eos = getattr(getattr(self.engine, "spec", None), "eos_token_id", None)
-                options = GenerateOptions(options.max_new_tokens, eos, options.sampling, options.use_kv_cache)
-            return ids, options, True
+            return self.tokenizer.encode(prompt, add_bos=True), options, True
         return [int(t) for t in prompt], options, False
 
     def _generate_without_cache(self, prompt: Sequence[int], options: GenerateOptions) -> List[int]:
         """Every new token from the whole sequence, computed afresh (GenerateOptions.use_kv_cache = false)."""
         toks, out = [int(t) for t in prompt], []
         probe = SequenceState("nocache", toks, options)
+        limit = getattr(getattr(self.engine, "rt", None), "max_tokens_per_step", None) or (1 << 30)
+        self._recomputed += 1
+        name = ("recomputed", self._recomputed)         # a name that no request of the scheduler has
         for _ in range(options.max_new_tokens):
-            logits = self.engine.step([StepEntry("__no_kv_cache__", toks + out, [len(toks) + len(out) - 1])])
-            self.engine.end("__no_kv_cache__")
+            whole = toks + out
+            try:
+                for p in range(0, len(whole), limit):       # longer than a step takes: in portions
+                    part = whole[p:p + limit]
+                    logits = self.engine.step([StepEntry(name, part, [len(part) - 1] if p + limit >= len(whole) else [])])
+            finally:
+                self.engine.end(name)
             probe.generated_ids = out
             tok = self.sampler.select(logits, [self._row(probe)])[0]
             if options.eos_token_id is not None and tok == options.eos_token_id:

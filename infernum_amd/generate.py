@@ -5,7 +5,7 @@ reference's ``generate`` example (infernum-examples/examples/generate.rs:37-86):
         [-t 0.7] [-p 0.9] [-s 42] [-r 1.1] [--repetition-penalty-window 64] [--max-seq-len N]
 
 Added here: ``--prompt-ids 1,2,3`` for model folders without a tokenizer (token
-ids in, token ids out), ``--dtype bfloat16|float32``, ``--kernels auto|generic``, and the cache's settings
+ids in, token ids out), ``--random CONFIG.json`` (random weights from a configuration and ``--seed``), ``--dtype bfloat16|float32``, ``--kernels auto|generic``, and the cache's settings
 (``--block-size``, ``--num-blocks``, ``--max-batch``, ``--chunk``).  The model class
 is chosen by config.json's ``model_type``, as everywhere in the package.
 """
@@ -37,6 +37,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-seq-len", type=int, default=None,
                     help="longest sequence (prompt and generated tokens); default min(model max, 4096)")
     ap.add_argument("--prompt-ids", default=None, help="comma-separated token ids instead of a text prompt")
+    ap.add_argument("--random", metavar="CONFIG.json", default=None,
+                    help="no model folder: random weights made from this configuration file and --seed "
+                         "(token ids in and out: give --prompt-ids)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "f32"])
     ap.add_argument("--kernels", default="auto", choices=["auto", "generic"],
                     help="generic: the plain twins of the fast kernels for every product and the attention")
@@ -53,6 +56,21 @@ def main(argv: Optional[List[str]] = None) -> int:
     from .engine import BatchConfig, Runtime
     from .sampling import GenerateOptions, SamplingParams
 
+    scratch = None
+    if a.random is not None:
+        # a model folder of random weights (the numbers of ``bin/random_model`` from the same file and seed), made in a
+        # temporary folder and loaded like any other; -s is its seed as well as the sampler's
+        import tempfile
+        import torch
+        from . import models  # noqa: F401  (registers the architectures)
+        from .config.base import read_config_json
+        from .config.registry import config_from_dict
+        from .weights import write_random_model
+        scratch = tempfile.TemporaryDirectory(prefix="infernum_random_")
+        print(f"Random weights from: {a.random} (seed {a.seed})")
+        stored = torch.float32 if a.dtype in ("float32", "f32") else torch.bfloat16
+        write_random_model(config_from_dict(read_config_json(a.random), where=a.random), scratch.name, a.seed, stored)
+        a.model = scratch.name
     print(f"Loading model from: {a.model}")
     config = load_config(a.model)
     max_seq_len = a.max_seq_len or min(getattr(config, "max_position_embeddings", 4096), 4096)
@@ -96,6 +114,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     dt = time.perf_counter() - t0
     print()
     print(f"Generated {n} tokens in {dt:.2f}s ({n / dt if dt > 0 else 0.0:.1f} tokens/sec)")
+    if scratch is not None:
+        scratch.cleanup()
     return 0
 
 

@@ -16,6 +16,11 @@ from ..parts.base import (Block, CacheSpec, CacheView, ModelSpec, Part, PartSpec
                           WeightSpec, block_factory, make_part)
 
 
+def _needs(part: Part) -> Tuple[Optional[CacheSpec], Optional[StateSpec]]:
+    return (part.cache_spec() if hasattr(part, "cache_spec") else None,
+            part.state_spec() if hasattr(part, "state_spec") else None)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, rt: Runtime):
         self.spec = spec
@@ -50,8 +55,8 @@ class DecoderModel:
                     raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_of}, which does not run before it")
                 if self.spec.schedule[e.cache_of].cache_of is not None:
                     raise ValueError(f"schedule entry {i} reads entry {e.cache_of}, which has no cache of its own")
-                a = self.blocks[e.layer].mixer.cache_spec()
-                b = self.blocks[self.spec.schedule[e.cache_of].layer].mixer.cache_spec()
+                a = {n: _needs(p) for n, p in self.blocks[e.layer].cached_parts().items()}
+                b = {n: _needs(p) for n, p in self.blocks[self.spec.schedule[e.cache_of].layer].cached_parts().items()}
                 if a != b:
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_of}: {a} != {b}")
 
@@ -89,17 +94,36 @@ class DecoderModel:
         return out
 
     # ---- cache needs ---------------------------------------------------------
+    def _cached(self) -> List[Tuple[int, str, Part]]:
+        """(schedule entry, name, part) of every part that keeps something between steps, in the schedule's order."""
+        return [(i, name, part) for i, e in enumerate(self.spec.schedule)
+                for name, part in self.blocks[e.layer].cached_parts().items()]
+
     def cache_needs(self) -> List[Tuple[Optional[CacheSpec], Optional[StateSpec]]]:
-        """Per schedule entry: the pages and the per-request state its mixer wants
-        (None, None for an entry that reads another entry's)."""
-        needs = []
-        for e in self.spec.schedule:
-            if e.cache_of is not None:
-                needs.append((None, None))
-            else:
-                m = self.blocks[e.layer].mixer
-                needs.append((m.cache_spec(), m.state_spec()))
-        return needs
+        """Per cached part of every schedule entry (mostly one: the mixer): the pages and the per-request state it
+        wants (None, None for an entry that reads another entry's)."""
+        return [(None, None) if self.spec.schedule[i].cache_of is not None else _needs(part)
+                for i, _, part in self._cached()]
+
+    def cache_sources(self) -> List[Optional[int]]:
+        """Per cached part: the index (in ``cache_needs``) of the part whose pages and state it reads, or None for
+        its own."""
+        index = {(i, name): k for k, (i, name, _) in enumerate(self._cached())}
+        return [None if self.spec.schedule[i].cache_of is None else index[(self.spec.schedule[i].cache_of, name)]
+                for i, name, _ in self._cached()]
+
+    def entry_views(self, views: List[CacheView]) -> List[CacheView]:
+        """From the cache manager's views (one per cached part) the view of each schedule entry: the mixer's,
+        with the layer's further cached parts under their names in ``others``."""
+        per_entry: List[Dict[str, CacheView]] = [{} for _ in self.spec.schedule]
+        for (i, name, _), view in zip(self._cached(), views):
+            per_entry[i][name] = view
+        out = []
+        for named in per_entry:
+            main = named.pop("mixer", None) or CacheView()
+            main.others = named
+            out.append(main)
+        return out
 
     # ---- the step as a program ------------------------------------------------------
     def native(self, program, views: List[CacheView]) -> None:

@@ -169,13 +169,16 @@ class CacheView:
     CacheSpec payload, each [num_pages, ...] with the page's tokens along the declared axis; ``k_pages`` and
     ``v_pages`` are the "k" and "v" of them.  ``group`` indexes the step's block tables and slots;
     ``writable`` is False when the pages belong to another entry.  ``state`` is the entry's
-    [num_slots, *shape] tensor when the mixer declared a StateSpec.
+    [num_slots, *shape] tensor when the mixer declared a StateSpec.  ``others``: the views of the layer's
+    further cached parts, under the names of ``Block.cached_parts`` (a layer with an attention and a mixer
+    with state side by side has two).
     """
 
     group: int = -1
     pages: Mapping[str, torch.Tensor] = field(default_factory=dict)
     writable: bool = True
     state: Optional[torch.Tensor] = None
+    others: Mapping[str, "CacheView"] = field(default_factory=dict)
 
     @property
     def k_pages(self) -> Optional[torch.Tensor]:
@@ -400,6 +403,12 @@ class Block:
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
                 cache: CacheView) -> torch.Tensor:
         raise NotImplementedError
+
+    def cached_parts(self) -> Dict[str, Part]:
+        """The parts of this layer that keep something between steps (those with a ``cache_spec`` or a
+        ``state_spec``), by name.  "mixer" gets the view that ``forward`` is handed; every other name is found in
+        that view's ``others``.  Each gets pages and state slots of its own from the cache manager."""
+        return {"mixer": self.mixer}
 
     def native(self, program: Any, view: CacheView) -> None:
         """Write the arrangement into a step's program: its parts' operations in the order ``forward`` runs them

@@ -35,7 +35,8 @@ def test_greedy_A_through_the_entry_point(folders):
     from infernum_amd import GenerateOptions
     d, cfg, w = folders["A"]
     prompt = [3, 141, 59, 26, 53, 58, 97]
-    want = P.greedy(cfg, w, prompt, 16)
+    want = P.greedy(cfg, w, prompt, 16, eos=cfg["eos_token_id"])     # the entry point stops at the model's own
+    assert len(want) == 16
     rt = _runtime(d, "float32", block_size=4, num_blocks=16, max_batch_size=2)
     assert rt.generate(prompt, GenerateOptions(max_new_tokens=16)) == want
     assert list(rt.generate_stream(prompt, GenerateOptions(max_new_tokens=16))) == want
@@ -52,7 +53,7 @@ def test_greedy_B_varied_tokens(folders, dtype):
     from infernum_amd import GenerateOptions
     d, cfg, w = folders["B"]
     prompt = [3, 141, 59, 26, 53, 58, 97]
-    want = P.greedy(cfg, w, prompt, 24)
+    want = P.greedy(cfg, w, prompt, 24, eos=cfg["eos_token_id"])
     assert len(set(want)) >= 5
     rt = _runtime(d, dtype, block_size=8, num_blocks=8, max_batch_size=2, max_prefill_tokens=4)
     assert rt.generate(prompt, GenerateOptions(max_new_tokens=24)) == want
@@ -77,14 +78,18 @@ def test_sampled_B_portions_mixed_with_decoding(folders):
     assert any(e[0] == 1 and e[-1] > 1 for e in sizes), f"no step mixed decoded tokens with a portion: {sizes}"
     assert max(sum(e) for e in sizes) <= 16 and max(max(e) for e in sizes) <= 8
     for p, s, out in zip(prompts, sp, got):
-        assert len(out) == 12
         toks = list(p)
-        for i, t in enumerate(out):
+        for i in range(12):
             logits = P.forward(cfg, w, toks)[-1]
             u = P.uniform_for_token(s.seed, i)
             want = P.sample_token(logits, s.temperature, s.top_p, u, s.repetition_penalty, toks[-8:])
-            assert want == t, f"request with seed {s.seed}: token {i} is {t}, the plain sampler gives {want}"
-            toks.append(t)
+            if want == cfg["eos_token_id"]:                 # the model's end-of-sequence token stops the request
+                assert len(out) == i
+                break
+            assert i < len(out) and want == out[i], f"request with seed {s.seed}: token {i}: the plain sampler gives {want}"
+            toks.append(want)
+        else:
+            assert len(out) == 12
 
 
 def test_too_few_pages_changes_no_greedy_token(folders):
@@ -92,11 +97,12 @@ def test_too_few_pages_changes_no_greedy_token(folders):
     d, cfg, w = folders["A"]
     g = torch.Generator().manual_seed(5)
     prompts = [torch.randint(0, 256, (n,), generator=g).tolist() for n in (9, 17, 6, 12)]
-    want = [P.greedy(cfg, w, p, 20) for p in prompts]
+    eos = cfg["eos_token_id"]
+    want = [P.greedy(cfg, w, p, 20, eos=eos) for p in prompts]
     roomy = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=4, max_prefill_tokens=8)
     assert roomy.generate_batch(prompts, GenerateOptions(max_new_tokens=20)) == want
     tight = _runtime(d, "float32", block_size=4, num_blocks=18, max_batch_size=4, max_prefill_tokens=8)
-    seqs = [tight.submit(p, GenerateOptions(max_new_tokens=20)) for p in prompts]
+    seqs = [tight.submit(p, GenerateOptions(max_new_tokens=20, eos_token_id=eos)) for p in prompts]
     n_back = 0
     while not tight.scheduler.is_idle():
         n_back += len(tight.step().set_back)
@@ -177,9 +183,10 @@ def test_too_few_pages_changes_no_sampled_token(folders):
     prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (9, 17, 6, 12)]
     sp = [SamplingParams(temperature=0.8, top_p=0.95, seed=7 + i, repetition_penalty=1.05,
                          repetition_penalty_window=6) for i in range(4)]
-    opts = [GenerateOptions(max_new_tokens=16, sampling=s) for s in sp]
+    opts = [GenerateOptions(max_new_tokens=16, sampling=s, eos_token_id=cfg["vocab_size"] - 1) for s in sp]
     roomy = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=4, max_prefill_tokens=8)
     want = roomy.generate_batch(prompts, opts)
+    assert all(len(out) == 16 for out in want), "a request stopped at its end-of-sequence token: take another"
     tight = _runtime(d, "float32", block_size=4, num_blocks=17, max_batch_size=4, max_prefill_tokens=8)
     seqs = [tight.submit(p, o) for p, o in zip(prompts, opts)]
     n_back = 0
@@ -202,7 +209,8 @@ def test_too_few_pages_changes_no_sampled_token(folders):
 def test_command_line(folders):
     d, cfg, w = folders["A"]
     prompt = [3, 141, 59, 26, 53, 58, 97]
-    want = P.greedy(cfg, w, prompt, 6)
+    want = P.greedy(cfg, w, prompt, 6, eos=cfg["eos_token_id"])
+    assert len(want) == 6
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), "-m", d, "--greedy", "-n", "6",
                            "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)), "--max-seq-len", "64"],
                           capture_output=True, text=True, timeout=600)
@@ -210,6 +218,25 @@ def test_command_line(folders):
     assert "Decoding: greedy (argmax)" in proc.stdout and "KV cache: enabled" in proc.stdout
     assert " ".join(map(str, want)) in proc.stdout
     assert "Generated 6 tokens in" in proc.stdout
+
+
+def test_command_line_with_random_weights(folders, tmp_path):
+    """--random CONFIG.json --seed S: the tokens of the folder that bin/random_model writes from the same two."""
+    import json
+    d, cfg, w = folders["B"]
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(cfg))
+    from infernum_amd.config import LlamaConfig
+    from infernum_amd.weights import write_random_model
+    folder = write_random_model(LlamaConfig.from_dict(cfg, where="B"), str(tmp_path / "model"), 9, torch.float32)
+    pcfg, pw = P.read_model(folder)
+    prompt = [3, 141, 59, 26, 53]
+    want = P.greedy(pcfg, pw, prompt, 6, eos=pcfg["eos_token_id"])
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), "--random", str(config), "-s", "9",
+                           "--greedy", "-n", "6", "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)),
+                           "--max-seq-len", "64"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert "Random weights from:" in proc.stdout and " ".join(map(str, want)) in proc.stdout
 
 
 def test_bench_command_line(folders):

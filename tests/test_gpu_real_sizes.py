@@ -12,6 +12,12 @@ plain implementation itself:
 * bfloat16: the plain model with every stored activation rounded to bfloat16 (``round_to``) differs from the
   exact one by Ebf; that is what rounding alone does at these sizes.  The engine may differ from the exact
   model by one and a half times that, and from the rounding model too (two sets of roundings, independent of each other).
+  The largest difference over millions of logits is a loose measure (one unlucky logit sets it), so the root mean
+  square of the difference is held as well, and tightly: the engine rounds where the rounding model rounds, so its
+  root-mean-square distance from the exact model may be 1.1 times the rounding model's (measured: 0.84 to 1.0
+  times), and its distance from the rounding model 1.2 times that (two sets of roundings of the same numbers,
+  partly the same ones: measured 0.6 to 1.03 times, where independent sets would give the square root of two).
+  A defect of three per cent in one bfloat16 kernel at these sizes adds some 3e-2 to distances of 1e-2.
 """
 import pytest
 import torch
@@ -63,9 +69,14 @@ def real(request, tmp_path_factory):
     short = min(reqs, key=lambda r: len(reqs[r]))
     e32 = _ratio(P.forward(pcfg, w, reqs[short], dtype=torch.float32), exact[short])
     ebf = max(_ratio(rounding[r], exact[r]) for r in reqs)
-    print(f"real sizes {request.param}: plain fp32 against float64 {e32:.2e}; plain with bfloat16 roundings against exact {ebf:.2e}")
+    # the same in the root mean square over all logits: what the rows are like, where the largest difference is
+    # set by one unlucky logit among millions
+    sq = sum(float((rounding[r] - exact[r]).pow(2).sum()) for r in reqs)
+    ebf_rms = (sq / sum(float(exact[r].pow(2).sum()) for r in reqs)) ** 0.5
+    print(f"real sizes {request.param}: plain fp32 against float64 {e32:.2e}; plain with bfloat16 roundings against exact "
+          f"{ebf:.2e} at the worst logit, {ebf_rms:.2e} in the root mean square")
     assert 1e-6 < e32 < 1e-4 and 1e-2 < ebf < 0.3, "the plain implementations disagree in a way rounding does not explain"
-    return d, reqs, exact, rounding, e32, ebf
+    return d, reqs, exact, rounding, e32, ebf, ebf_rms
 
 
 def _traces(reqs):
@@ -78,7 +89,7 @@ def _traces(reqs):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_all_ways_of_cutting_at_real_sizes(real, dtype):
     from infernum_amd import CacheConfig, Engine
-    d, reqs, exact, rounding, e32, ebf = real
+    d, reqs, exact, rounding, e32, ebf, ebf_rms = real
     max_tokens, traces = _traces(reqs)
     eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(
         page_size=16, num_pages=max_tokens // 16 + 1, num_state_slots=4, poison_freed_pages=True))
@@ -93,6 +104,10 @@ def test_all_ways_of_cutting_at_real_sizes(real, dtype):
             worst_r, rms_r, where_r = TT.error_against(got, rounding)
             line += f"; against the rounding plain model {worst_r / rms_r:.2e}"
             assert worst_r <= tol * rms_r, line
+            to_exact, to_rounding = TT.rms_error_against(got, exact), TT.rms_error_against(got, rounding)
+            line += (f"; root mean square: {to_exact:.2e} from the exact model, {to_rounding:.2e} from the rounding one "
+                     f"(which is {ebf_rms:.2e} from the exact one)")
+            assert to_exact <= 1.1 * ebf_rms and to_rounding <= 1.2 * ebf_rms, line
         print(line)
     eng.cache.check()
     assert all(g.allocator.num_free == g.allocator.num_pages for g in eng.cache.groups)

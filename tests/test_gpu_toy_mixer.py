@@ -765,3 +765,114 @@ def test_a_norm_an_embedding_and_a_head_of_the_models_own(tmp_path, dtype):
         worst, rms, where = TT.error_against(got, ref)
         print(f"toy5 {dtype} {name}: {worst / rms:.2e} at {where}")
         assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+
+
+# ------------------------------------------------------------------------------------------------
+# Two cached parts in one layer: an attention (pages) and the mixer with state of this file's top side by side,
+# each with memory of its own from the cache manager.
+class HybridBlock(Block):
+    """h += attention(n) + ema(n) with n = norm1(h); then h += feed_forward(norm2(h))."""
+
+    def cached_parts(self):
+        return {"mixer": self.mixer, "second": self.extra["second"]}
+
+    def forward(self, h, pending, ctx, cache):
+        n = self.mixer_norm.forward(h, pending)
+        a = self.mixer.forward(n, ctx, cache)
+        a = a.joined(n.dtype) if hasattr(a, "joined") else a
+        b = self.extra["second"].forward(n, ctx, cache.others["second"])
+        n2 = self.feed_forward_norm.forward(h, (a.float() + b.float()).to(n.dtype))
+        return self.feed_forward.forward(n2, ctx)
+
+
+@dataclass(frozen=True)
+class Toy6Config:
+    vocab_size: int = 70
+    hidden_size: int = 48
+    state_size: int = 10
+    num_heads: int = 3
+    intermediate_size: int = 64
+    model_type: str = "toy-hybrid"
+
+    @staticmethod
+    def from_dict(raw, where="config.json"):
+        return Toy6Config(**{k: v for k, v in raw.items() if k in Toy6Config.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy6_spec(cfg: Toy6Config) -> ModelSpec:
+    H, d = cfg.hidden_size, cfg.hidden_size // cfg.num_heads
+    norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "init": ("uniform", 0.5, 1.5)}, prefix)
+    layers = [LayerSpec("hybrid",
+                        PartSpec("attention", {"hidden_size": H, "num_heads": cfg.num_heads, "num_kv_heads": 1,
+                                               "head_dim": d, "init_std": 0.1, "position": {
+                                                   "kind": "rope", "params": {"head_dim": d, "theta": 1000.0, "scaling": None}}},
+                                 f"l.{i}.attn."),
+                        PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size, "init_std": 0.1},
+                                 f"l.{i}.ff."),
+                        norm(f"l.{i}.n1."), norm(f"l.{i}.n2."),
+                        extra={"second": ("mixer", PartSpec("ema", {"hidden_size": H, "state_size": cfg.state_size},
+                                                            f"l.{i}.ema."))})
+              for i in range(2)]
+    return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.5}, "emb."),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn."),
+                     head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "init_std": 0.1}, "head."))
+
+
+def plain_forward6(cfg: Toy6Config, w, ids):
+    W = {k: v.double() for k, v in w.items()}
+    H, nh = cfg.hidden_size, cfg.num_heads
+    d, T = H // nh, len(ids)
+    freqs, pos = P.rope_frequencies(d, 1000.0, None), torch.arange(T)
+    h = P.embedding(W["emb.weight"], ids)
+    for l in range(2):
+        n = P.rms_norm(h, W[f"l.{l}.n1.weight"], 1e-5)
+        p = f"l.{l}.attn."
+        q = P.rope(P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d), pos, freqs)
+        k = P.rope(P.linear(n, W[p + "k_proj.weight"]).reshape(T, 1, d), pos, freqs)
+        v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, 1, d)
+        a = P.linear(P.causal_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, H), W[p + "o_proj.weight"])
+        p = f"l.{l}.ema."
+        u = P.linear(n, W[p + "in_proj.weight"])
+        s, rows = torch.zeros(cfg.state_size, dtype=torch.float64), []
+        for t in range(T):
+            s = W[p + "decay"] * s + u[t]
+            rows.append(s)
+        h = h + a + P.linear(torch.stack(rows), W[p + "out_proj.weight"])
+        m = P.rms_norm(h, W[f"l.{l}.n2.weight"], 1e-5)
+        h = h + P.linear(P.swiglu(P.linear(m, W[f"l.{l}.ff.gate_proj.weight"]), P.linear(m, W[f"l.{l}.ff.up_proj.weight"])),
+                         W[f"l.{l}.ff.down_proj.weight"])
+    return P.linear(P.rms_norm(h, W["fn.weight"], 1e-5), W["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_two_cached_parts_side_by_side_in_one_layer(tmp_path, dtype):
+    register_part("mixer", "ema", EmaMixer, replace=True)
+    register_part("block", "hybrid", HybridBlock, replace=True)
+    register_architecture("toy-hybrid", Toy6Config, toy6_spec, replace=True)
+    cfg = Toy6Config()
+    d = write_random_model(cfg, str(tmp_path / "toy6"), seed=44,
+                           dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    _, w = P.read_model(d)
+    eng = Engine.from_pretrained(d, dtype=dtype, cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4,
+                                                                          poison_freed_pages=True))
+    # per layer the attention's pages and the other mixer's state, each its own
+    assert [sorted(p) for p in eng.cache.pages] == [["k", "v"], [], ["k", "v"], []]
+    assert [s is not None for s in eng.cache.state] == [False, True, False, True]
+    assert all(v.k_pages is not None and v.others["second"].state is not None for v in eng.views)
+    assert eng.views[0].others["second"].state is not eng.views[1].others["second"].state
+    reqs = TT.make_requests(cfg.vocab_size, (31, 6, 47, 19), seed=6)
+    ref = {r: plain_forward6(cfg, w, t) for r, t in reqs.items()}
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=3)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy6 {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+        eng.cache.check()
+        assert eng.cache.slots.num_free == 4 and all(g.allocator.num_free == 48 for g in eng.cache.groups)

@@ -135,3 +135,15 @@ def error_against(got: Dict[Tuple[str, int], torch.Tensor], want: Dict[str, torc
         sq += float((ref * ref).sum())
         n += ref.numel()
     return worst, (sq / max(n, 1)) ** 0.5, where
+
+
+def rms_error_against(got: Dict[Tuple[str, int], torch.Tensor], want: Dict[str, torch.Tensor]) -> float:
+    """Root mean square of the difference over all rows, as a fraction of the RMS of the wanted logits: where the
+    largest difference is set by one unlucky logit among millions, this one tells what the rows are like."""
+    sq_d, sq_w, n = 0.0, 0.0, 0
+    for (r, p), row in got.items():
+        ref = want[r][p].to(torch.float64)
+        sq_d += float((row.to(torch.float64) - ref).pow(2).sum())
+        sq_w += float((ref * ref).sum())
+        n += ref.numel()
+    return (sq_d / max(sq_w, 1e-300)) ** 0.5
