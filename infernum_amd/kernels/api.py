@@ -480,17 +480,31 @@ def _attn(d: int) -> ctypes.CDLL:
     return lib
 
 
-def decode_splits(batch: int, nh: int, nkv: int, max_len: int) -> int:
+_compute_units: Dict[int, int] = {}
+
+
+def compute_units(device: Optional[torch.device] = None) -> int:
+    """Compute units of the device (asked once): what the launch shapes below are sized against."""
+    idx = device.index if (device is not None and device.index is not None) else torch.cuda.current_device()
+    cus = _compute_units.get(idx)
+    if cus is None:
+        cus = _compute_units[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
+    return cus
+
+
+def decode_splits(batch: int, nh: int, nkv: int, max_len: int, device: Optional[torch.device] = None) -> int:
     """Parts the keys of a request are cut into, so that a small batch still fills the GPU (workgroups of
-    four waves, each wave one tile of 16 keys at a time): about 256 workgroups while the batch alone gives at
-    most 64, about 512 up to 160, and no parts above that (8B shape, 527 keys: 24 requests 13.9 us whole against
-    15.3 in three parts, 32 requests 15.4 against 17.1 in two); at least 8 tiles a workgroup (more and shorter
-    parts cost more in the join than they gain)."""
+    four waves, each wave one tile of 16 keys at a time): about one workgroup a compute unit while the batch alone
+    gives at most a quarter of that, about two up to five eighths, and no parts above that (measured on 256
+    compute units with the 8B shape and 527 keys: 24 requests 13.9 us whole against 15.3 in three parts, 32
+    requests 15.4 against 17.1 in two); at least 8 tiles a workgroup (more and shorter parts cost more in the
+    join than they gain)."""
+    cus = compute_units(device)
     groups = batch * nkv * ((nh // nkv + 15) // 16)
     tiles = max(1, (max_len + 15) // 16)
-    if groups >= 160:
+    if 8 * groups >= 5 * cus:
         return 1
-    wanted = 256 // groups if groups <= 64 else 512 // groups
+    wanted = cus // groups if 4 * groups <= cus else 2 * cus // groups
     return max(1, min(wanted, tiles // 8, 64))
 
 
@@ -509,7 +523,7 @@ def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Te
     ps = k_pages.shape[2]
     _need(ps % 4 == 0, f"attention_decode: page size {ps} is not a multiple of 4")
     _need(block_tables.shape[1] * ps >= max_len, "attention_decode: block_tables are narrower than max_len")
-    splits = num_splits or decode_splits(B, nh, nkv, max_len)
+    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)
@@ -559,7 +573,7 @@ def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[t
     ps = k_pages.shape[2]
     _need(ps % 4 == 0, f"attention_decode_rotating: page size {ps} is not a multiple of 4")
     _need(block_tables.shape[1] * ps >= max_len, "attention_decode_rotating: block_tables are narrower than max_len")
-    splits = num_splits or decode_splits(B, nh, nkv, max_len)
+    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)
@@ -605,9 +619,6 @@ def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
         "attention_prefill")
 
 
-_compute_units: Dict[int, int] = {}
-
-
 def prefill_launch_shape(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_lens: Sequence[int],
                          window: int, device: torch.device) -> int:
     """The shape of the :func:`attention_prefill` launch for these portions of prompts (``q_lens`` new tokens
@@ -639,10 +650,7 @@ def prefill_launch_shape(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_l
             longest = max(longest, keys)
     if tiles == 0:
         return 0
-    idx = device.index if device.index is not None else torch.cuda.current_device()
-    cus = _compute_units.get(idx)
-    if cus is None:
-        cus = _compute_units[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
+    cus = compute_units(device)
     workgroups = tiles * nkv * ((G + hpw - 1) // hpw)
     if hpw == 4 and 4 * workgroups < 3 * cus:
         hpw, workgroups = 2, tiles * nkv * ((G + 1) // 2)
