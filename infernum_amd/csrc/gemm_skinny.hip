@@ -50,7 +50,10 @@ template <> __device__ __forceinline__ void store_out<uint16_t>(uint16_t* p, flo
 // GLU (one split only): a workgroup takes 32 columns n of the result; waves 0 and 1 multiply with the rows n
 // of the first half of W, waves 2 and 3 with the rows N/2 + n of the second half; the halves meet in LDS and
 // silu(first) * second goes to C[m, n], n < N/2.
-template <int MT, bool GLU, typename TO, int KC>
+// TILED: W is the copy that tile_weight_kernel lays out, in which the 64 rows x 256 values that a workgroup
+// multiplies with in one chunk are 32 KB of consecutive memory, chunk after chunk: every workgroup then reads one
+// stretch of memory front to back, where the rows of the matrix as the file holds it lie K values apart.
+template <int MT, bool GLU, typename TO, int KC, bool TILED>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ X,
                                                                     const uint16_t* __restrict__ W,
                                                                     TO* __restrict__ C, float* __restrict__ part,
@@ -77,6 +80,9 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
 
   const int n_row = (n_base + r < NO) ? n_base + r : NO - 1;
   const uint16_t* wrow = W + ((size_t)n_row + (size_t)half * NO) * K;
+  // TILED: this lane's row within the workgroup's tiles, which follow each other chunk by chunk
+  const int chunks256 = (K + SK_KC - 1) / SK_KC;
+  const uint16_t* wtile = W + ((size_t)blockIdx.x * chunks256 * SK_BN + (size_t)(wave * 16 + r)) * SK_KC;
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -106,6 +112,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   };
   uint4 wcur[NLD], wnext[NLD];
   auto load_w = [&](int c, uint4 (&dst)[NLD]) {
+    if (TILED) {
+      // piece c of KC values lies in chunk c / PER_CHUNK of 256; the copy is padded with zeros to whole chunks
+      const uint16_t* src = wtile + (size_t)(c / PER_CHUNK) * (SK_BN * SK_KC) + (c % PER_CHUNK) * KC;
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) dst[i] = load_stream_16(src + (i * 4 + q) * 8);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int k = c * KC + (i * 4 + q) * 8;
@@ -216,23 +229,23 @@ static int skinny_splits(int N, int K) {
 // Number of K splits the kernel uses for a weight [N, K] (a function of N and K only).
 extern "C" int ia_gemm_skinny_splits(int N, int K) { return (N > 0 && K > 0) ? skinny_splits(N, K) : 0; }
 
-template <int MT, bool GLU, typename TO, int KC>
+template <int MT, bool GLU, typename TO, int KC, bool TILED>
 static int launch_skinny_one(dim3 grid, const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K,
                              int cps, hipStream_t stream) {
   constexpr size_t lds = (size_t)2 * MT * 16 * (KC + SK_XPAD) * sizeof(uint16_t);
   static bool allowed = false;      // more than 64 KB of LDS has to be asked for, once per kernel
   if (lds > 65536 && !allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, GLU, TO, KC>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, GLU, TO, KC, TILED>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     allowed = true;
   }
-  gemm_skinny_kernel<MT, GLU, TO, KC><<<grid, SK_WAVES * 64, lds, stream>>>(x, w, c, part, M, N, K, cps);
+  gemm_skinny_kernel<MT, GLU, TO, KC, TILED><<<grid, SK_WAVES * 64, lds, stream>>>(x, w, c, part, M, N, K, cps);
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
 
-template <bool GLU, typename TO>
+template <bool GLU, typename TO, bool TILED = false>
 static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* part, int M, int N, int K, int splits,
                          hipStream_t stream) {
   const int nchunks = (K + SK_KC - 1) / SK_KC;
@@ -241,15 +254,15 @@ static int launch_skinny(const uint16_t* x, const uint16_t* w, TO* c, float* par
   const int cols = GLU ? SK_BN / 2 : SK_BN;           // columns of the result per workgroup
   dim3 grid((NO + cols - 1) / cols, splits);
   switch ((M + 15) / 16) {
-    case 1: return launch_skinny_one<1, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 2: return launch_skinny_one<2, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 3: return launch_skinny_one<3, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 4: return launch_skinny_one<4, GLU, TO, SK_KC>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 1: return launch_skinny_one<1, GLU, TO, SK_KC, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 2: return launch_skinny_one<2, GLU, TO, SK_KC, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 3: return launch_skinny_one<3, GLU, TO, SK_KC, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 4: return launch_skinny_one<4, GLU, TO, SK_KC, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
     // above 64 rows: pieces of 128, so that the two stages of X of two workgroups fit a compute unit's LDS
-    case 5: return launch_skinny_one<5, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 6: return launch_skinny_one<6, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 7: return launch_skinny_one<7, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
-    case 8: return launch_skinny_one<8, GLU, TO, SK_KC / 2>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 5: return launch_skinny_one<5, GLU, TO, SK_KC / 2, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 6: return launch_skinny_one<6, GLU, TO, SK_KC / 2, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 7: return launch_skinny_one<7, GLU, TO, SK_KC / 2, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
+    case 8: return launch_skinny_one<8, GLU, TO, SK_KC / 2, TILED>(grid, x, w, c, part, M, N, K, cps, stream);
     default: return IA_ERR_UNSUPPORTED;
   }
 }
@@ -270,8 +283,9 @@ static int launch_join(const float* part, TO* c, int M, int N, int splits, int e
 // epilogue.  workspace: fp32, at least ia_gemm_skinny_splits(N, K) * M * N values when that count is above one
 // or an epilogue is asked for; may be null otherwise.  C == null: the partial sums are left in the workspace
 // as [splits, M, N] for a later kernel to join.
-extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
-                              int epilogue, float* workspace, size_t workspace_floats, hipStream_t stream) {
+template <bool TILED>
+static int skinny_product(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K, int epilogue,
+                          float* workspace, size_t workspace_floats, hipStream_t stream) {
   if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
   if (epilogue != SK_EPI_NONE && epilogue != SK_EPI_SWIGLU) return IA_ERR_BAD_ARG;
   if (epilogue == SK_EPI_SWIGLU && (N & 1)) return IA_ERR_BAD_ARG;
@@ -282,32 +296,98 @@ extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dty
   const uint16_t* w = (const uint16_t*)W;
   if (splits == 1 && epilogue == SK_EPI_SWIGLU && C != nullptr) {
     // one pass: both halves of W in the same wave, the activation in the epilogue
-    if (out_dtype == IA_F32) return launch_skinny<true, float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
-    return launch_skinny<true, uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
+    if (out_dtype == IA_F32) return launch_skinny<true, float, TILED>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
+    return launch_skinny<true, uint16_t, TILED>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
   }
   const bool via_workspace = splits > 1 || epilogue != SK_EPI_NONE || C == nullptr;
   if (via_workspace && (!workspace || workspace_floats < (size_t)splits * M * N)) return IA_ERR_BAD_ARG;
   if (!via_workspace) {
-    if (out_dtype == IA_F32) return launch_skinny<false, float>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
-    return launch_skinny<false, uint16_t>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
+    if (out_dtype == IA_F32) return launch_skinny<false, float, TILED>(x, w, (float*)C, nullptr, M, N, K, 1, stream);
+    return launch_skinny<false, uint16_t, TILED>(x, w, (uint16_t*)C, nullptr, M, N, K, 1, stream);
   }
-  const int rc = launch_skinny<false, float>(x, w, nullptr, workspace, M, N, K, splits, stream);
+  const int rc = launch_skinny<false, float, TILED>(x, w, nullptr, workspace, M, N, K, splits, stream);
   if (rc != IA_OK || C == nullptr) return rc;
   if (out_dtype == IA_F32) return launch_join<float>(workspace, (float*)C, M, N, splits, epilogue, stream);
   return launch_join<uint16_t>(workspace, (uint16_t*)C, M, N, splits, epilogue, stream);
 }
 
+extern "C" int ia_gemm_skinny(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
+                              int epilogue, float* workspace, size_t workspace_floats, hipStream_t stream) {
+  return skinny_product<false>(X, W, C, out_dtype, M, N, K, epilogue, workspace, workspace_floats, stream);
+}
+
+// ---- the weight laid out for the kernel: every workgroup's 64 rows x 256 values of a chunk consecutive ----------
+// Whether the copy for this weight and use is laid out for the kernel that multiplies with both halves of
+// [gate | up] at once (a workgroup then takes 32 rows of each half).
+static bool tiled_glu(int N, int K, int epilogue) { return epilogue == SK_EPI_SWIGLU && skinny_splits(N, K) == 1; }
+
+// Elements (bf16) of the copy: rows padded to whole workgroups, K to whole chunks.
+extern "C" size_t ia_gemm_skinny_tiled_elements(int N, int K, int epilogue) {
+  if (N <= 0 || K <= 0) return 0;
+  const int NO = tiled_glu(N, K, epilogue) ? N / 2 : N, cols = tiled_glu(N, K, epilogue) ? SK_BN / 2 : SK_BN;
+  const size_t blocks = (size_t)(NO + cols - 1) / cols, chunks = (size_t)(K + SK_KC - 1) / SK_KC;
+  return blocks * chunks * SK_BN * SK_KC;
+}
+
+__global__ __launch_bounds__(256) void tile_weight_kernel(const uint16_t* __restrict__ W, uint16_t* __restrict__ T,
+                                                          int N, int K, int glu, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;      // one element of the copy
+  if (idx >= total) return;
+  const int kk = (int)(idx % SK_KC);
+  const size_t rowi = idx / SK_KC;
+  const int rib = (int)(rowi % SK_BN);                            // row within the workgroup's tile
+  const size_t bc = rowi / SK_BN;
+  const int chunks = (K + SK_KC - 1) / SK_KC;
+  const int chunk = (int)(bc % chunks);
+  const size_t block = bc / chunks;
+  const int k = chunk * SK_KC + kk;
+  int n;
+  bool ok;
+  if (glu) {
+    const int NO = N / 2, col = (int)block * (SK_BN / 2) + (rib & 15) + ((rib >> 4) & 1) * 16, half = rib >> 5;
+    ok = col < NO;
+    n = half * NO + col;
+  } else {
+    n = (int)block * SK_BN + rib;
+    ok = n < N;
+  }
+  T[idx] = (ok && k < K) ? W[(size_t)n * K + k] : (uint16_t)0;
+}
+
+// T (ia_gemm_skinny_tiled_elements(N, K, epilogue) values) = W [N, K] laid out for ia_gemm_skinny_tiled with the
+// same epilogue.
+extern "C" int ia_gemm_skinny_tile(const void* W, void* T, int N, int K, int epilogue, hipStream_t stream) {
+  if (!W || !T || N <= 0 || K <= 0 || (epilogue != SK_EPI_NONE && epilogue != SK_EPI_SWIGLU)) return IA_ERR_BAD_ARG;
+  const size_t total = ia_gemm_skinny_tiled_elements(N, K, epilogue);
+  const size_t grid = (total + 255) / 256;
+  if (grid > 0x7fffffffu) return IA_ERR_UNSUPPORTED;
+  tile_weight_kernel<<<(unsigned)grid, 256, 0, stream>>>((const uint16_t*)W, (uint16_t*)T, N, K,
+                                                         tiled_glu(N, K, epilogue) ? 1 : 0, total);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ia_gemm_skinny with the weight given as the copy that ia_gemm_skinny_tile made for the same epilogue: the same
+// sums in the same order, the same bits.
+extern "C" int ia_gemm_skinny_tiled(const void* X, const void* T, void* C, int out_dtype, int M, int N, int K,
+                                    int epilogue, float* workspace, size_t workspace_floats, hipStream_t stream) {
+  return skinny_product<true>(X, T, C, out_dtype, M, N, K, epilogue, workspace, workspace_floats, stream);
+}
+
 // The same product for any number of rows, 128 at a time (a result in fp32 from bf16 operands has no other
 // kernel here: the head of a step that wants the logits of many places).  The workspace serves every piece in turn.
-extern "C" int ia_gemm_skinny_rows(const void* X, const void* W, void* C, int out_dtype, int M, int N, int K,
+// tiled != 0: W is the copy of ia_gemm_skinny_tile (no epilogue).
+extern "C" int ia_gemm_skinny_rows(const void* X, const void* W, int tiled, void* C, int out_dtype, int M, int N, int K,
                                    float* workspace, size_t workspace_floats, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0) return IA_ERR_UNSUPPORTED;
   if (out_dtype != IA_F32 && out_dtype != IA_BF16) return IA_ERR_BAD_ARG;
   const size_t out_bytes = out_dtype == IA_F32 ? 4 : 2;
   for (int m0 = 0; m0 < M; m0 += 128) {
     const int m = M - m0 < 128 ? M - m0 : 128;
-    const int rc = ia_gemm_skinny((const char*)X + (size_t)m0 * K * 2, W, (char*)C + (size_t)m0 * N * out_bytes, out_dtype,
-                                  m, N, K, SK_EPI_NONE, workspace, workspace_floats, stream);
+    const void* x = (const char*)X + (size_t)m0 * K * 2;
+    void* c = (char*)C + (size_t)m0 * N * out_bytes;
+    const int rc = tiled ? ia_gemm_skinny_tiled(x, W, c, out_dtype, m, N, K, SK_EPI_NONE, workspace, workspace_floats, stream)
+                         : ia_gemm_skinny(x, W, c, out_dtype, m, N, K, SK_EPI_NONE, workspace, workspace_floats, stream);
     if (rc != IA_OK) return rc;
   }
   return IA_OK;
@@ -366,4 +446,5 @@ extern "C" int ia_gemm_skinny_no_alloc(const void* X, const void* W, void* C, in
 // ---- the launchers of this file as operations of a step's program (see op_call.h) ----
 #include "op_call.h"
 IA_OP(ia_gemm_skinny)
+IA_OP(ia_gemm_skinny_tiled)
 IA_OP(ia_gemm_skinny_rows)

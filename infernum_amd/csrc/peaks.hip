@@ -34,6 +34,46 @@ __global__ __launch_bounds__(PK_THREADS) void peak_read_kernel(const uint4* __re
   sink[(size_t)blockIdx.x * PK_THREADS + threadIdx.x] = acc;
 }
 
+// The same pass with every workgroup on a stretch of its own: workgroup b reads the pieces [b * per, (b + 1) * per)
+// front to back, a wave 1 KB at a time, the workgroup 4 KB at a time (where the strided walk above has all
+// workgroups moving through the buffer side by side, a power-of-two number of bytes apart).
+__global__ __launch_bounds__(PK_THREADS) void peak_read_blocks_kernel(const uint4* __restrict__ p, size_t pieces,
+                                                                      size_t per, uint4* __restrict__ sink) {
+  const size_t first = (size_t)blockIdx.x * per;
+  const size_t last = first + per < pieces ? first + per : pieces;
+  size_t i = first + threadIdx.x;
+  uint4 acc = make_uint4(0u, 0u, 0u, 0u);
+  for (; i + (PK_UNROLL - 1) * PK_THREADS < last; i += PK_UNROLL * PK_THREADS) {
+    uint4 v[PK_UNROLL];
+#pragma unroll
+    for (int u = 0; u < PK_UNROLL; ++u) v[u] = p[i + u * PK_THREADS];
+#pragma unroll
+    for (int u = 0; u < PK_UNROLL; ++u) {
+      acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w;
+    }
+  }
+  for (; i < last; i += PK_THREADS) {
+    const uint4 v = p[i];
+    acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+  }
+  sink[(size_t)blockIdx.x * PK_THREADS + threadIdx.x] = acc;
+}
+
+// A copy: every piece is read once and written once (2 * bytes of traffic).
+__global__ __launch_bounds__(PK_THREADS) void peak_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                               size_t pieces) {
+  const size_t stride = (size_t)gridDim.x * PK_THREADS;
+  size_t i = (size_t)blockIdx.x * PK_THREADS + threadIdx.x;
+  for (; i + (PK_UNROLL - 1) * stride < pieces; i += PK_UNROLL * stride) {
+    uint4 v[PK_UNROLL];
+#pragma unroll
+    for (int u = 0; u < PK_UNROLL; ++u) v[u] = src[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < PK_UNROLL; ++u) dst[i + u * stride] = v[u];
+  }
+  for (; i < pieces; i += stride) dst[i] = src[i];
+}
+
 // Every wave keeps four independent accumulators of v_mfma_f32_32x32x16_bf16 busy: 4 * 32768 flops a round.
 __global__ __launch_bounds__(PK_THREADS) void peak_mfma_kernel(int rounds, float* __restrict__ sink) {
   const int lane = threadIdx.x & 63;
@@ -63,6 +103,23 @@ __global__ __launch_bounds__(PK_THREADS) void peak_mfma_kernel(int rounds, float
 extern "C" int ia_peak_read(const void* buffer, size_t bytes, void* sink, int workgroups, hipStream_t stream) {
   if (buffer == nullptr || sink == nullptr || bytes < 16 || (bytes & 15) || workgroups <= 0) return IA_ERR_BAD_ARG;
   peak_read_kernel<<<workgroups, PK_THREADS, 0, stream>>>((const uint4*)buffer, bytes / 16, (uint4*)sink);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// The same bytes, every workgroup on a contiguous stretch of its own (see peak_read_blocks_kernel).
+extern "C" int ia_peak_read_blocks(const void* buffer, size_t bytes, void* sink, int workgroups, hipStream_t stream) {
+  if (buffer == nullptr || sink == nullptr || bytes < 16 || (bytes & 15) || workgroups <= 0) return IA_ERR_BAD_ARG;
+  const size_t pieces = bytes / 16, per = (pieces + workgroups - 1) / workgroups;
+  peak_read_blocks_kernel<<<workgroups, PK_THREADS, 0, stream>>>((const uint4*)buffer, pieces, per, (uint4*)sink);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// dst[0 .. bytes) = src[0 .. bytes) (both multiples of 16 bytes, not overlapping).
+extern "C" int ia_peak_copy(const void* src, void* dst, size_t bytes, int workgroups, hipStream_t stream) {
+  if (src == nullptr || dst == nullptr || bytes < 16 || (bytes & 15) || workgroups <= 0) return IA_ERR_BAD_ARG;
+  peak_copy_kernel<<<workgroups, PK_THREADS, 0, stream>>>((const uint4*)src, (uint4*)dst, bytes / 16);
   IA_LAUNCH_CHECK();
   return IA_OK;
 }

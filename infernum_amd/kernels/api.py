@@ -390,9 +390,25 @@ def gemm_skinny_splits(N: int, K: int) -> int:
     return int(_core().ia_gemm_skinny_splits(N, K))
 
 
+def tile_weight(w: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
+    """A copy of the weight [N, K] (bf16) laid out for :func:`gemm_skinny` with this epilogue: the 64 rows x 256
+    values that a workgroup multiplies with in one chunk are 32 KB of consecutive memory, chunk after chunk, so
+    every workgroup reads one stretch of memory front to back (rows padded to whole workgroups, K to whole chunks,
+    with zeros).  Pass it as ``tiled``; the result has the same bits."""
+    _dev(w)
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16 and epilogue in EPILOGUE, "tile_weight: a bf16 matrix [N, K]")
+    N, K = w.shape
+    lib = _core()
+    lib.ia_gemm_skinny_tiled_elements.restype = ctypes.c_size_t
+    n = int(lib.ia_gemm_skinny_tiled_elements(N, K, EPILOGUE[epilogue]))
+    out = torch.empty(n, dtype=torch.bfloat16, device=w.device)
+    _ok(lib.ia_gemm_skinny_tile(_p(w), _p(out), N, K, EPILOGUE[epilogue], _stream()), "tile_weight")
+    return out
+
+
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
                 epilogue: Optional[str] = None, keep_split: bool = False,
-                out_dtype: torch.dtype = torch.bfloat16):
+                out_dtype: torch.dtype = torch.bfloat16, tiled: Optional[torch.Tensor] = None):
     """a[M, K] @ w[N, K]^T for M <= 64 on MFMA, weights streamed once; bf16 operands, fp32 sums.
 
     Returns ``out`` ([M, N] bf16 or fp32; [M, N/2] with the "swiglu" epilogue, silu(left half) * right half),
@@ -410,21 +426,24 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     ws = None
     if splits > 1:
         ws = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+    launch, wp = _core().ia_gemm_skinny, _p(w)
+    if tiled is not None:
+        _need(tiled.is_cuda and tiled.dtype == torch.bfloat16 and tiled.is_contiguous(), "gemm_skinny: the tiled copy")
+        launch, wp = _core().ia_gemm_skinny_tiled, _p(tiled)
     if keep_split and epilogue is None and splits > 1:
-        _ok(_core().ia_gemm_skinny(_p(a), _p(w), None, 0, M, N, K, 0, _p(ws), ctypes.c_size_t(ws.numel()),
-                                   _stream()), "gemm_skinny")
+        _ok(launch(_p(a), wp, None, 0, M, N, K, 0, _p(ws), ctypes.c_size_t(ws.numel()), _stream()), "gemm_skinny")
         return SplitSum(ws)
     n_out = N // 2 if epilogue == "swiglu" else N
     if out is None:
         out = torch.empty((M, n_out), dtype=out_dtype, device=a.device)
     _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (M, n_out) and out.is_contiguous(),
           f"gemm_skinny: out must be contiguous [{M}, {n_out}]")
-    _ok(_core().ia_gemm_skinny(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, EPILOGUE[epilogue], _p(ws),
-                               ctypes.c_size_t(ws.numel() if ws is not None else 0), _stream()), "gemm_skinny")
+    _ok(launch(_p(a), wp, _p(out), DTYPE_CODE[out.dtype], M, N, K, EPILOGUE[epilogue], _p(ws),
+               ctypes.c_size_t(ws.numel() if ws is not None else 0), _stream()), "gemm_skinny")
     return out
 
 
-def gemm_skinny_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def gemm_skinny_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[M, N] = a[M, K] @ w[N, K]^T for any M through :func:`gemm_skinny`'s kernel, 128 rows at a time (an fp32
     result from bf16 operands has no other kernel: the head of a step that wants the logits of many places)."""
     _dev(a, w, out)
@@ -436,7 +455,8 @@ def gemm_skinny_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
     _need(out.dtype in DTYPE_CODE and tuple(out.shape) == (M, N), f"gemm_skinny_rows: out must be contiguous [{M}, {N}]")
     splits = gemm_skinny_splits(N, K)
     ws = torch.empty((splits, min(M, SKINNY_MAX_M), N), dtype=torch.float32, device=a.device) if splits > 1 else None
-    _ok(_core().ia_gemm_skinny_rows(_p(a), _p(w), _p(out), DTYPE_CODE[out.dtype], M, N, K, _p(ws),
+    _ok(_core().ia_gemm_skinny_rows(_p(a), _p(tiled if tiled is not None else w), int(tiled is not None), _p(out),
+                                    DTYPE_CODE[out.dtype], M, N, K, _p(ws),
                                     ctypes.c_size_t(ws.numel() if ws is not None else 0), _stream()), "gemm_skinny_rows")
     return out
 

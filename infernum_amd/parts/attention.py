@@ -24,7 +24,7 @@ import torch
 from ..kernels import api as K
 from .base import (CacheSpec, CacheView, Mixer, PartSpec, Runtime, StepContext, WeightSpec, make_part,
                    register_part)
-from .linear import emit_linear, linear, measure_routes_for
+from .linear import emit_linear, linear, prepare_weights
 
 
 # Steps of up to this many single tokens rotate inside the attention kernel (8B shape: 1.5 % faster at 1 and 8
@@ -111,7 +111,7 @@ class Attention(Mixer):
         self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
         self.w_qkv = self.w_qkv.contiguous()
         self.w_o = tensors["o_proj.weight"].contiguous()
-        measure_routes_for(self.rt, [(self.w_qkv, None, True), (self.w_qkv[: self.nh * self.d], None, True),
+        prepare_weights(self.rt, [(self.w_qkv, None, True), (self.w_qkv[: self.nh * self.d], None, True),
                                      (self.w_o, None, True)])
         if self.qk_transform is not None:
             self.qk_transform.load({name: tensors[name] for name in self.qk_transform.weights()})

@@ -15,7 +15,7 @@ import torch
 
 from ..kernels import api as K
 from .base import Embedding, Head, Runtime, StepContext, WeightSpec, register_part
-from .linear import emit_linear, linear
+from .linear import emit_linear, linear, prepare_weights
 
 
 class TokenEmbedding(Embedding):
@@ -60,6 +60,7 @@ class LinearHead(Head):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors["weight"]
+        prepare_weights(self.rt, [(self.weight, None, False)])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)

@@ -10,7 +10,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import FeedForward, Runtime, StepContext, WeightSpec, register_part
-from .linear import emit_linear, linear, measure_routes_for
+from .linear import emit_linear, linear, prepare_weights
 
 
 class SwiGLUFeedForward(FeedForward):
@@ -34,7 +34,7 @@ class SwiGLUFeedForward(FeedForward):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"].contiguous()
-        measure_routes_for(self.rt, [(self.w_gate_up, "swiglu", False), (self.w_down, None, True)])
+        prepare_weights(self.rt, [(self.w_gate_up, "swiglu", False), (self.w_down, None, True)])
 
     def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):
         act = linear(x, self.w_gate_up, epilogue="swiglu", kernels=self.rt.kernels)

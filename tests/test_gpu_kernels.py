@@ -446,6 +446,50 @@ def test_linear_fp32_result_of_many_rows_from_bf16_operands():
         assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
 
 
+@pytest.mark.parametrize("N,Kd,epilogue", [(28672, 4096, "swiglu"), (330, 264, "swiglu"), (1000, 96, None), (6144, 512, None),
+                                          (4096, 4096, None), (77, 1032, None), (16640, 264, "swiglu")])
+def test_gemm_skinny_with_the_weight_laid_out_for_it(N, Kd, epilogue):
+    """A copy of the weight in which a workgroup's rows of a chunk are consecutive memory (rows padded to whole
+    workgroups, K to whole chunks): the same sums in the same order, so the same bits, for every number of rows,
+    with the activation, with the partial sums kept, and 128 rows at a time."""
+    api = K()
+    w = _rand(N, Kd, dtype=torch.bfloat16, scale=0.1, seed=N % 97)
+    t = api.tile_weight(w, epilogue)
+    assert t.dtype == torch.bfloat16 and t.numel() % (64 * 256) == 0 and t.numel() >= N * Kd
+    for M in (1, 8, 17, 64, 65, 128):
+        x = _rand(M, Kd, dtype=torch.bfloat16, seed=M)
+        a, b = api.gemm_skinny(x, w, epilogue=epilogue), api.gemm_skinny(x, w, epilogue=epilogue, tiled=t)
+        assert torch.equal(a, b), M
+        if epilogue is None:
+            a, b = api.gemm_skinny(x, w, keep_split=True), api.gemm_skinny(x, w, keep_split=True, tiled=t)
+            parts = lambda y: y.parts if isinstance(y, api.SplitSum) else y
+            assert torch.equal(parts(a), parts(b)), M
+            a = api.gemm_skinny(x, w, out_dtype=torch.float32)
+            assert torch.equal(a, api.gemm_skinny(x, w, out_dtype=torch.float32, tiled=t)), M
+    if epilogue is None:
+        x = _rand(300, Kd, dtype=torch.bfloat16, seed=5)
+        a = api.gemm_skinny_rows(x, w, torch.empty(300, N, device=DEV))
+        assert torch.equal(a, api.gemm_skinny_rows(x, w, torch.empty(300, N, device=DEV), tiled=t))
+
+
+def test_wide_weights_get_a_copy_laid_out_for_the_kernel_and_narrow_ones_do_not():
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    from part_harness import runtime
+    rt = runtime("bfloat16")
+    wide, narrow = _rand(16640, 264, dtype=torch.bfloat16), _rand(512, 2048, dtype=torch.bfloat16)
+    L.prepare_weights(rt, [(wide, "swiglu", False), (wide, None, False), (narrow, None, True)])
+    assert L.tiled_copy(wide, "swiglu") is not None and L.tiled_copy(wide, None) is not None
+    assert L.tiled_copy(wide, "swiglu") is not L.tiled_copy(wide, None)          # two layouts: with both halves, without
+    assert L.tiled_copy(narrow, None) is None and K().gemm_skinny_splits(512, 2048) > 1
+    x = _rand(8, 264, dtype=torch.bfloat16, seed=1)
+    assert torch.equal(L.linear(x, wide, epilogue="swiglu"), K().gemm_skinny(x, wide, epilogue="swiglu"))
+    fp = runtime("float32")
+    w32 = _rand(16640, 264)
+    L.prepare_weights(fp, [(w32, None, False)])
+    assert L.tiled_copy(w32, None) is None
+
+
 def test_known_routes_send_rows_to_the_library_where_the_table_says():
     import importlib
     L = importlib.import_module("infernum_amd.parts.linear")
