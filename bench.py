@@ -91,6 +91,9 @@ class DecodeRun:
         self.seqs = [self.rt.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(),
                                     GenerateOptions(max_new_tokens=new_tokens)) for _ in range(batch)]
         while any(s.phase != SequencePhase.DECODE for s in self.seqs):
+            if any(s.phase == SequencePhase.FINISHED for s in self.seqs):
+                raise RuntimeError("a request of the benchmark ended before it decoded: " +
+                                   str([s.error or s.finish_reason for s in self.seqs if s.phase == SequencePhase.FINISHED]))
             self.rt.step()
         sync()
 
@@ -197,6 +200,13 @@ LLAMA_1B = dict(
 )
 
 
+SHAPES = {
+    "8b": (LLAMA_8B, "Llama-3-8B", "llama-3.1-8b-shape-random", "llama3(8,1,4,8192) theta 5e5"),
+    "13b": (LLAMA_13B, "Llama-2-13B", "llama-2-13b-shape-random", "theta 1e4"),
+    "1b": (LLAMA_1B, "Llama-3.2-1B", "llama-3.2-1b-shape-random", "llama3(32,1,4,8192) theta 5e5"),
+}
+
+
 def serve(a) -> int:
     """Continuous batching of 128 requests on the Llama-3.2-1B shape: prompts of 64 to 2,048 tokens, 32 to 512
     new tokens each (uniform, seeded), greedy, context 4,096.  Prints one JSON line of its own: tokens a second
@@ -274,27 +284,34 @@ def serve(a) -> int:
 
 
 def long_contexts(a) -> int:
-    """Further points of the 8B shape: decode at batch 8 with 16,384 and 32,768 tokens of context, and the prefill of
-    one prompt of 8,192 and of 16,384 tokens in a single step.  One JSON line of its own."""
+    """Further points of the 8B shape, one JSON line of its own: decode with 16,384 to 131,072 tokens of context
+    (Llama-3.1's longest; fewer requests as the contexts grow, so that their prompts go in within seconds), the
+    prefill of one prompt of 8,192, 16,384 and 32,768 tokens in a single step, and a prompt of 32,768 tokens going
+    in in portions of 8,192 beside eight requests that decode meanwhile."""
     import torch
-    from infernum_amd import CacheConfig, Engine, LlamaConfig
+    from infernum_amd import BatchConfig, CacheConfig, Engine, GenerateOptions, LlamaConfig, Runtime
     from infernum_amd.engine import StepEntry
+    from infernum_amd.engine.scheduler import SequencePhase
     cfg = LlamaConfig.from_dict(dict(LLAMA_8B))
-    batch, longest = 8, 32768
-    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens_per_step=16384,
-                                cache_config=CacheConfig(page_size=PAGE_SIZE, num_state_slots=batch + 1,
-                                                         num_pages=batch * (longest + 64 + prefill_steps(batch, longest)
-                                                                            + 2 * PAGE_SIZE) // PAGE_SIZE + 8))
-    out = {"metric": "long contexts, Llama-3-8B shape", "dtype": "bf16", "data": "synthetic", "batch": batch, "decode": {},
-           "prefill": {}}
-    for ctx_len in (16384, 32768):
+    points = ((16384, 8), (32768, 8), (65536, 4), (131072 - 1024, 2))     # the last: up to the model's longest sequence
+    tokens = max(b * (c + 64 + prefill_steps(b, c) + 2 * PAGE_SIZE) for c, b in points)
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens_per_step=32768,
+                                cache_config=CacheConfig(page_size=PAGE_SIZE, num_state_slots=10,
+                                                         num_pages=tokens // PAGE_SIZE + 8))
+    out = {"metric": "long contexts, Llama-3-8B shape", "dtype": "bf16", "data": "synthetic", "decode": {}, "prefill": {},
+           "prompt_beside_decoding": {}}
+    for ctx_len, batch in points:
         steps = 32
+        t_in = time.perf_counter()
         dt, ctx_mid = time_decode(engine, batch, steps, 4, ctx_len)
         gbs = decode_bytes(cfg, ctx_mid) / (dt / steps) / 1e9
-        out["decode"][str(ctx_len)] = {"tokens_per_s": round(batch * steps / dt, 1), "ms_per_step": round(dt / steps * 1e3, 3),
-                                       "gb_per_s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        out["decode"][str(ctx_len)] = {"batch": batch, "tokens_per_s": round(batch * steps / dt, 1),
+                                       "ms_per_step": round(dt / steps * 1e3, 3), "gb_per_s": round(gbs, 1),
+                                       "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        print(f"[bench] decode after {ctx_len} tokens x {batch}: {time.perf_counter() - t_in:.1f} s with the prompts",
+              file=sys.stderr, flush=True)
     g = torch.Generator().manual_seed(7)
-    for T in (8192, 16384):
+    for T in (8192, 16384, 32768):
         prompt = torch.randint(0, cfg.vocab_size, (T,), generator=g).tolist()
         best = None
         for i in range(3):
@@ -308,6 +325,38 @@ def long_contexts(a) -> int:
                 best = t if best is None else min(best, t)
         out["prefill"][str(T)] = {"tokens_per_s": round(T / best, 1), "ms": round(best * 1e3, 2),
                                   "frac": round(prefill_flops(cfg, T) / best / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    # a long prompt in portions beside decoding requests: eight requests decode (512 tokens of context each), then a
+    # prompt of 32,768 tokens arrives and goes in 8,192 tokens a step while they go on
+    cc = engine.cache.config
+    bc = BatchConfig(max_batch_size=9, max_prefill_tokens=8192, block_size=cc.page_size, num_blocks=cc.num_pages,
+                     max_tokens_per_step=8192 + 8)
+    rt = Runtime(engine, None, bc)
+    V = cfg.vocab_size
+    short = [rt.submit(torch.randint(0, V, (PROMPT_LEN,), generator=g).tolist(), GenerateOptions(max_new_tokens=64))
+             for _ in range(8)]
+    while any(s.phase != SequencePhase.DECODE for s in short):
+        rt.step()
+    for _ in range(4):
+        rt.step()
+    sync()
+    before = sum(len(s.generated_ids) + s.pending for s in short)
+    t0 = time.perf_counter()
+    big = rt.submit(torch.randint(0, V, (32768,), generator=g).tolist(), GenerateOptions(max_new_tokens=1))
+    steps = 0
+    while big.phase != SequencePhase.FINISHED and not big.generated_ids and big.pending == 0:
+        rt.step()
+        steps += 1
+    sync()
+    dt = time.perf_counter() - t0
+    decoded = sum(len(s.generated_ids) + s.pending for s in short) - before
+    flops = prefill_flops(cfg, 32768) + 2.0 * sum(matmul_params(cfg)) * decoded
+    out["prompt_beside_decoding"] = {"prompt_tokens": 32768, "portion": 8192, "steps": steps, "ms": round(dt * 1e3, 2),
+                                     "prompt_tokens_per_s": round(32768 / dt, 1), "decoded_meanwhile": decoded,
+                                     "ms_per_step": round(dt / max(steps, 1) * 1e3, 2),
+                                     "frac": round(flops / dt / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    for s in short + [big]:
+        rt.scheduler.cancel(s)
+    rt.run()
     print(json.dumps(out))
     return 0
 
@@ -323,8 +372,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the prefill of 2,048 tokens, a few times (for profiles); prints its record alone")
-    ap.add_argument("--shape", default="8b", choices=["8b", "13b"],
-                    help="8b: Llama-3.1-8B (the default, the headline); 13b: Llama-2-13B (40 key/value heads)")
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
+                    help="8b: Llama-3.1-8B (the default, the headline); 13b: Llama-2-13B (40 key/value heads); "
+                         "1b: Llama-3.2-1B (heads of 64, tied head)")
+    ap.add_argument("--points", default="1,64", help="batches of the further decode points, e.g. 1,64,128,256")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every request's prompt")
     ap.add_argument("--peaks", action="store_true",
                     help="only measure this GPU's streaming read bandwidth and bf16 matrix rate; a JSON line of its own")
@@ -356,14 +407,15 @@ def main() -> int:
     import torch
     from infernum_amd import CacheConfig, Engine, LlamaConfig
 
-    raw = dict(LLAMA_8B if a.shape == "8b" else LLAMA_13B)
+    raw = dict(SHAPES[a.shape][0])
+    point_batches = [int(b) for b in a.points.split(",") if b] if not a.no_points else []
     full_layers = raw["num_hidden_layers"]
     if a.layers:
         raw["num_hidden_layers"] = a.layers
     cfg = LlamaConfig.from_dict(raw)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
-    max_batch = 1 if a.prefill_only else max(a.batch, 1 if a.no_points else 64)
+    max_batch = 1 if a.prefill_only else max([a.batch] + point_batches)
     tokens_needed = max(max_batch * (a.prompt_len + a.steps + a.warmup + prefill_steps(max_batch, a.prompt_len)
                                      + 2 * PAGE_SIZE), PREFILL_TOKENS + PAGE_SIZE)
     t_load = time.perf_counter()
@@ -387,16 +439,16 @@ def main() -> int:
     value = a.batch * a.steps / dt
     achieved = decode_bytes(cfg, ctx_mid, elem) / (dt / a.steps) / 1e9
     out = {
-        "metric": f"decode tok/s @ batch {a.batch}, {'Llama-3-8B' if a.shape == '8b' else 'Llama-2-13B'} shape", "value": round(value, 2), "unit": "tokens/s",
+        "metric": f"decode tok/s @ batch {a.batch}, {SHAPES[a.shape][1]} shape", "value": round(value, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
         "config": {
-            "model": "llama-3.1-8b-shape-random" if a.shape == "8b" else "llama-2-13b-shape-random", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
+            "model": SHAPES[a.shape][2], "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
             "hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads, "num_kv_heads": cfg.num_kv_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LEN, "page_size": PAGE_SIZE,
             "parallelism": "none", "sampling": "greedy", "gemm_route": gemm_route,
-            "rope": "llama3(8,1,4,8192) theta 5e5" if a.shape == "8b" else "theta 1e4",
+            "rope": SHAPES[a.shape][3],
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -404,10 +456,12 @@ def main() -> int:
 
     if not a.no_points:
         points = {}
-        for b in (1, 64):
+        for b in point_batches:
             steps = max(16, min(a.steps, 64))
-            d, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)), a.prompt_len)
+            d, ctx_b = time_decode(engine, b, steps, max(4, min(a.warmup, 8)), a.prompt_len)
             points[f"decode_b{b}"] = round(b * steps / d, 2)
+            if b > 64:          # the further points carry their place against the roofline with them
+                points[f"decode_b{b}_hbm_frac"] = round(decode_bytes(cfg, ctx_b, elem) / (d / steps) / 1e9 / HBM_PEAK_GBS, 4)
         out["points"] = points
         out["prefill"] = time_prefill(engine, cfg, a.dtype)
         # the same fractions against what a bare stream of loads and a bare chain of matrix instructions reach here
