@@ -361,6 +361,56 @@ def long_contexts(a) -> int:
     return 0
 
 
+def decode_kernels_alone(a) -> int:
+    """The two kernels that a decode step of the 8B shape spends its time in, alone, on operands of the step's
+    sizes at batch 8 (what is in the operands does not change what the kernels do): the weight-streaming product
+    with each of a layer's four weights (the gate+up matrix in the layout made for it), and the attention over
+    527 cached tokens with the rotation and the write of the token's key and value inside.  For hardware counters
+    (``rocprofv3 --pmc ... -- python3 bench.py --decode-kernels``): nothing else runs on the GPU, no library kernel
+    either (the operands are uninitialised memory; tables and positions come from the host by copies)."""
+    import math
+    import torch
+    from infernum_amd.kernels import api as K
+    cfg = dict(LLAMA_8B)
+    H, I, nh, nkv = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d, B, ctx, dev = H // nh, a.batch, PROMPT_LEN + 15, "cuda:0"
+    bf = dict(dtype=torch.bfloat16, device=dev)
+    weights = [("qkv", (nh + 2 * nkv) * d, H, None), ("o", H, nh * d, None), ("gate_up", 2 * I, H, "swiglu"), ("down", H, I, None)]
+    x = {Kd: torch.empty((B, Kd), **bf) for _, _, Kd, _ in weights}
+    pages_per = -(-(ctx + 1) // PAGE_SIZE)
+    kp = torch.empty((B * pages_per, nkv, PAGE_SIZE, d), **bf)
+    vp = torch.empty((B * pages_per, nkv, d, PAGE_SIZE), **bf)
+    bt = torch.arange(B * pages_per, dtype=torch.int32).reshape(B, pages_per).to(dev)
+    pos = torch.full((B,), ctx, dtype=torch.int32).to(dev)
+    slots = (torch.arange(B, dtype=torch.int32) * pages_per * PAGE_SIZE + ctx).to(dev)
+    inv_freq = (500000.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)).to(dev)
+    out = torch.empty((B, nh * d), **bf)
+    times = {}
+    for name, N, Kd, epilogue in weights:
+        w = torch.empty((N, Kd), **bf)
+        tiled = K.tile_weight(w, epilogue) if K.gemm_skinny_splits(N, Kd) == 1 else None
+        for _ in range(a.warmup):
+            K.gemm_skinny(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None, tiled=tiled)
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            y = K.gemm_skinny(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None, tiled=tiled)
+        sync()
+        times[name] = round((time.perf_counter() - t0) / a.steps * 1e6, 1)
+        if name == "qkv":
+            qkv = y                      # the partial sums of the QKV product: what the attention kernel reads
+    for i in range(a.warmup + a.steps):
+        if i == a.warmup:
+            sync()
+            t0 = time.perf_counter()
+        K.attention_decode_rotating(qkv, pos, inv_freq, d, slots, kp, vp, out, bt, nh, nkv, d, 1.0 / math.sqrt(d), 0, ctx + 1)
+    sync()
+    times["attention"] = round((time.perf_counter() - t0) / a.steps * 1e6, 1)
+    print(json.dumps({"metric": "decode kernels alone, Llama-3-8B shape", "batch": B, "context": ctx,
+                      "us_per_call_from_the_host": times}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -382,6 +432,8 @@ def main() -> int:
     ap.add_argument("--long", action="store_true",
                     help="decode at 16k and 32k tokens of context and prefills of 8k and 16k tokens instead (a JSON line of its own)")
     ap.add_argument("--no-fp32-check", action="store_true", help="skip the comparison with the 32-bit path")
+    ap.add_argument("--decode-kernels", action="store_true",
+                    help="only the decode step's two kernels on operands of the 8B shape (for hardware counters)")
     ap.add_argument("--serve", action="store_true",
                     help="continuous batching of 128 requests on the 1B shape instead (a JSON line of its own)")
     ap.add_argument("--serve-requests", type=int, default=128)
@@ -396,6 +448,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
         return 2
 
+    if a.decode_kernels:
+        return decode_kernels_alone(a)
     if a.serve:
         return serve(a)
     if a.long:
