@@ -13,7 +13,6 @@ int32 buffer, copies it to the device once, and runs the model's forward pass.
 """
 from __future__ import annotations
 
-import os
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
@@ -79,7 +78,7 @@ class Engine:
         # model's parts wrote (engine/program.py; a part without launchers of its own is called back); "parts":
         # by the parts' own forward, one Python call per launch (the twin that tests hold the program to, and
         # the way of INFERNUM_PROFILE=1).  The same launches either way.
-        executor = executor or os.environ.get("INFERNUM_EXECUTOR", "native")
+        executor = executor or "native"
         if executor not in ("native", "parts"):
             raise ValueError(f"executor must be 'native' or 'parts', got {executor!r}")
         self.program = None

@@ -76,8 +76,7 @@ class Runtime:
         # host reads a step's tokens while the next step runs.  Needs an engine that takes tokens from the device
         # and a sampler that leaves them there; requests whose choice looks at their own history (a repetition
         # penalty) are served one step at a time.
-        self.look_ahead = (os.environ.get("INFERNUM_LOOK_AHEAD", "1") != "0"
-                           and getattr(engine, "supports_device_tokens", False)
+        self.look_ahead = (getattr(engine, "supports_device_tokens", False)
                            and hasattr(self.sampler, "select_on_device") and hasattr(self.sampler, "needs_history"))
         self._inflight = None                 # (plan, tokens on the device, row of each request, download)
         self._download = None

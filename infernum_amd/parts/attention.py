@@ -16,7 +16,6 @@ infernum-cuda/src/inner/weights/generic_impl.rs:153-180).
 from __future__ import annotations
 
 import math
-import os
 from typing import Any, Dict, Mapping, Optional
 
 import torch
@@ -32,9 +31,7 @@ from .linear import emit_linear, linear, prepare_weights
 # with the rotation, and with many of them that costs more than the one launch it saves).
 ROTATE_IN_ATTENTION_UP_TO = 64
 DECODE_ROTATIONS = ("attention", "separate")
-_decode_rotation = os.environ.get("INFERNUM_DECODE_ROTATE", "attention")
-if _decode_rotation not in DECODE_ROTATIONS:
-    raise ValueError(f"INFERNUM_DECODE_ROTATE={_decode_rotation!r}: one of {DECODE_ROTATIONS}")
+_decode_rotation = "attention"
 
 
 def set_decode_rotation(name: str) -> str:
