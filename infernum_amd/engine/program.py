@@ -34,6 +34,7 @@ _ARG_CONST, _ARG_VAR, _ARG_PTR, _ARG_STREAM = 0, 1, 2, 3
 _TERM_RANGE, _TERM_BLOCKS = 0, 1
 ALL_BLOCKS = 0x1FF          # bits 0..7: 1-16, 17-32, ... 113-128 rows; bit 8: more than 128
 PYTHON_FAILED = 10007
+_GUARD, _GUARD_BYTE = 256, 0xA5
 
 
 class ProgramError(K.KernelError):
@@ -427,12 +428,17 @@ class StepProgram:
     # ---- finishing ---------------------------------------------------------------------------
     def finish(self) -> None:
         self._not_finished()
+        # buffers one after the other, each followed by a guard of 256 bytes that holds a pattern: a launch that
+        # writes past its buffer's end writes into the guard first (``check_guards``; tests look after their steps)
         at = 0
         for b in self._buffers.values():
             b.offset = at
-            at += (b.nbytes + 255) & ~255
+            at += ((b.nbytes + 255) & ~255) + _GUARD
         self.arena_bytes = at
         self._arena = torch.empty(max(at, 256), dtype=torch.uint8, device=self.rt.device)
+        for b in self._buffers.values():
+            end = b.offset + ((b.nbytes + 255) & ~255)
+            self._arena[end:end + _GUARD].fill_(_GUARD_BYTE)
         add = self._lib.ia_program_add_op
         for fn, name, args, when, if_unsupported in self._ops:
             flat: List[int] = []
@@ -513,6 +519,13 @@ class StepProgram:
     def step_logits(self) -> torch.Tensor:
         """(Inside a Python operation.)  The logits [wanted rows, vocabulary] that the running step returns."""
         return self._logits
+
+    def check_guards(self) -> None:
+        """Raises when something wrote past the end of one of the program's buffers."""
+        for b in self._buffers.values():
+            end = b.offset + ((b.nbytes + 255) & ~255)
+            if not bool((self._arena[end:end + _GUARD] == _GUARD_BYTE).all()):
+                raise ProgramError(f"something wrote past the end of buffer {b.key!r} ({b.nbytes} bytes)")
 
     def last_launches(self) -> int:
         return int(self._lib.ia_program_last_launches(self._h))

@@ -305,7 +305,45 @@ def test_native_program_makes_the_launches_of_the_parts(models, name, dtype):
         assert a.keys() == b.keys()
         for k in a:
             assert torch.equal(a[k], b[k]), k
+        native.program.check_guards()              # no launch wrote past the end of its intermediate
     for kernels in ("generic",):
         a = TT.run_steps(_engine(d, dtype, PAGE[name], 64, kernels=kernels), TT.trace_portions(reqs))
         b = TT.run_steps(_engine(d, dtype, PAGE[name], 64, kernels=kernels, executor="parts"), TT.trace_portions(reqs))
         assert all(torch.equal(a[k], b[k]) for k in a)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("limit", [7, 64, 129, 300])
+def test_intermediates_of_the_program_are_large_enough_for_steps_of_every_shape(models, dtype, limit):
+    """An engine whose steps take at most ``limit`` tokens has intermediates for exactly that many: steps that fill
+    the limit (one long portion; single tokens only; both) leave the guards behind every intermediate untouched and
+    give the bits of the parts' own forward."""
+    from infernum_amd import CacheConfig, Engine, StepEntry
+    d, cfg, reqs, ref = models[("C", dtype, "mixed")]
+    V = cfg["vocab_size"]
+    engines = [Engine.from_pretrained(d, dtype=dtype, max_tokens_per_step=limit, executor=ex, use_graphs=False,
+                                      cache_config=CacheConfig(page_size=8, num_pages=limit + 40, num_state_slots=limit + 2))
+               for ex in ("native", "parts")]
+    g = torch.Generator().manual_seed(limit)
+    toks = lambda n: torch.randint(0, V, (n,), generator=g).tolist()
+    singles = min(limit, 90)
+    steps = [[StepEntry("long", toks(limit), [0, limit - 1])],
+             [StepEntry(("s", i), toks(1), [0]) for i in range(singles)],
+             [StepEntry(("s", i), toks(1), [0]) for i in range(singles)]]
+    if limit > 3:
+        half = limit // 2
+        steps.append([StepEntry(("s", i), toks(1), [0]) for i in range(min(half, singles))] +
+                     [StepEntry("other", toks(limit - min(half, singles)), [])])
+    outs = []
+    for eng in engines:
+        res = []
+        for entries in steps:
+            res.append(eng.step(entries).cpu())
+            if entries[0].request == "long":
+                eng.end("long")
+        outs.append(res)
+    engines[0].program.check_guards()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with pytest.raises(Exception):
+        engines[0].step([StepEntry("too long", toks(limit + 1), [])])

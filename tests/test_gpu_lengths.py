@@ -105,6 +105,7 @@ def test_long_prompts_whole_in_portions_and_with_a_decoded_tail(name, dtype, tmp
             assert worst == worst and worst <= TOL[dtype] * rms, line
             print(line)
     eng.cache.check()
+    eng.program.check_guards()
     assert all(g.allocator.num_free == g.allocator.num_pages for g in eng.cache.groups)
     if name == "E" and dtype == "bfloat16":
         from infernum_amd.kernels import api

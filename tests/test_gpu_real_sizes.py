@@ -110,4 +110,5 @@ def test_all_ways_of_cutting_at_real_sizes(real, dtype):
             assert to_exact <= 1.1 * ebf_rms and to_rounding <= 1.2 * ebf_rms, line
         print(line)
     eng.cache.check()
+    eng.program.check_guards()
     assert all(g.allocator.num_free == g.allocator.num_pages for g in eng.cache.groups)
