@@ -105,7 +105,16 @@ class Attention(Mixer):
         return own
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
+        wq, wk = tensors["q_proj.weight"], tensors["k_proj.weight"]
+        perm = self.position.head_permutation()
+        if perm is not None:
+            # the position encoding's own order of a head's values (see PositionEncoding.head_permutation)
+            perm = perm.to(wq.device).long()
+            if sorted(perm.tolist()) != list(range(self.d)):
+                raise ValueError("the position encoding's head_permutation is no permutation of a head's values")
+            wq = wq.view(self.nh, self.d, -1)[:, perm].reshape(wq.shape)
+            wk = wk.view(self.nkv, self.d, -1)[:, perm].reshape(wk.shape)
+        self.w_qkv = torch.cat([wq, wk, tensors["v_proj.weight"]], dim=0)
         self.w_qkv = self.w_qkv.contiguous()
         self.w_o = tensors["o_proj.weight"].contiguous()
         prepare_weights(self.rt, [(self.w_qkv, None, True), (self.w_qkv[: self.nh * self.d], None, True),

@@ -298,7 +298,21 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    """Owns what the rotation kernel needs: ``inv_freq`` (float64 or fp32 [rotary_dim / 2] on the device, or None
+    for no rotation) and ``rotary_dim``.  The kernels pair the first half of a head's rotated values with the
+    second, (x[i], x[i + rotary_dim / 2]); an encoding that pairs other values gives the order in which it wants
+    a head's values through ``head_permutation``."""
+
     category = "position"
+
+    def head_permutation(self) -> Optional[torch.Tensor]:
+        """None, or a permutation p of range(head_dim) (int64, on any device): the attention mixer then keeps its
+        query and key projections with the rows of every head in the order p, so that value p[j] of the
+        encoding's own order stands at place j.  Scores are sums over a head's values and do not care about their
+        order, as long as queries and keys share it; an encoding that rotates neighbouring pairs
+        (x[2i], x[2i + 1]) asks for [0, 2, 4, ..., 1, 3, 5, ...] and is then served by the kernels' half-split
+        pairs.  (A ``qk_transform`` sees the heads in the permuted order.)"""
+        return None
 
 
 class QKTransform(Part):

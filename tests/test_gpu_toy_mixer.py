@@ -876,3 +876,101 @@ def test_two_cached_parts_side_by_side_in_one_layer(tmp_path, dtype):
         assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
         eng.cache.check()
         assert eng.cache.slots.num_free == 4 and all(g.allocator.num_free == 48 for g in eng.cache.groups)
+
+
+# ------------------------------------------------------------------------------------------------
+# A position encoding that rotates neighbouring pairs (x[2i], x[2i + 1]) where the kernels pair the halves of a
+# head: it asks the attention for its heads' values in the order [0, 2, 4, ..., 1, 3, 5, ...] and is then served
+# by the stock kernels.
+class NeighbourPairsRope(PositionEncoding):
+    graph_safe = True
+
+    def __init__(self, rt, head_dim, theta):
+        super().__init__(rt)
+        self.rotary_dim = head_dim
+        self.inv_freq = (float(theta) ** (-torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim)).to(rt.device)
+
+    def head_permutation(self):
+        return torch.cat([torch.arange(0, self.rotary_dim, 2), torch.arange(1, self.rotary_dim, 2)])
+
+
+def _rope_neighbours(x, positions, freqs):
+    """x [T, heads, d]: out[2i] = x[2i] cos a - x[2i+1] sin a; out[2i+1] = x[2i] sin a + x[2i+1] cos a, a = p f_i."""
+    ang = positions.to(freqs.dtype)[:, None] * freqs[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[..., 0::2], x[..., 1::2]
+    out = torch.empty_like(x)
+    out[..., 0::2] = a * cos - b * sin
+    out[..., 1::2] = a * sin + b * cos
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_position_encoding_that_pairs_neighbours(tmp_path, dtype):
+    register_part("position", "neighbour_pairs", NeighbourPairsRope, replace=True)
+    H, nh, nkv, d, V, I = 64, 4, 2, 16, 80, 96
+
+    @dataclass(frozen=True)
+    class Toy7Config:
+        model_type: str = "toy-neighbours"
+
+        @staticmethod
+        def from_dict(raw, where="config.json"):
+            return Toy7Config()
+
+        def to_dict(self):
+            return {"model_type": self.model_type}
+
+    def spec(cfg):
+        norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "init": ("uniform", 0.5, 1.5)}, prefix)
+        layers = [LayerSpec("prenorm",
+                            PartSpec("attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                   "init_std": 0.15, "position": {"kind": "neighbour_pairs", "params": {
+                                                       "head_dim": d, "theta": 100.0}}}, f"l.{i}.attn."),
+                            PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I, "init_std": 0.1}, f"l.{i}.ff."),
+                            norm(f"l.{i}.n1."), norm(f"l.{i}.n2.")) for i in range(2)]
+        return ModelSpec(vocab_size=V, hidden_size=H,
+                         embedding=PartSpec("token", {"vocab_size": V, "hidden_size": H, "init_std": 0.5}, "emb."),
+                         layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn."),
+                         head=PartSpec("linear", {"vocab_size": V, "hidden_size": H, "init_std": 0.1}, "head."))
+
+    register_architecture("toy-neighbours", Toy7Config, spec, replace=True)
+    folder = write_random_model(Toy7Config(), str(tmp_path / "toy7"), seed=51,
+                                dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    _, w = P.read_model(folder)
+
+    def plain(ids):
+        W = {k: v.double() for k, v in w.items()}
+        T = len(ids)
+        freqs, pos = 100.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d), torch.arange(T)
+        h = P.embedding(W["emb.weight"], ids)
+        for l in range(2):
+            n = P.rms_norm(h, W[f"l.{l}.n1.weight"], 1e-5)
+            p = f"l.{l}.attn."
+            q = _rope_neighbours(P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d), pos, freqs)
+            k = _rope_neighbours(P.linear(n, W[p + "k_proj.weight"]).reshape(T, nkv, d), pos, freqs)
+            v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, nkv, d)
+            h = h + P.linear(P.causal_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, nh * d), W[p + "o_proj.weight"])
+            m = P.rms_norm(h, W[f"l.{l}.n2.weight"], 1e-5)
+            h = h + P.linear(P.swiglu(P.linear(m, W[f"l.{l}.ff.gate_proj.weight"]), P.linear(m, W[f"l.{l}.ff.up_proj.weight"])),
+                             W[f"l.{l}.ff.down_proj.weight"])
+        return P.linear(P.rms_norm(h, W["fn.weight"], 1e-5), W["head.weight"])
+
+    # the pairing matters: the stock half-split rotation of the same weights gives other logits
+    ids = [3, 9, 27, 1, 60, 44, 12]
+    halves = P.rope(torch.ones(7, 1, d, dtype=torch.float64), torch.arange(7), 100.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d))
+    assert not torch.allclose(halves, _rope_neighbours(torch.ones(7, 1, d, dtype=torch.float64), torch.arange(7),
+                                                       100.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)))
+    eng = Engine.from_pretrained(folder, dtype=dtype, cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4,
+                                                                               poison_freed_pages=True))
+    assert eng.use_graphs                                  # nothing of the model's own runs on the host
+    reqs = TT.make_requests(V, (33, 6, 41, 20), seed=9)
+    ref = {r: plain(t) for r, t in reqs.items()}
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r: max(2, len(t) - 8) for r, t in reqs.items()}, seed=5)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy7 {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
