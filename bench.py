@@ -200,10 +200,21 @@ LLAMA_1B = dict(
 )
 
 
+LLAMA_70B = dict(
+    model_type="llama", num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8,
+    intermediate_size=28672, vocab_size=128256, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+    max_position_embeddings=131072,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+
+
 SHAPES = {
     "8b": (LLAMA_8B, "Llama-3-8B", "llama-3.1-8b-shape-random", "llama3(8,1,4,8192) theta 5e5"),
     "13b": (LLAMA_13B, "Llama-2-13B", "llama-2-13b-shape-random", "theta 1e4"),
     "1b": (LLAMA_1B, "Llama-3.2-1B", "llama-3.2-1b-shape-random", "llama3(32,1,4,8192) theta 5e5"),
+    # 141 GB of weights in bf16 and 77 GB of second copies of the wide ones: one GPU's memory holds them
+    "70b": (LLAMA_70B, "Llama-3.1-70B", "llama-3.1-70b-shape-random", "llama3(8,1,4,8192) theta 5e5"),
 }
 
 
@@ -424,7 +435,8 @@ def main() -> int:
                     help="only the prefill of 2,048 tokens, a few times (for profiles); prints its record alone")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
                     help="8b: Llama-3.1-8B (the default, the headline); 13b: Llama-2-13B (40 key/value heads); "
-                         "1b: Llama-3.2-1B (heads of 64, tied head)")
+                         "1b: Llama-3.2-1B (heads of 64, tied head); 70b: Llama-3.1-70B (all 80 layers on the one GPU; give "
+                         "--no-fp32-check, the 32-bit twin does not fit beside it)")
     ap.add_argument("--points", default="1,64", help="batches of the further decode points, e.g. 1,64,128,256")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every request's prompt")
     ap.add_argument("--peaks", action="store_true",

@@ -263,13 +263,16 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
     }
   }
 
+  // the start of the request's block table is asked for together with its position, not after it: a request of
+  // up to NT pages (all but the longest) then knows its pages one trip to memory earlier
+  const int* bt = block_tables + (size_t)b * bt_stride;
+  const int bt_ahead = tid < bt_stride ? bt[tid] : -1;
   const int p = positions[b];
   const int lo0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int t_first = lo0 / 16, t_last = p / 16;
   const int per = (t_last - t_first + 1 + num_splits - 1) / num_splits;
   const int ta = t_first + split * per;
   const int tb = (ta + per < t_last + 1) ? ta + per : t_last + 1;
-  const int* bt = block_tables + (size_t)b * bt_stride;
 
   DecGeom geo;
   geo.ps = ps;
@@ -294,7 +297,11 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
     if (count > DEC_BT_LDS) count = DEC_BT_LDS;
     geo.bt_first = first;
     geo.bt_count = count;
-    for (int i = tid; i < count; i += NT) s_bt[i] = bt[first + i];
+    if (first + count <= NT) {
+      if (tid >= first && tid < first + count) s_bt[tid - first] = bt_ahead;
+    } else {
+      for (int i = tid; i < count; i += NT) s_bt[i] = bt[first + i];
+    }
   }
   const int pos = col_ok ? p : -1;
   f32x4 o[NS];

@@ -1,6 +1,6 @@
 """The engine against the plain implementation at the layer sizes of Llama-3.1-8B (width 4,096, 32 heads on 8
-key/value heads of 128, feed-forward width 14,336, the vocabulary of 128,256; two layers), and of the 13B and 1B
-shapes that the benchmarks also run, under all four ways of cutting, in 32-bit and in bfloat16.
+key/value heads of 128, feed-forward width 14,336, the vocabulary of 128,256; two layers), and of the 13B, 1B and
+70B shapes that the benchmarks also run, under all four ways of cutting, in 32-bit and in bfloat16.
 
 The tiny configurations cannot show what only these sizes have: inner dimensions of 4,096 and 14,336 split over
 workgroups and joined by the next kernel, four heads of 128 to a workgroup, a head of 128,256 rows.  Their
@@ -43,6 +43,11 @@ SHAPES = {
            "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
            "rope_theta": 500000.0, "max_position_embeddings": 131072, "rms_norm_eps": 1e-5,
            "tie_word_embeddings": True, "rope_scaling": dict(_LLAMA3, factor=32.0)},
+    # one layer of the 70B shape: widths 8,192 and 28,672 (112 chunks of 256 in the down projection), eight query heads
+    # to a key/value head, products whose rows go to the library from 17 on by the table; a short vocabulary again
+    "70b": {"model_type": "llama", "vocab_size": 16001, "hidden_size": 8192, "intermediate_size": 28672,
+            "num_hidden_layers": 1, "num_attention_heads": 64, "num_key_value_heads": 8, "rope_theta": 500000.0,
+            "max_position_embeddings": 131072, "rms_norm_eps": 1e-5, "rope_scaling": dict(_LLAMA3, factor=8.0)},
 }
 LENGTHS = (200, 61, 130)
 
