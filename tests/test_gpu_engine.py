@@ -300,6 +300,7 @@ def test_native_program_makes_the_launches_of_the_parts(models, name, dtype):
     parts = _engine(d, dtype, PAGE[name], max_tokens // PAGE[name], executor="parts")
     assert native.program is not None and parts.program is None
     assert native.program.num_ops >= 9 * cfg["num_hidden_layers"]      # norm, product, rotation, attention, product; norm, two products (three with the activation)
+    assert native.program.num_python_ops == 0                              # nothing of a Llama step is a call into Python
     for steps in traces:
         a, b = TT.run_steps(native, steps), TT.run_steps(parts, steps)
         assert a.keys() == b.keys()

@@ -176,7 +176,7 @@ def test_toy_model_is_registered_built_loaded_and_stepped(toy, dtype):
         assert eng.cache.slots.num_free == 4 and all(g.allocator.num_free == 48 for g in eng.cache.groups)
     # the step ran as one program: the stock parts' launches made by the host library, the mixer of this file
     # called back in its place among them; the parts' own forward, call by call from Python, gives the same bits
-    assert eng.program is not None and eng.program.num_ops > 30
+    assert eng.program is not None and eng.program.num_ops > 30 and eng.program.num_python_ops > 0
     twin = Engine.from_pretrained(d, dtype=dtype, executor="parts",
                                   cache_config=CacheConfig(page_size=4, num_pages=48, num_state_slots=4))
     assert twin.program is None
@@ -974,3 +974,105 @@ def test_a_position_encoding_that_pairs_neighbours(tmp_path, dtype):
         worst, rms, where = TT.error_against(got, ref)
         print(f"toy7 {dtype} {name}: {worst / rms:.2e} at {where}")
         assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+
+
+# ------------------------------------------------------------------------------------------------
+# A feed-forward of the test's own that writes its own launches into the step's program (two products through a
+# narrow middle, y = W_out (W_in x), no activation), so that no operation of the program calls back into Python:
+# the part uses the framework's products and intermediates, and nothing under the framework's folders changes.
+class BottleneckFeedForward(FeedForward):
+    graph_safe = True
+
+    def __init__(self, rt, hidden_size, rank):
+        super().__init__(rt)
+        self.H, self.r = hidden_size, rank
+
+    def weights(self):
+        return {"in.weight": WeightSpec((self.r, self.H), ("normal", 0.2)),
+                "out.weight": WeightSpec((self.H, self.r), ("normal", 0.2))}
+
+    def load(self, tensors):
+        self.w_in, self.w_out = tensors["in.weight"].contiguous(), tensors["out.weight"].contiguous()
+
+    def forward(self, x, ctx=None):
+        from infernum_amd.parts.linear import linear
+        return linear(linear(x, self.w_in, kernels=self.rt.kernels), self.w_out, keep_split=True, kernels=self.rt.kernels)
+
+    def native(self, program, view=None):
+        from infernum_amd.parts.linear import emit_linear
+        dt = self.rt.dtype
+        mid = emit_linear(program, program.x, program.N, self.w_in, dt, None, False, "bottleneck.mid", "bottleneck.in")
+        program.pending = emit_linear(program, mid.tensor(), program.N, self.w_out, dt, None, True, "bottleneck.out",
+                                      "bottleneck.out")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_feed_forward_that_writes_its_own_launches(tmp_path, dtype):
+    register_part("feed_forward", "bottleneck", BottleneckFeedForward, replace=True)
+    H, nh, nkv, d, V, r = 80, 5, 5, 16, 90, 24
+
+    @dataclass(frozen=True)
+    class Toy8Config:
+        model_type: str = "toy-bottleneck"
+
+        @staticmethod
+        def from_dict(raw, where="config.json"):
+            return Toy8Config()
+
+        def to_dict(self):
+            return {"model_type": self.model_type}
+
+    def spec(cfg):
+        norm = lambda prefix: PartSpec("rmsnorm", {"size": H, "eps": 1e-6, "init": ("uniform", 0.5, 1.5)}, prefix)
+        layers = [LayerSpec("prenorm",
+                            PartSpec("attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                   "init_std": 0.15, "position": {"kind": "rope", "params": {
+                                                       "head_dim": d, "theta": 1000.0}}}, f"l.{i}.attn."),
+                            PartSpec("bottleneck", {"hidden_size": H, "rank": r}, f"l.{i}.ff."),
+                            norm(f"l.{i}.n1."), norm(f"l.{i}.n2.")) for i in range(3)]
+        return ModelSpec(vocab_size=V, hidden_size=H,
+                         embedding=PartSpec("token", {"vocab_size": V, "hidden_size": H, "init_std": 0.5}, "emb."),
+                         layers=layers, schedule=[ScheduleEntry(i) for i in range(3)], final_norm=norm("fn."),
+                         head=PartSpec("linear", {"vocab_size": V, "hidden_size": H, "init_std": 0.1}, "head."))
+
+    register_architecture("toy-bottleneck", Toy8Config, spec, replace=True)
+    folder = write_random_model(Toy8Config(), str(tmp_path / "toy8"), seed=77,
+                                dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    _, w = P.read_model(folder)
+
+    def plain(ids):
+        W = {k: v.double() for k, v in w.items()}
+        T = len(ids)
+        freqs, pos = 1000.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d), torch.arange(T)
+        h = P.embedding(W["emb.weight"], ids)
+        for l in range(3):
+            n = P.rms_norm(h, W[f"l.{l}.n1.weight"], 1e-6)
+            p = f"l.{l}.attn."
+            q = P.rope(P.linear(n, W[p + "q_proj.weight"]).reshape(T, nh, d), pos, freqs)
+            k = P.rope(P.linear(n, W[p + "k_proj.weight"]).reshape(T, nkv, d), pos, freqs)
+            v = P.linear(n, W[p + "v_proj.weight"]).reshape(T, nkv, d)
+            h = h + P.linear(P.causal_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, nh * d), W[p + "o_proj.weight"])
+            m = P.rms_norm(h, W[f"l.{l}.n2.weight"], 1e-6)
+            h = h + P.linear(P.linear(m, W[f"l.{l}.ff.in.weight"]), W[f"l.{l}.ff.out.weight"])
+        return P.linear(P.rms_norm(h, W["fn.weight"], 1e-6), W["head.weight"])
+
+    cache = lambda: CacheConfig(page_size=4, num_pages=48, num_state_slots=4, poison_freed_pages=True)
+    eng = Engine.from_pretrained(folder, dtype=dtype, cache_config=cache())
+    # the whole step is launched by the host library: no operation of the program is a call into Python
+    assert eng.program is not None and eng.program.num_python_ops == 0 and eng.use_graphs
+    twin = Engine.from_pretrained(folder, dtype=dtype, cache_config=cache(), executor="parts")
+    assert twin.program is None
+    reqs = TT.make_requests(V, (29, 7, 38, 18), seed=12)
+    ref = {r_: plain(t) for r_, t in reqs.items()}
+    tol = {"float32": 3e-5, "bfloat16": 8e-2}[dtype]
+    for name, steps in (("whole", TT.trace_whole(reqs)), ("tail", TT.trace_tail_one_by_one(reqs, 12)),
+                        ("portions", TT.trace_portions(reqs)),
+                        ("mixed", TT.trace_mixed(reqs, {r_: max(2, len(t) - 8) for r_, t in reqs.items()}, seed=8)[0])):
+        got = TT.run_steps(eng, steps)
+        worst, rms, where = TT.error_against(got, ref)
+        print(f"toy8 {dtype} {name}: {worst / rms:.2e} at {where}")
+        assert worst == worst and worst <= tol * rms, (name, worst / rms, where)
+        # the part's own launches make the bits of its forward
+        by_parts = TT.run_steps(twin, steps)
+        assert all(torch.equal(got[key], by_parts[key]) for key in got), name
+    eng.program.check_guards()
