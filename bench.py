@@ -339,8 +339,10 @@ def long_contexts(a) -> int:
     # a long prompt in portions beside decoding requests: eight requests decode (512 tokens of context each), then a
     # prompt of 32,768 tokens arrives and goes in 8,192 tokens a step while they go on
     cc = engine.cache.config
+    # (a step holds 8,192 tokens with the decoded ones: the library's products lose a third to half of their rate at
+    # 8,200 rows, which fill one tile of 256 more than two rounds of workgroups hold)
     bc = BatchConfig(max_batch_size=9, max_prefill_tokens=8192, block_size=cc.page_size, num_blocks=cc.num_pages,
-                     max_tokens_per_step=8192 + 8)
+                     max_tokens_per_step=8192)
     rt = Runtime(engine, None, bc)
     V = cfg.vocab_size
     short = [rt.submit(torch.randint(0, V, (PROMPT_LEN,), generator=g).tolist(), GenerateOptions(max_new_tokens=64))
@@ -349,19 +351,24 @@ def long_contexts(a) -> int:
         rt.step()
     for _ in range(4):
         rt.step()
-    sync()
-    before = sum(len(s.generated_ids) + s.pending for s in short)
-    t0 = time.perf_counter()
-    big = rt.submit(torch.randint(0, V, (32768,), generator=g).tolist(), GenerateOptions(max_new_tokens=1))
-    steps = 0
-    while big.phase != SequencePhase.FINISHED and not big.generated_ids and big.pending == 0:
-        rt.step()
-        steps += 1
-    sync()
-    dt = time.perf_counter() - t0
+    big_prompt = torch.randint(0, V, (32768,), generator=g).tolist()
+    for attempt in range(2):          # the second time is the one that counts: the first also loads the library's kernels for these rows
+        sync()
+        before = sum(len(s.generated_ids) + s.pending for s in short)
+        t0 = time.perf_counter()
+        big = rt.submit(big_prompt, GenerateOptions(max_new_tokens=1))
+        steps = 0
+        while big.phase != SequencePhase.FINISHED and not big.generated_ids and big.pending == 0:
+            rt.step()
+            steps += 1
+        sync()
+        dt = time.perf_counter() - t0
+        if attempt == 0:
+            rt.scheduler.cancel(big)
+            rt.step()
     decoded = sum(len(s.generated_ids) + s.pending for s in short) - before
     flops = prefill_flops(cfg, 32768) + 2.0 * sum(matmul_params(cfg)) * decoded
-    out["prompt_beside_decoding"] = {"prompt_tokens": 32768, "portion": 8192, "steps": steps, "ms": round(dt * 1e3, 2),
+    out["prompt_beside_decoding"] = {"prompt_tokens": 32768, "tokens_a_step": 8192, "steps": steps, "ms": round(dt * 1e3, 2),
                                      "prompt_tokens_per_s": round(32768 / dt, 1), "decoded_meanwhile": decoded,
                                      "ms_per_step": round(dt / max(steps, 1) * 1e3, 2),
                                      "frac": round(flops / dt / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
