@@ -105,6 +105,17 @@ def tiled_copy(w: torch.Tensor, epilogue: Optional[str]) -> Optional[torch.Tenso
     return made.get(epilogue) if made else None
 
 
+COPIES_LEAVE_FREE = 0.15      # of the device's memory: second copies are made only while this much stays free
+
+
+def _room_for_copy(w: torch.Tensor) -> bool:
+    """Whether a second copy of ``w`` still leaves COPIES_LEAVE_FREE of the device's memory free (for the cache and
+    the steps' intermediates): a model that fills the memory keeps the file's layout for the rest of its weights
+    (the same bits, a few per cent slower), where copies of all would leave no room for the cache."""
+    free, total = torch.cuda.mem_get_info(w.device)
+    return free - w.numel() * w.element_size() >= COPIES_LEAVE_FREE * total
+
+
 def prepare_weights(rt, uses) -> None:
     """``uses``: (weight, epilogue, keep_split) of a part that has just been loaded.  On a GPU, in bfloat16 with the
     fast kernels: a weight with so many rows that the weight-streaming kernel gives every workgroup all of K (no
@@ -113,8 +124,9 @@ def prepare_weights(rt, uses) -> None:
     (``kernels.api.tile_weight``; the same bits).  Rows of the matrix as the file holds it lie K values apart, and a
     workgroup that walks 64 of them side by side gets less out of the memory: measured on an MI355X, the head of
     128,256 rows 177 against 194 us at one row, the 8B shape's decode step 3.83 against 3.98 ms at 8 requests (267
-    against 256 tokens/s at one), for 8.5 GB more memory; weights whose K is split over workgroups gain nothing
-    (3.84 ms with copies of all).  The copy in the file's layout stays: the library's product for many rows reads
+    against 256 tokens/s at one), for 8.5 GB more memory (the 70B shape: 77 GB beside 141 GB of weights; copies are
+    made while COPIES_LEAVE_FREE of the device's memory stays free); weights whose K is split over workgroups gain
+    nothing (3.84 ms with copies of all).  The copy in the file's layout stays: the library's product for many rows reads
     it.  With the measured route switched on, each use's shape is timed as well (once a process)."""
     if not (rt.device.type == "cuda" and rt.dtype == torch.bfloat16 and rt.kernels == "auto"):
         return
@@ -124,7 +136,7 @@ def prepare_weights(rt, uses) -> None:
             made = getattr(w, "_infernum_tiled", None)
             if made is None:
                 made = w._infernum_tiled = {}
-            if epilogue not in made:
+            if epilogue not in made and _room_for_copy(w):
                 made[epilogue] = K.tile_weight(w, epilogue)
         if _route == "measured":
             measure_route(w, epilogue, keep_split)

@@ -488,6 +488,15 @@ def test_wide_weights_get_a_copy_laid_out_for_the_kernel_and_narrow_ones_do_not(
     w32 = _rand(16640, 264)
     L.prepare_weights(fp, [(w32, None, False)])
     assert L.tiled_copy(w32, None) is None
+    # no copy where it would take memory that has to stay free: the weight then runs from the file's layout
+    other = wide.clone()
+    keep, L.COPIES_LEAVE_FREE = L.COPIES_LEAVE_FREE, 1.0
+    try:
+        L.prepare_weights(rt, [(other, None, False)])
+    finally:
+        L.COPIES_LEAVE_FREE = keep
+    assert L.tiled_copy(other, None) is None
+    assert torch.equal(L.linear(x, other), L.linear(x, wide))
 
 
 def test_known_routes_send_rows_to_the_library_where_the_table_says():
