@@ -84,6 +84,30 @@ def test_llama3_scaling_three_bands():
     assert torch.allclose(P.rope_frequencies(32, 500000.0, one), base)      # rope.rs:982 in spirit
 
 
+def test_llama3_scaling_blends_in_the_frequency_between_the_bands_edges():
+    """Between the edges the scaled frequency over the unscaled one is affine in the frequency itself, from 1/factor
+    at the edge of the long waves (f = 2 pi low / n) to 1 at the edge of the short ones (f = 2 pi high / n):
+    the reference's ramp (infernum/src/rope.rs:104-110) is (n / wavelength - low) / (high - low), and n / wavelength
+    is n f / (2 pi).  A blend that is affine in the wavelength, or in the index of the pair, fails this; so do
+    swapped edges."""
+    n, low, high, factor = 8192, 1.0, 4.0, 8.0
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
+              original_max_position_embeddings=n)
+    base = P.rope_frequencies(2048, 500000.0, None)           # many pairs, so that dozens fall between the edges
+    scaled = P.rope_frequencies(2048, 500000.0, sc)
+    f_long, f_short = 2 * math.pi * low / n, 2 * math.pi * high / n
+    inside = (base > f_long) & (base < f_short)
+    assert int(inside.sum()) >= 40
+    ratio = scaled[inside] / base[inside]
+    want = 1 / factor + (1 - 1 / factor) * (base[inside] - f_long) / (f_short - f_long)
+    assert torch.allclose(ratio, want, rtol=1e-12, atol=0)
+    assert torch.all(ratio[:-1] > ratio[1:])                    # pairs of rising index have falling frequencies
+    # and it is not affine in the wavelength: the middle of the band in wavelength is not its middle in the ratio
+    wl = 2 * math.pi / base[inside]
+    mid = torch.argmin((wl - (n / low + n / high) / 2).abs())
+    assert abs(float(ratio[mid]) - (1 / factor + 1) / 2) > 0.1
+
+
 def _sdpa(q, k, v, scale):
     # library attention on [heads, T, d]
     return torch.nn.functional.scaled_dot_product_attention(
