@@ -339,10 +339,10 @@ def long_contexts(a) -> int:
     # a long prompt in portions beside decoding requests: eight requests decode (512 tokens of context each), then a
     # prompt of 32,768 tokens arrives and goes in 8,192 tokens a step while they go on
     cc = engine.cache.config
-    # (a step holds 8,192 tokens with the decoded ones: the library's products lose a third to half of their rate at
-    # 8,200 rows, which fill one tile of 256 more than two rounds of workgroups hold)
+    # (the scheduler cuts the portions so that a step holds 8,192 tokens with the decoded ones: the library's products
+    # lose a third to half of their rate at 8,200 rows, which fill one tile of 256 more than two rounds of workgroups)
     bc = BatchConfig(max_batch_size=9, max_prefill_tokens=8192, block_size=cc.page_size, num_blocks=cc.num_pages,
-                     max_tokens_per_step=8192)
+                     max_tokens_per_step=8192 + 8)
     rt = Runtime(engine, None, bc)
     V = cfg.vocab_size
     short = [rt.submit(torch.randint(0, V, (PROMPT_LEN,), generator=g).tolist(), GenerateOptions(max_new_tokens=64))

@@ -62,7 +62,7 @@ _SIGNATURES = {
                                    POINTER(c_int32), c_int, c_int, POINTER(c_int32), c_int]),
     "ia_cache_packed": (POINTER(c_int32), [c_void_p]),
     "ia_sched_step": (c_int, [c_void_p, c_int, POINTER(c_int64), POINTER(c_int), POINTER(c_int64), c_int,
-                              POINTER(c_int64), c_int, c_int, c_int, POINTER(c_int), c_int]),
+                              POINTER(c_int64), c_int, c_int, c_int, c_int, POINTER(c_int), c_int]),
 }
 
 

@@ -638,7 +638,7 @@ int ia_cache_pack_step(void* h, int n, const int64_t* reqs, const int* q_lens, c
 // Returns the number of actions, or IA_HOST_ERROR.
 int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run_phase, const int64_t* run_tokens,
                   int n_waiting, const int64_t* wait_tokens, int max_batch, int max_prefill, int max_step_tokens,
-                  int* actions, int cap) {
+                  int step_multiple, int* actions, int cap) {
   Cache* c = static_cast<Cache*>(h);
   const size_t G = c->groups.size();
   struct Act { int kind, index, a, b; };
@@ -671,6 +671,14 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
     for (const Act& a : acts)
       if (a.kind == 1 || a.kind == 2 || a.kind == 5) return true;
     return false;
+  };
+  // A portion that does not reach its prompt's end stops where the step's tokens are a multiple of step_multiple
+  // (the rows of the products' tiles), if that leaves it at least half of what it could take.
+  auto cut = [&](int64_t n, int64_t remaining) {
+    if (step_multiple <= 1 || n >= remaining) return n;
+    const int64_t used = (int64_t)max_step_tokens - budget;
+    const int64_t whole = (used + n) / step_multiple * step_multiple;
+    return (whole - used) * 2 >= n ? whole - used : n;
   };
   auto drop_from_live = [&](int s) { live.erase(std::find(live.begin(), live.end(), s)); };
   // the request admitted last among those that can be set back (-1: none), and whether one is on its way out
@@ -741,6 +749,7 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
     const int64_t cached = r >= 0 ? c->tokens[r] : 0;
     int64_t n = std::min<int64_t>(std::min<int64_t>(run_tokens[s] - cached, max_prefill), budget);
     n = std::min<int64_t>(n, tokens_that_fit(r));
+    if (n > 0) n = cut(n, run_tokens[s] - cached);
     if (n <= 0) {
       if (!planned() && !any_leaving()) {
         const int victim = last_movable();        // nobody can move: the last admitted request makes room
@@ -769,13 +778,14 @@ int ia_sched_step(void* h, int n_running, const int64_t* run_rid, const int* run
   while (w < n_waiting && !blocked && !any_set_back && budget > 0 &&
          (int)live.size() + admitted_now < max_batch && (int)c->free_slots.size() - new_slots > 0) {
     const int64_t running_now = (int64_t)live.size() + admitted_now;
-    int64_t n = std::min<int64_t>(std::min<int64_t>(wait_tokens[w], max_prefill), budget);
+    int64_t n = cut(std::min<int64_t>(std::min<int64_t>(wait_tokens[w], max_prefill), budget), wait_tokens[w]);
     pages_needed(-1, n);
     // one page in hand for every running request, so that a newcomer is not set back at once
     if (!fits(running_now)) {
       if (running_now == 0 && !planned()) {
         // alone and still too large for one portion: shrink the portion to the pool
         n = std::min<int64_t>(n, tokens_that_fit(-1));
+        if (n > 0) n = cut(n, wait_tokens[w]);
         if (n <= 0) {
           acts.push_back({4, w, 3, 0});
           ++w;

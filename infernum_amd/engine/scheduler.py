@@ -75,11 +75,16 @@ class BatchConfig:
     max_prefill_tokens: int = 512     # longest portion of one prompt in one step
     block_size: int = 16              # tokens per page
     num_blocks: int = 1024            # pages in the pool
-    max_tokens_per_step: int = 2048   # all tokens of one step, decoded ones included (a multiple of 256 fills the
-                                      # tiles of the library's products: 8,200 rows take what 8,448 do)
+    max_tokens_per_step: int = 2048   # all tokens of one step, decoded ones included
+    # A portion that does not reach its prompt's end stops where the step's tokens are a multiple of this, if that
+    # leaves it at least half of what it could take: the library's products work in tiles of 256 rows (8,200 rows
+    # take what 8,448 do, a third to half more than 8,192), so a portion beside decoded tokens leaves them their rows.
+    # 1: portions are cut by the other limits alone, as the reference cuts them.
+    step_token_multiple: int = 256
 
     def __post_init__(self) -> None:
-        for name in ("max_batch_size", "max_prefill_tokens", "block_size", "num_blocks", "max_tokens_per_step"):
+        for name in ("max_batch_size", "max_prefill_tokens", "block_size", "num_blocks", "max_tokens_per_step",
+                     "step_token_multiple"):
             if int(getattr(self, name)) <= 0:
                 raise ValueError(f"{name} must be positive")
         if self.max_tokens_per_step < self.max_batch_size:
@@ -214,7 +219,7 @@ class Scheduler:
         actions = (ctypes.c_int * (4 * cap))()
         n = native.lib().ia_sched_step(cache.native_handle(), nr, rid, phase, tokens, nw, wait_tokens,
                                        cfg.max_batch_size, cfg.max_prefill_tokens, cfg.max_tokens_per_step,
-                                       actions, cap)
+                                       cfg.step_token_multiple, actions, cap)
         if n < 0:
             cache._fail()
         cache.poison_freed()

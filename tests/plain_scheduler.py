@@ -26,6 +26,16 @@ class PlainScheduler(Scheduler):
             for i, n in enumerate(need):
                 promised[i] += n
 
+        def cut(n: int, remaining: int) -> int:
+            """A portion that does not reach its prompt's end stops where the step's tokens are a multiple of
+            ``step_token_multiple``, if that leaves it at least half of what it could take."""
+            m = cfg.step_token_multiple
+            if m <= 1 or n >= remaining:
+                return n
+            used = cfg.max_tokens_per_step - budget
+            whole = (used + n) // m * m
+            return whole - used if (whole - used) * 2 >= n else n
+
         # requests that are done but for a token still on its way: they hold their pages, do nothing, are never
         # set back; who cannot move because of them waits
         leaving = [s for s in self.running if self._awaits_last_token(s)]
@@ -72,6 +82,8 @@ class PlainScheduler(Scheduler):
             n = min(seq.num_tokens - cached, cfg.max_prefill_tokens, budget)
             n = min(n, cache.tokens_that_fit(seq.id, promised) if cache.has(seq.id)
                     else cache.tokens_that_fit(None, promised))
+            if n > 0:
+                n = cut(n, seq.num_tokens - cached)
             if n <= 0:
                 if out.is_empty() and not leaving:
                     # nobody can move: the last admitted request makes room
@@ -99,7 +111,7 @@ class PlainScheduler(Scheduler):
         while (self.waiting and not blocked and not out.set_back and budget > 0
                and len(self.running) < cfg.max_batch_size and cache.slots.num_free - new_slots > 0):
             seq = self.waiting[0]
-            n = min(seq.num_tokens, cfg.max_prefill_tokens, budget)
+            n = cut(min(seq.num_tokens, cfg.max_prefill_tokens, budget), seq.num_tokens)
             need = cache.pages_needed(seq.id, n)
             # keep one page in hand for every running request, so that a newcomer is not set back at once
             spare = [len(self.running)] * len(need) if self.running else [0] * len(need)
@@ -107,6 +119,8 @@ class PlainScheduler(Scheduler):
                 if not self.running and out.is_empty():
                     # alone and still too large for one portion: shrink the portion to the pool
                     n = min(n, cache.tokens_that_fit(None, promised))
+                    if n > 0:
+                        n = cut(n, seq.num_tokens)
                     if n <= 0:
                         self.waiting.popleft()
                         self._fail(seq, "the page pool has no free page although nothing is running")

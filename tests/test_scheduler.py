@@ -101,6 +101,39 @@ def test_token_budget_bounds_every_step_and_decoding_goes_first():
     assert all(s.generated_ids == reference_generation(list(range(30)), GenerateOptions(max_new_tokens=6)) for s in seqs)
 
 
+def _decoding_beside_a_long_prompt(chunk, budget, multiple, decoders, prompt_len):
+    """``decoders`` requests decode, then a prompt of ``prompt_len`` tokens arrives; returns the sizes of its portions."""
+    eng = FakeEngine(50, 16, 4096, decoders + 2)
+    bc = BatchConfig(max_batch_size=decoders + 1, max_prefill_tokens=chunk, block_size=16, num_blocks=4096,
+                     max_tokens_per_step=budget, step_token_multiple=multiple)
+    rt = Runtime(eng, None, bc, sampler=CpuSampler())
+    rt.look_ahead = False
+    for _ in range(decoders):
+        rt.submit([1, 2, 3], GenerateOptions(max_new_tokens=1000))
+    rt.step()
+    big = rt.submit(list(range(prompt_len)), GenerateOptions(max_new_tokens=1))
+    sizes = []
+    while big.phase != SequencePhase.DECODE and not big.generated_ids:
+        plan = rt.step()
+        assert len(plan.decode) == decoders and plan.num_tokens <= budget
+        sizes += [len(t.token_ids) for t in plan.prefill]
+    assert sum(sizes) == prompt_len
+    return sizes
+
+
+def test_a_portion_beside_decoded_tokens_leaves_the_step_a_multiple_of_the_tiles_rows():
+    # eight decoded tokens and portions of up to 8,192 under a budget of 8,200: the step holds 8,192 tokens, not 8,200
+    assert _decoding_beside_a_long_prompt(8192, 8200, 256, 8, 20000) == [8184, 8184, 3632]
+    # as the reference cuts them with a multiple of 1
+    assert _decoding_beside_a_long_prompt(8192, 8200, 1, 8, 20000) == [8192, 8192, 3616]
+    # the defaults' portion of 512 beside twenty decoded tokens: 512 tokens in all
+    assert _decoding_beside_a_long_prompt(512, 2048, 256, 20, 1100) == [492, 512 - 20, 116]
+    # a portion that reaches its prompt's end is not cut, and none is cut to less than half of what it could take
+    assert _decoding_beside_a_long_prompt(512, 2048, 256, 20, 500) == [500]
+    assert _decoding_beside_a_long_prompt(100, 2048, 256, 250, 180) == [100, 80]
+    assert _decoding_beside_a_long_prompt(100, 2048, 256, 200, 180) == [56, 56, 68]
+
+
 def test_config_is_checked():
     with pytest.raises(ValueError):
         BatchConfig(max_batch_size=8, max_tokens_per_step=4)

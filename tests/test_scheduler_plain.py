@@ -20,7 +20,8 @@ def pair(seed, look_ahead=False):
     if seed % 3 == 0:
         needs.append((CacheSpec("window", 1, 16, window=rng.choice((3, 9))), None))
     bc = BatchConfig(max_batch_size=rng.choice((2, 3, 5)), max_prefill_tokens=rng.choice((3, 8, 64)),
-                     block_size=ps, num_blocks=kw["num_pages"], max_tokens_per_step=rng.choice((8, 16, 64)))
+                     block_size=ps, num_blocks=kw["num_pages"], max_tokens_per_step=rng.choice((8, 16, 64)),
+                     step_token_multiple=random.Random(seed + 977).choice((1, 4, 8, 256)))
     out = []
     for plain in (False, True):
         eng = FakeEngine(50, needs=list(needs), **kw)
