@@ -18,7 +18,7 @@ import torch
 import plain_llama as P
 import tiny_models as TM
 import trace_tools as TT
-from part_harness import DEV, build, rel_err, runtime
+from part_harness import build, rel_err, runtime
 
 pytestmark = pytest.mark.gpu
 TOL = {"float32": 2e-5, "bfloat16": 6e-2}
