@@ -11,6 +11,7 @@ from __future__ import annotations
 import atexit
 import ctypes
 import functools
+import math
 import os
 import sys
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -512,20 +513,32 @@ def compute_units(device: Optional[torch.device] = None) -> int:
     return cus
 
 
-def decode_splits(batch: int, nh: int, nkv: int, max_len: int, device: Optional[torch.device] = None) -> int:
+def decode_splits(batch: int, nh: int, nkv: int, max_len: int, device: Optional[torch.device] = None,
+                  head_dim: int = 128) -> int:
     """Parts the keys of a request are cut into, so that a small batch still fills the GPU (workgroups of
-    four waves, each wave one tile of 16 keys at a time): about one workgroup a compute unit while the batch alone
-    gives at most a quarter of that, about two up to five eighths, and no parts above that (measured on 256
-    compute units with the 8B shape and 527 keys: 24 requests 13.9 us whole against 15.3 in three parts, 32
-    requests 15.4 against 17.1 in two); at least 8 tiles a workgroup (more and shorter parts cost more in the
-    join than they gain)."""
+    four waves, each wave one tile of 16 keys at a time).  Measured on 256 compute units, with the join's launch:
+
+    * head sizes up to 128: about one workgroup a compute unit while the batch alone gives at most a quarter of
+      that, about two up to five eighths, and no parts above that (8B shape, 527 keys: 24 requests 13.9 us whole
+      against 15.3 in three parts, 32 requests 15.4 against 17.1 in two); at head sizes up to 64 a tile is half the
+      bytes and twice as many workgroups are wanted (8 requests with 32,768 keys each: 97 us in eight parts, 138
+      in four; 32 requests: 364 in two, 520 whole);
+    * above 128 a compute unit holds one workgroup, and more parts than compute units only cost (head size 256, 32
+      requests on 4 key/value heads: 19 us in two parts, 23 in four);
+    * the join grows with the parts as the work of a part shrinks with them: the best number of parts for one
+      request went with the square root of its tiles (4 parts at 512 keys, 8 at 2,048, 16 at 8,192, 32 at 32,768, for
+      head sizes 64, 128 and 256 alike), so that bounds the parts; never more than 64."""
     cus = compute_units(device)
+    fill = cus * (2 if head_dim <= 64 else 1)
     groups = batch * nkv * ((nh // nkv + 15) // 16)
     tiles = max(1, (max_len + 15) // 16)
-    if 8 * groups >= 5 * cus:
+    if 8 * groups >= 5 * fill:
         return 1
-    wanted = cus // groups if 4 * groups <= cus else 2 * cus // groups
-    return max(1, min(wanted, tiles // 8, 64))
+    if head_dim > 128:
+        wanted = fill // groups
+    else:
+        wanted = fill // groups if 4 * groups <= fill else 2 * fill // groups
+    return max(1, min(wanted, math.isqrt(tiles // 2), 64))
 
 
 def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
@@ -543,7 +556,7 @@ def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Te
     ps = k_pages.shape[2]
     _need(ps % 4 == 0, f"attention_decode: page size {ps} is not a multiple of 4")
     _need(block_tables.shape[1] * ps >= max_len, "attention_decode: block_tables are narrower than max_len")
-    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device)
+    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device, d)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)
@@ -593,7 +606,7 @@ def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[t
     ps = k_pages.shape[2]
     _need(ps % 4 == 0, f"attention_decode_rotating: page size {ps} is not a multiple of 4")
     _need(block_tables.shape[1] * ps >= max_len, "attention_decode_rotating: block_tables are narrower than max_len")
-    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device)
+    splits = num_splits or decode_splits(B, nh, nkv, max_len, out.device, d)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(B * nh * splits * d, dtype=torch.float32, device=out.device)

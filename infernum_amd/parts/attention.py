@@ -205,7 +205,7 @@ class Attention(Mixer):
                     return 1
                 if ctx.block_tables[g].shape[1] * ps < ctx.max_total_len:
                     raise K.KernelError("attention: the block tables are narrower than the longest request")
-                n = K.decode_splits(nd, nh, nkv, ctx.max_total_len, dev)
+                n = K.decode_splits(nd, nh, nkv, ctx.max_total_len, dev, d)
                 if nd * n > records:
                     raise K.KernelError("attention: the parts of the keys do not fit the program's arena")
                 return n
