@@ -215,15 +215,41 @@ __global__ __launch_bounds__(256) void gemm_skinny_join_kernel(const float* __re
   store_out<TO>(C + idx, EPI == SK_EPI_SWIGLU ? a / (1.0f + expf(-a)) * b : a);
 }
 
-static int skinny_splits(int N, int K) {
-  const int nb = (N + SK_BN - 1) / SK_BN;
-  const int nchunks = (K + SK_KC - 1) / SK_KC;
-  if (nb >= SK_ENOUGH_BLOCKS) return 1;      // measured: a split costs more than it gains here
-  int ks = (SK_TARGET_BLOCKS + nb - 1) / nb;
+// Shapes whose number of splits was measured (ia_gemm_skinny_set_splits, filled from a table when the library is
+// loaded): few entries, looked up per launch.
+struct KnownSplits { int N, K, splits; };
+static KnownSplits g_known_splits[64];
+static int g_known_count = 0;
+
+static int split_count(int nchunks, int ks) {
   if (ks > nchunks) ks = nchunks;
   if (ks < 1) ks = 1;
   const int cps = (nchunks + ks - 1) / ks;
   return (nchunks + cps - 1) / cps;
+}
+
+static int skinny_splits(int N, int K) {
+  const int nb = (N + SK_BN - 1) / SK_BN;
+  const int nchunks = (K + SK_KC - 1) / SK_KC;
+  for (int i = 0; i < g_known_count; ++i)
+    if (g_known_splits[i].N == N && g_known_splits[i].K == K) return split_count(nchunks, g_known_splits[i].splits);
+  if (nb >= SK_ENOUGH_BLOCKS) return 1;      // measured: a split costs more than it gains here
+  return split_count(nchunks, (SK_TARGET_BLOCKS + nb - 1) / nb);
+}
+
+// Says into how many parts (about: the chunks of K are dealt out evenly) the inner dimension of a weight [N, K] is
+// split from now on, in place of the rule of sizes.  To be called before the first product of that shape (the
+// partial sums' layout follows the number).  Returns 0, or 10001 for bad arguments or a full table.
+extern "C" int ia_gemm_skinny_set_splits(int N, int K, int splits) {
+  if (N <= 0 || K <= 0 || splits < 1) return IA_ERR_BAD_ARG;
+  for (int i = 0; i < g_known_count; ++i)
+    if (g_known_splits[i].N == N && g_known_splits[i].K == K) {
+      g_known_splits[i].splits = splits;
+      return IA_OK;
+    }
+  if (g_known_count >= 64) return IA_ERR_BAD_ARG;
+  g_known_splits[g_known_count++] = KnownSplits{N, K, splits};
+  return IA_OK;
 }
 
 // Number of K splits the kernel uses for a weight [N, K] (a function of N and K only).

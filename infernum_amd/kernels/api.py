@@ -36,6 +36,19 @@ _ERRORS = {10001: "bad argument", 10002: "size not supported by this kernel",
            10003: "a call into the GEMM library failed"}
 
 
+# Into how many parts the weight-streaming product splits the inner dimension of a weight [N, K], where that was
+# measured and differs from the rule of sizes (about 512 workgroups): the 13B, 70B and 1B shapes' products on an
+# MI355X, with cold weights and the norm that joins the parts behind them, at 1, 8 and 64 rows (13B down projection:
+# 35.0 us in six even parts of nine chunks, 42.3 in the rule's seven; 70B QKV: 35.4 us in three parts, 43.5 in four).
+# The sums of a product are taken in the order that its number of parts gives: a shape's entry is part of its
+# arithmetic, the same in every process.
+KNOWN_SPLITS = {
+    (15360, 5120): 2, (5120, 5120): 5, (5120, 13824): 6,       # Llama-2-13B: QKV, output and down projection
+    (10240, 8192): 3,                                          # Llama-3.1-70B: QKV
+    (2048, 8192): 8,                                           # Llama-3.2-1B: down projection
+}
+
+
 def load_library(name: str) -> ctypes.CDLL:
     lib = _libs.get(name)
     if lib is None:
@@ -46,6 +59,9 @@ def load_library(name: str) -> ctypes.CDLL:
             lib = ctypes.CDLL(path)
         except (OSError, _build.BuildError) as e:
             raise KernelError(f"the HIP kernel library '{name}' could not be built or loaded: {e}") from e
+        if name == "core":
+            for (N, K), parts in KNOWN_SPLITS.items():
+                _ok(lib.ia_gemm_skinny_set_splits(N, K, parts), "gemm_skinny_set_splits")
         _libs[name] = lib
     return lib
 

@@ -54,9 +54,9 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
     (2048, 8192, None, True): 0,
     (6144, 4096, None, True): 0, (4096, 4096, None, True): 0, (28672, 4096, "swiglu", False): 0b11110000,
     (4096, 14336, None, True): 0,
-    (15360, 5120, None, True): 0b11111110, (5120, 5120, None, True): 0b01010010,
-    (27648, 5120, "swiglu", False): 0b11101010, (5120, 13824, None, True): 0b01001110,
-    (10240, 8192, None, True): 0b11101110, (8192, 8192, None, True): 0b01011110,
+    (15360, 5120, None, True): 0b11111110, (5120, 5120, None, True): 0,
+    (27648, 5120, "swiglu", False): 0b11111010, (5120, 13824, None, True): 0,
+    (10240, 8192, None, True): 0b01001110, (8192, 8192, None, True): 0b01011110,
     (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
 }
 

@@ -307,6 +307,25 @@ def test_gemm_skinny_partial_sums_and_swiglu(M, N, K_):
     assert torch.equal(actb, act.bfloat16())
 
 
+def test_gemm_skinny_takes_the_measured_number_of_parts_for_the_shapes_of_its_table():
+    """The table of measured shapes is in force from the library's load on: its shapes are split as it says (the
+    chunks of K dealt out evenly), others by the rule of sizes; a product of such a shape is right and its partial sums
+    add up to it."""
+    api = K()
+    assert api.KNOWN_SPLITS[(5120, 13824)] == 6 and api.gemm_skinny_splits(5120, 13824) == 6     # 54 chunks: 6 x 9
+    assert api.gemm_skinny_splits(10240, 8192) == 3 and api.gemm_skinny_splits(2048, 8192) == 8
+    assert api.gemm_skinny_splits(4096, 14336) == 8 and api.gemm_skinny_splits(4096, 4096) == 8  # the rule: 512 workgroups
+    for (N, Kd), parts in api.KNOWN_SPLITS.items():
+        assert 1 <= api.gemm_skinny_splits(N, Kd) <= parts
+    N, Kd, M = 5120, 5120, 5
+    a, w = _rand(M, Kd, dtype=torch.bfloat16, seed=1), _rand(N, Kd, dtype=torch.bfloat16, seed=2)
+    out = api.gemm_skinny(a, w, out_dtype=torch.float32)
+    want = a.double() @ w.double().t()
+    assert ((out.double() - want).abs().max() / want.abs().max()).item() < 1e-5
+    kept = api.gemm_skinny(a, w, keep_split=True)
+    assert kept.parts.shape[0] == 5 and torch.allclose(kept.parts.sum(0), out, rtol=1e-5, atol=1e-3)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     api = K()
     a, w = _rand(129, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
