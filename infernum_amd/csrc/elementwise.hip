@@ -408,11 +408,58 @@ __global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(
       store4(dst + i, load4(row + (size_t)head * d + i));
     }
   }
-  if (do_write) {                      // values: plain copies into the transposed pages
+  if (do_write && write_kv == 1) {     // values: plain copies into the transposed pages (2: another launch writes them)
     const TS* v = row + (size_t)(nh + nkv) * d;
     for (int it = tid; it < nkv * d; it += 256) {
       const int g = it / d, i = it - g * d;
       v_pages[(((size_t)page * nkv + g) * d + i) * page_size + off] = from_float<T>(to_float(v[it]));
+    }
+  }
+}
+
+// The values of many tokens into their transposed pages [page, head, d, page_size]: a token's d values of a head lie
+// page_size apart there, and one store a value costs more than everything else the launch above does once there are
+// many key/value heads.  A workgroup takes 16 tokens of one head through LDS; tokens that follow each other in a page
+// (the tokens of a prompt's portion do) are written eight at a time, 16 bytes in bfloat16.  grid (ceil(N / 16), nkv),
+// 256 threads; d <= 256 and a multiple of 4, page_size a multiple of 8, row_stride a multiple of 4.
+template <typename TS, typename T>
+__global__ __launch_bounds__(256) void append_values_rows_kernel(const TS* __restrict__ src, const int* __restrict__ slots,
+                                                                 T* __restrict__ v_pages, int row_stride, int v_col0,
+                                                                 int nkv, int d, int page_size, int num_pages, int N) {
+  __shared__ __attribute__((aligned(16))) T tile[16][256 + 8];
+  __shared__ int s_slot[16];
+  const int n0 = blockIdx.x * 16, g = blockIdx.y, tid = threadIdx.x;
+  const int cnt = N - n0 < 16 ? N - n0 : 16;
+  if (tid < 16) {
+    const int sl = tid < cnt ? slots[n0 + tid] : -1;
+    s_slot[tid] = (sl >= 0 && sl < num_pages * page_size) ? sl : -1;
+  }
+  const int d4 = d >> 2;
+  for (int it = tid; it < cnt * d4; it += 256) {
+    const int t = it / d4, i = (it - t * d4) << 2;
+    store4(&tile[t][i], load4(src + (size_t)(n0 + t) * row_stride + v_col0 + (size_t)g * d + i));
+  }
+  __syncthreads();
+  for (int i = tid; i < d; i += 256) {
+    int t = 0;
+    while (t < cnt) {                  // the same walk in every thread: the slots are the workgroup's
+      const int sl = s_slot[t];
+      if (sl < 0) { ++t; continue; }
+      const int page = sl / page_size, off = sl - page * page_size;
+      int run = 1;
+      while (t + run < cnt && s_slot[t + run] == sl + run && off + run < page_size) ++run;
+      T* dst = v_pages + (((size_t)page * nkv + g) * d + i) * page_size + off;
+      int k = 0;
+      while (k < run && ((off + k) & 7)) { dst[k] = tile[t + k][i]; ++k; }
+      for (; k + 8 <= run; k += 8) {
+        float e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = to_float(tile[t + k + j][i]);
+        store4(dst + k, make_float4(e[0], e[1], e[2], e[3]));          // exact: the values have T's precision already
+        store4(dst + k + 4, make_float4(e[4], e[5], e[6], e[7]));
+      }
+      for (; k < run; ++k) dst[k] = tile[t + k][i];
+      t += run;
     }
   }
 }
@@ -437,10 +484,18 @@ extern "C" int ia_rope_kv_append(const void* src, int src_dtype, int splits, int
   const bool aligned = (((uintptr_t)src | (uintptr_t)q_out | (uintptr_t)k_pages) & 15) == 0;
   if (N >= 32 && splits == 1 && (rot & 7) == 0 && (d & 3) == 0 && d <= 256 && (row_stride & 3) == 0 &&
       (q_stride & 3) == 0 && aligned) {
+    // values by the launch that writes them eight tokens at a time, where the sizes allow it
+    const bool values_apart = write_kv && (page_size & 7) == 0 && nkv <= 65535 && (((uintptr_t)v_pages) & 15) == 0;
+    const int kv_mode = write_kv ? (values_apart ? 2 : 1) : 0;
 #define ROPE_ROWS_LAUNCH(TS, T)                                                                                    \
-  rope_kv_append_rows_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, (T*)q_out, q_stride, positions, slots,  \
-                                                           inv_freq, freq_f64, (T*)k_pages, (T*)v_pages, row_stride, nh, nkv, \
-                                                           d, rot, page_size, num_pages, write_kv, copy_q_tail)
+  do {                                                                                                             \
+    rope_kv_append_rows_kernel<TS, T><<<N, 256, 0, stream>>>((const TS*)src, (T*)q_out, q_stride, positions, slots, \
+                                                             inv_freq, freq_f64, (T*)k_pages, (T*)v_pages, row_stride, nh, \
+                                                             nkv, d, rot, page_size, num_pages, kv_mode, copy_q_tail); \
+    if (values_apart)                                                                                              \
+      append_values_rows_kernel<TS, T><<<dim3((N + 15) / 16, nkv), 256, 0, stream>>>(                               \
+          (const TS*)src, slots, (T*)v_pages, row_stride, (nh + nkv) * d, nkv, d, page_size, num_pages, N);        \
+  } while (0)
     if (act_dtype == IA_F32 && src_dtype == IA_F32) ROPE_ROWS_LAUNCH(float, float);
     else if (act_dtype == IA_BF16 && src_dtype == IA_BF16) ROPE_ROWS_LAUNCH(bf16_t, bf16_t);
     else if (act_dtype == IA_BF16 && src_dtype == IA_F32) ROPE_ROWS_LAUNCH(float, bf16_t);

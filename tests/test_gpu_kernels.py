@@ -240,6 +240,46 @@ def test_rope_of_many_tokens_equals_rope_of_few(dtype, nh, nkv, d, rot, ps):
     assert torch.equal(q_out, many[:, :nh * d]) and torch.equal(src, qkv) and torch.equal(kp3, kp1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,ps", [(40, 40, 128, 16), (8, 2, 64, 8), (4, 4, 256, 32), (6, 3, 48, 24), (4, 2, 32, 12)])
+def test_values_of_a_portion_go_to_their_pages_in_runs(dtype, nh, nkv, d, ps):
+    """The values of many tokens are written by a launch of their own that takes the tokens which follow each other
+    in a page eight at a time: three requests' portions in one call (one starts in the middle of a page, pages in any
+    order, a token without a slot between them, a count that is no multiple of sixteen) leave the pages that
+    calls of a few tokens leave, which write every value alone."""
+    pages = 40
+    order = torch.randperm(pages, generator=torch.Generator().manual_seed(ps + d)).tolist()
+    slots, pos = [], []
+    for first, count in ((5, 45), (0, 33), (ps - 1, 2 * ps + 3)):
+        need = (first + count + ps - 1) // ps
+        table, order = order[:need], order[need:]
+        for p_ in range(first, first + count):
+            slots.append(table[p_ // ps] * ps + p_ % ps)
+            pos.append(p_)
+    slots[50] = -1                                           # a token whose key and value are not kept
+    N = len(slots)
+    assert N % 16 != 0 and N >= 32
+    qkv = _rand(N, (nh + 2 * nkv) * d, dtype=dtype, seed=13)
+    slots_t, pos_t = torch.tensor(slots, dtype=torch.int32, device=DEV), torch.tensor(pos, dtype=torch.int32, device=DEV)
+    inv = (10000.0 ** (-torch.arange(d // 2, dtype=torch.float64) * 2 / d)).to(DEV)
+    kp1 = torch.full((pages, nkv, ps, d), 7.0, dtype=dtype, device=DEV)
+    vp1 = torch.full((pages, nkv, d, ps), 7.0, dtype=dtype, device=DEV)
+    kp2, vp2 = kp1.clone(), vp1.clone()
+    many, few = qkv.clone(), qkv.clone()
+    K().rope_kv_append(many, pos_t, inv, nh, nkv, d, d, slots_t, kp1, vp1)
+    for n0 in range(0, N, 10):
+        K().rope_kv_append(few[n0:n0 + 10], pos_t[n0:n0 + 10].contiguous(), inv, nh, nkv, d, d,
+                           slots_t[n0:n0 + 10].contiguous(), kp2, vp2)
+    assert torch.equal(many, few) and torch.equal(kp1, kp2) and torch.equal(vp1, vp2)
+    # the values themselves, at their places; what no token owns is untouched
+    want = torch.full_like(vp1, 7.0)
+    v = qkv[:, (nh + nkv) * d:].reshape(N, nkv, d)
+    for n, sl in enumerate(slots):
+        if sl >= 0:
+            want[sl // ps, :, :, sl % ps] = v[n]
+    assert torch.equal(vp1, want)
+
+
 # -------------------------------------------------------------- matrix products
 @pytest.mark.parametrize("M,N,K_", [(1, 250, 96), (7, 384, 176), (70, 129, 1000), (300, 64, 33)])
 def test_gemm_generic(M, N, K_):
