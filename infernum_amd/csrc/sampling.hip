@@ -90,8 +90,11 @@ extern "C" int ia_argmax(const float* logits, int ld, int* out, int R, int V, hi
 // divided by penalty[r], another is multiplied by it.  A token that stands in the
 // list twice is penalised twice.  Rows are independent; one thread walks a row's
 // list so that the order of the updates is fixed.
+// previous (nullable): tokens that an earlier launch left on the device; previous_index[r] >= 0 names the one that
+// is row r's newest token and stands behind its list (a request whose last token has not reached the host yet).
 __global__ void penalty_kernel(float* __restrict__ logits, int ld, const int* __restrict__ recent, int recent_stride,
-                               const int* __restrict__ counts, const float* __restrict__ penalty, int V) {
+                               const int* __restrict__ counts, const float* __restrict__ penalty,
+                               const int* __restrict__ previous, const int* __restrict__ previous_index, int V) {
   if (threadIdx.x != 0) return;
   const int r = blockIdx.x;
   const float pen = penalty[r];
@@ -104,13 +107,21 @@ __global__ void penalty_kernel(float* __restrict__ logits, int ld, const int* __
     const float v = x[tok];
     x[tok] = v > 0.f ? v / pen : v * pen;
   }
+  if (previous && previous_index && previous_index[r] >= 0) {
+    const int tok = previous[previous_index[r]];
+    if (tok >= 0 && tok < V) {
+      const float v = x[tok];
+      x[tok] = v > 0.f ? v / pen : v * pen;
+    }
+  }
 }
 
 extern "C" int ia_repetition_penalty(float* logits, int ld, const int* recent, int recent_stride, const int* counts,
-                                     const float* penalty, int R, int V, hipStream_t stream) {
+                                     const float* penalty, const int* previous, const int* previous_index, int R, int V,
+                                     hipStream_t stream) {
   if (R < 0 || V <= 0 || ld < V || recent_stride <= 0) return IA_ERR_BAD_ARG;
   if (R == 0) return IA_OK;
-  penalty_kernel<<<R, 64, 0, stream>>>(logits, ld, recent, recent_stride, counts, penalty, V);
+  penalty_kernel<<<R, 64, 0, stream>>>(logits, ld, recent, recent_stride, counts, penalty, previous, previous_index, V);
   IA_LAUNCH_CHECK();
   return IA_OK;
 }

@@ -74,8 +74,9 @@ class Runtime:
         self.tokens_run = 0
         # One step ahead: a step is launched with the tokens of the step before it still on the device, and the
         # host reads a step's tokens while the next step runs.  Needs an engine that takes tokens from the device
-        # and a sampler that leaves them there; requests whose choice looks at their own history (a repetition
-        # penalty) are served one step at a time.
+        # and a sampler that leaves them there; a choice that looks at the request's own last tokens (a repetition
+        # penalty) finds the newest of them on the device too, with a sampler that says so (``history_on_device``;
+        # with another, such requests are served one step at a time).
         self.look_ahead = (getattr(engine, "supports_device_tokens", False)
                            and hasattr(self.sampler, "select_on_device") and hasattr(self.sampler, "needs_history"))
         self._inflight = None                 # (plan, tokens on the device, row of each request, download)
@@ -144,6 +145,8 @@ class Runtime:
 
     # ---- one step ahead ------------------------------------------------------------------
     def _all_can_wait(self) -> bool:
+        if getattr(self.sampler, "history_on_device", False):
+            return True                           # the sampler finds a request's newest token on the device
         needs = self.sampler.needs_history
         return not any(needs(s.options.sampling) for s in self.scheduler.running) and \
             not any(needs(s.options.sampling) for s in self.scheduler.waiting)
@@ -184,7 +187,7 @@ class Runtime:
                 entries.append(StepEntry(s.id, [s.generated_ids[-1]], [0]))
                 index.append(-1)
             row_of[s.id] = len(rows)
-            rows.append(self._row(s))
+            rows.append(self._row(s, index[-1]))
         for t in plan.prefill:
             entries.append(StepEntry(t.seq.id, t.token_ids, [len(t.token_ids) - 1] if t.completes else []))
             index.append(-1)
@@ -194,7 +197,10 @@ class Runtime:
         try:
             feed = (before[1], index) if before is not None and any(j >= 0 for j in index) else None
             logits = self.engine.step(entries, device_tokens=feed, borrow_logits=True)
-            chosen = self.sampler.select_on_device(logits, rows)
+            if any(r.pending_row >= 0 for r in rows):
+                chosen = self.sampler.select_on_device(logits, rows, previous=before[1])
+            else:
+                chosen = self.sampler.select_on_device(logits, rows)
         except Exception as e:                    # the requests of this batch end with an error event
             for t in list(plan.decode) + list(plan.prefill):
                 self.scheduler._fail(t.seq, f"{type(e).__name__}: {e}")
@@ -216,18 +222,21 @@ class Runtime:
         return plan
 
     @staticmethod
-    def _row(s: SequenceState) -> RowRequest:
+    def _row(s: SequenceState, pending_row: int = -1) -> RowRequest:
+        """``pending_row`` >= 0: the request's newest token is that entry of the tokens which the step in flight
+        leaves on the device; the host's list then ends one token earlier."""
         sp = s.options.sampling
         if sp is None:
             return RowRequest(None)
         hist: Sequence[int] = ()
-        if abs(sp.repetition_penalty - 1.0) > 1.1920929e-07 and sp.repetition_penalty_window > 0:
+        looks_back = abs(sp.repetition_penalty - 1.0) > 1.1920929e-07 and sp.repetition_penalty_window > 0
+        if looks_back:
             # the last tokens of prompt and generation that the penalty looks at, not the whole sequence
-            n = sp.repetition_penalty_window
-            hist = s.generated_ids[-n:]
+            n = sp.repetition_penalty_window - (1 if pending_row >= 0 else 0)
+            hist = s.generated_ids[-n:] if n > 0 else []
             if len(hist) < n:
                 hist = s.prompt_ids[len(s.prompt_ids) - min(n - len(hist), len(s.prompt_ids)):] + hist
-        return RowRequest(sp, len(s.generated_ids) + s.pending, hist)
+        return RowRequest(sp, len(s.generated_ids) + s.pending, hist, pending_row if looks_back else -1)
 
     def run(self, until: Optional[Callable[[], bool]] = None) -> None:
         """Step until nothing waits or runs (or until ``until()`` is true)."""

@@ -723,15 +723,24 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 
 def repetition_penalty(logits: torch.Tensor, recent: torch.Tensor, counts: torch.Tensor,
-                       penalty: torch.Tensor) -> None:
-    _dev(logits, recent, counts, penalty)
+                       penalty: torch.Tensor, previous: Optional[torch.Tensor] = None,
+                       previous_index: Optional[torch.Tensor] = None) -> None:
+    """Every token of recent[r, :counts[r]] is penalised in row r (a positive logit divided by penalty[r], another
+    multiplied by it; a token that stands twice, twice).  ``previous`` (int32 tokens that an earlier launch left
+    on the device) and ``previous_index`` (int32 [R]: which of them is row r's newest token, -1: none) add a token
+    that the host has not seen yet."""
+    _dev(logits, recent, counts, penalty, previous, previous_index)
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "penalty: logits must be fp32")
     _need(recent.dtype == torch.int32 and recent.dim() == 2 and recent.shape[0] == R, "penalty: recent int32 [R, W]")
     _i32(counts, R, "penalty counts")
     _need(penalty.dtype == torch.float32 and penalty.numel() == R, "penalty: one fp32 factor per row")
-    _ok(_core().ia_repetition_penalty(_p(logits), V, _p(recent), recent.shape[1], _p(counts), _p(penalty), R, V,
-                                      _stream()), "repetition_penalty")
+    if previous is not None or previous_index is not None:
+        _need(previous is not None and previous_index is not None and previous.dtype == torch.int32
+              and previous.is_contiguous(), "penalty: previous tokens int32 with their index")
+        _i32(previous_index, R, "penalty previous_index")
+    _ok(_core().ia_repetition_penalty(_p(logits), V, _p(recent), recent.shape[1], _p(counts), _p(penalty),
+                                      _p(previous), _p(previous_index), R, V, _stream()), "repetition_penalty")
 
 
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,

@@ -32,9 +32,14 @@ class RowRequest:
     sampling: Optional[SamplingParams]          # None: greedy
     generated_before: int = 0                   # tokens the request has generated so far
     history: Sequence[int] = ()                 # prompt and generated tokens so far (for the penalty)
+    pending_row: int = -1                       # >= 0: the request's newest token is this entry of ``previous``
 
 
 class Sampler:
+    # a request's newest token may still be on the device (``RowRequest.pending_row``, ``previous``): the penalty
+    # finds it there, so a generation loop need not wait for a step's tokens before it launches the next
+    history_on_device = True
+
     def __init__(self, device: torch.device):
         self.device = device
         self._staging = None
@@ -58,8 +63,10 @@ class Sampler:
         """logits fp32 [R, V] on the device (left unchanged); one token per row."""
         return self.select_on_device(logits, rows).tolist()
 
-    def select_on_device(self, logits: torch.Tensor, rows: Sequence[RowRequest]) -> torch.Tensor:
-        """The same, with the tokens left on the device: int32 [R]."""
+    def select_on_device(self, logits: torch.Tensor, rows: Sequence[RowRequest],
+                         previous: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The same, with the tokens left on the device: int32 [R].  ``previous``: the tokens an earlier call left
+        on the device, for rows whose ``pending_row`` names one of them as their newest token."""
         R, V = logits.shape
         if R != len(rows):
             raise ValueError(f"{R} rows of logits for {len(rows)} requests")
@@ -95,12 +102,19 @@ class Sampler:
                 n = min(p.repetition_penalty_window, len(h))
                 tails.append(list(h[len(h) - n:]) if n else [])
             W = max(1, max(len(t) for t in tails))
-            ints = np.zeros(S * W + S, dtype=np.int32)           # the rows' tokens, then how many of each row count
-            for s, t in enumerate(tails):
+            # the rows' tokens, how many of each row count, and which token on the device is a row's newest
+            ints = np.zeros(S * W + 2 * S, dtype=np.int32)
+            pending = False
+            for s, (t, i) in enumerate(zip(tails, sampled)):
                 ints[s * W:s * W + len(t)] = t
                 ints[S * W + s] = len(t)
+                ints[S * W + S + s] = rows[i].pending_row
+                pending = pending or rows[i].pending_row >= 0
+            if pending and previous is None:
+                raise ValueError("a row's newest token is said to be on the device, but no tokens were given")
             dev_ints = self._to_device(ints)
-            K.repetition_penalty(work_logits, dev_ints[:S * W].view(S, W), dev_ints[S * W:], dev_nums[3])
+            K.repetition_penalty(work_logits, dev_ints[:S * W].view(S, W), dev_ints[S * W:S * W + S], dev_nums[3],
+                                 previous if pending else None, dev_ints[S * W + S:] if pending else None)
         picked = out if idx is None else torch.empty(S, dtype=torch.int32, device=logits.device)
         K.sample(work_logits, torch.empty_like(work_logits), dev_nums[0], dev_nums[1], dev_nums[2], picked)
         if idx is not None:

@@ -258,7 +258,7 @@ def test_one_step_ahead_changes_no_token(folders, num_blocks):
     d, cfg, w = folders["B"]
     g = torch.Generator().manual_seed(12)
     prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (9, 17, 6, 12, 5)]
-    probe = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=5, max_prefill_tokens=8)
+    probe = _runtime(d, "float32", block_size=4, num_blocks=64, max_batch_size=6, max_prefill_tokens=8)
     probe.look_ahead = False
     free_run = probe.generate(prompts[1], GenerateOptions(max_new_tokens=16))
     eos = free_run[9]                                          # request 1 stops where this token first comes
@@ -269,9 +269,14 @@ def test_one_step_ahead_changes_no_token(folders, num_blocks):
             GenerateOptions(max_new_tokens=1),
             GenerateOptions(max_new_tokens=15, sampling=SamplingParams(temperature=1.1, top_p=1.0, seed=5,
                                                                        repetition_penalty=1.0))]
+    # one more that looks back at its own tokens: its newest one is still on the device when the next is chosen
+    prompts.append(torch.randint(0, cfg["vocab_size"], (7,), generator=g).tolist())
+    opts.append(GenerateOptions(max_new_tokens=16, sampling=SamplingParams(temperature=0.9, top_p=0.95, seed=8,
+                                                                           repetition_penalty=1.3,
+                                                                           repetition_penalty_window=5)))
     results = {}
     for ahead in (False, True):
-        rt = _runtime(d, "float32", block_size=4, num_blocks=num_blocks, max_batch_size=5, max_prefill_tokens=8)
+        rt = _runtime(d, "float32", block_size=4, num_blocks=num_blocks, max_batch_size=6, max_prefill_tokens=8)
         assert rt.look_ahead
         rt.look_ahead = ahead
         with_device_tokens, real_step = [], rt.engine.step
@@ -291,11 +296,24 @@ def test_one_step_ahead_changes_no_token(folders, num_blocks):
         assert rt.engine.cache.free_pages() == num_blocks
     assert results[True] == results[False]
     assert results[True][1][0] == free_run[:free_run.index(eos)] and len(results[True][3][0]) == 1
+    # the penalty changed what the last request drew (the test would not see a lost token otherwise), and its tokens
+    # are the plain rule's over the plain model's logits
+    import plain_llama as P
+    from infernum_amd.sampling import token_uniform
+    toks, sp = list(prompts[5]), opts[5].sampling
+    differs = False
+    for i, tok in enumerate(results[True][5][0]):
+        logits = P.forward(cfg, w, toks)[-1]
+        u = token_uniform(sp.seed, i)
+        assert tok == P.sample_token(logits, sp.temperature, sp.top_p, u, sp.repetition_penalty, toks[-5:]), i
+        differs = differs or tok != P.sample_token(logits, sp.temperature, sp.top_p, u, 1.0, [])
+        toks.append(tok)
+    assert differs
 
 
 @pytest.mark.parametrize("seed", range(16))
 def test_one_step_ahead_under_random_loads(folders, seed):
-    """Random requests (greedy and sampled, some with a stop token) over pools so small that requests are set
+    """Random requests (greedy and sampled, some with a penalty on their last tokens, some with a stop token) over pools so small that requests are set
     back, with random limits of batch, portion and budget: in 32-bit, where a token's logits do not depend on what
     else is in its step, one step ahead and one step at a time give every request the same tokens and endings."""
     import random
@@ -310,7 +328,9 @@ def test_one_step_ahead_under_random_loads(folders, seed):
         opts = []
         for _ in range(n_req):
             sp = None if rng.random() < 0.5 else SamplingParams(temperature=rng.choice((0.3, 0.7, 1.2)),
-                                                               top_p=rng.choice((1.0, 0.9, 0.5)), seed=rng.randrange(1 << 30))
+                                                               top_p=rng.choice((1.0, 0.9, 0.5)), seed=rng.randrange(1 << 30),
+                                                               repetition_penalty=rng.choice((1.0, 1.2, 1.5)),
+                                                               repetition_penalty_window=rng.choice((1, 3, 64)))
             opts.append(GenerateOptions(max_new_tokens=rng.randint(1, 24), sampling=sp,
                                         eos_token_id=rng.randrange(vocab) if rng.random() < 0.5 else None))
         longest = max(len(p) + o.max_new_tokens for p, o in zip(prompts, opts))

@@ -946,6 +946,12 @@ def test_repetition_penalty():
     K().repetition_penalty(x, recent, counts, pen)
     # a token that stands twice is penalised twice (infernum-cuda/src/inner/cuda/ops/sample.rs:101-112)
     assert x.tolist() == [[0.5, -4.0, 1.0, 4.0], [2.0, -2.0, 1.0, 1.0]]
+    # a row's newest token may still be where an earlier launch left it: row 0 takes entry 2 of `previous` (token 1,
+    # once more), row 1 none
+    x = torch.tensor([[2.0, -2.0, 1.0, 4.0], [2.0, -2.0, 1.0, 4.0]], device=DEV)
+    previous = torch.tensor([3, 0, 1], dtype=torch.int32, device=DEV)
+    K().repetition_penalty(x, recent, counts, pen, previous, torch.tensor([2, -1], dtype=torch.int32, device=DEV))
+    assert x.tolist() == [[0.5, -8.0, 1.0, 4.0], [2.0, -2.0, 1.0, 1.0]]
 
 
 def _host_sample(logits, T, top_p, u):
