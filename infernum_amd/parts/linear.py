@@ -113,6 +113,8 @@ def _room_for_copy(w: torch.Tensor) -> bool:
     the steps' intermediates): a model that fills the memory keeps the file's layout for the rest of its weights
     (the same bits, a few per cent slower), where copies of all would leave no room for the cache."""
     free, total = torch.cuda.mem_get_info(w.device)
+    # what the allocator holds without using it counts as free: it hands that out again before it asks for more
+    free += torch.cuda.memory_reserved(w.device) - torch.cuda.memory_allocated(w.device)
     return free - w.numel() * w.element_size() >= COPIES_LEAVE_FREE * total
 
 

@@ -13,7 +13,7 @@ it stays as stored: fp32 stays fp32, integer tables become int32.
 from __future__ import annotations
 
 import fnmatch
-from typing import Dict, List
+from typing import Callable, Dict, Hashable, List
 
 import torch
 
@@ -79,17 +79,42 @@ def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], wher
     return source
 
 
+class LazyTensors:
+    """name -> tensor, made when a part asks for it: a model's parts are loaded one after the other, and what a part
+    does not keep (the three projections it has put into one matrix) is gone before the next part's tensors come, so
+    that loading needs the memory of the model and of one part's tensors, not twice the model's.  Names that share a
+    key share one tensor (a tied head and its embedding): ``make(name, key)`` is called once, for the name that asks
+    first, and the tensor is kept until the last of them has asked."""
+
+    def __init__(self, keys: Dict[str, Hashable], make: Callable[[str, Hashable], torch.Tensor]):
+        self._keys, self._make = dict(keys), make
+        self._left: Dict[Hashable, int] = {}
+        for key in self._keys.values():
+            self._left[key] = self._left.get(key, 0) + 1
+        self._kept: Dict[Hashable, torch.Tensor] = {}
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._keys
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        key = self._keys[name]
+        t = self._kept.get(key)
+        if t is None:
+            t = self._make(name, key)
+        self._left[key] -= 1
+        if self._left[key] > 0:
+            self._kept[key] = t
+        else:
+            self._kept.pop(key, None)
+        return t
+
+
 def load_weights(model, model_dir: str) -> None:
-    """Read every tensor the model expects from ``model_dir`` and hand them to its parts."""
+    """Read every tensor the model expects from ``model_dir`` and hand them to its parts, part by part."""
     rt: Runtime = model.rt
     expected = model.expected_weights()
     entries: Dict[str, TensorEntry] = open_model_tensors(model_dir)
     source = check_against(expected, {n: e.shape for n, e in entries.items()}, model_dir)
-    cache: Dict[tuple, torch.Tensor] = {}
-    tensors: Dict[str, torch.Tensor] = {}
-    for name, spec in expected.items():
-        key = (source[name], spec.follows_compute_dtype)
-        if key not in cache:                       # a tied head shares the embedding's buffer
-            cache[key] = _convert(entries[source[name]].read(), spec, rt)
-        tensors[name] = cache[key]
-    model.load_weights(tensors)
+    # a tied head shares the embedding's buffer: one key for both
+    keys = {name: (source[name], spec.follows_compute_dtype) for name, spec in expected.items()}
+    model.load_weights(LazyTensors(keys, lambda name, key: _convert(entries[key[0]].read(), expected[name], rt)))

@@ -140,17 +140,17 @@ def random_weights_on_device(model, seed: int, stored_as: Optional[torch.dtype] 
     compute type (a 32-bit model with ``stored_as=torch.bfloat16`` holds the numbers of the bfloat16 one)."""
     rt: Runtime = model.rt
     expected = model.expected_weights()
-    tensors: Dict[str, torch.Tensor] = {}
-    for name, spec in sorted(expected.items()):
-        if not spec.write_when_random and spec.fallback is not None:
-            continue                              # shares its fallback's buffer, below
+    from .loader import LazyTensors
+    # a tied head shares its fallback's buffer: the fallback's name is the key of both
+    keys = {name: spec.fallback if not spec.write_when_random and spec.fallback is not None else name
+            for name, spec in expected.items()}
+
+    def make(name: str, key: str) -> torch.Tensor:
         # what loading the folder that write_random_model(dtype=rt.dtype) writes would give: every tensor
         # rounded to that type once, also those that do not follow the compute type
-        tensors[name] = draw(spec, seed, name, rt.device).to(stored_as or rt.dtype).to(rt.dtype)
-    for name, spec in expected.items():          # a tied head whose fallback sorts after it
-        if name not in tensors:
-            tensors[name] = tensors[spec.fallback]
-    model.load_weights(tensors)
+        return draw(expected[key], seed, key, rt.device).to(stored_as or rt.dtype).to(rt.dtype)
+
+    model.load_weights(LazyTensors(keys, make))
 
 
 def main(argv: Optional[list] = None) -> int:

@@ -221,3 +221,36 @@ def test_random_values_are_a_function_of_the_element_alone(monkeypatch):
     assert 4.0 < z.abs().max().item() < 5.0
     u = R.draw(WeightSpec((1 << 16,), ("uniform", -1.0, 3.0)), 0, "u", torch.device("cpu")).double()
     assert -1.0 <= u.min().item() < -0.99 and 2.99 < u.max().item() < 3.0 and abs(u.mean().item() - 1.0) < 2e-2
+
+
+def test_tensors_come_part_by_part_and_a_shared_one_is_made_once(tmp_path):
+    """Loading asks for a part's tensors when that part is loaded and keeps none that the part did not keep, so the
+    originals of a fused matrix are gone before the next part's come; a tied head's tensor is made once."""
+    import weakref
+    from infernum_amd.weights.loader import LazyTensors
+    made = []
+    lazy = LazyTensors({"a": "k", "b": "k", "c": "c"}, lambda name, key: made.append((name, key)) or torch.zeros(3))
+    a = lazy["a"]
+    assert lazy["b"] is a and made == [("a", "k")] and "c" in lazy and "d" not in lazy
+    ref = weakref.ref(lazy["c"])
+    assert ref() is None and made == [("a", "k"), ("c", "c")]         # nothing but the caller held it
+    assert not lazy._kept                                              # the shared one was let go with its last name
+    # through the model: when a block's fused matrix is built, no tensor of an earlier block is alive any more
+    m = _model("A", torch.float32)
+    alive = []
+    expected = m.expected_weights()
+    keys = {n: n for n in expected}
+
+    def make(name, key):
+        assert not [r for r in alive if r[1]() is not None and r[0].split(".")[:3] != name.split(".")[:3]
+                    and "q_proj" in r[0]], name
+        t = torch.zeros(expected[name].shape)
+        alive.append((name, weakref.ref(t)))
+        return t
+
+    m.load_weights(LazyTensors(keys, make))
+    assert len(alive) == len(expected)
+    # the tied configuration on random weights: head and embedding are one buffer
+    from infernum_amd.weights.random_init import random_weights_on_device
+    random_weights_on_device(m, 3)
+    assert m.head.weight.data_ptr() == m.embedding.table.data_ptr()
