@@ -3,6 +3,7 @@ outside Python would: its output against ``ia_gemm_skinny``'s (the same kernels 
 caller brings) on two calls in a row, the second with a smaller input, so that what the first left in the
 library's array lies beside what the second writes."""
 import ctypes
+import gc
 
 import pytest
 import torch
@@ -76,6 +77,7 @@ def test_two_calls_in_a_row_give_what_the_workspace_entry_point_gives(first, sec
     for (M, N, K, epi) in (first, second):
         outs.append(torch.full((M, N // 2 if epi else N), float("nan"), dtype=out_dtype, device=DEV))
     torch.cuda.synchronize()
+    gc.collect()            # what earlier tests left in reference cycles goes now, not between the two readings
     before = torch.cuda.memory_allocated()
     for (M, N, K, epi), (x, w), out in zip((first, second), operands, outs):
         assert _no_alloc(lib, x, w, out, epi, stream) == 0
