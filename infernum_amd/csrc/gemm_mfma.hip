@@ -30,11 +30,13 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef const __attribute__((address_space(1))) void* gm_global_ptr;
 typedef __attribute__((address_space(3))) void* gm_lds_ptr;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X,
                                                                            const uint16_t* __restrict__ W,
-                                                                           uint16_t* __restrict__ C, int M, int N,
-                                                                           int K, int tiles_m, int tiles_n) {
+                                                                           uint16_t* __restrict__ C,
+                                                                           float* __restrict__ P, int M, int N,
+                                                                           int K, int tiles_m, int tiles_n,
+                                                                           int splits) {
   constexpr int WAVES = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // tile of a wave
   constexpr int TM = WM / 32, TN = WN / 32;             // in accumulator tiles of 32 x 32
@@ -49,9 +51,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
 
   // workgroups go to the 8 dies in turn (workgroup i to die i % 8), and each die has an L2 of its own:
   // give every die one contiguous run of tiles, so that W is read from memory once and not once per die
-  const int total = tiles_m * tiles_n;
+  const int tiles = tiles_m * tiles_n;
+  const int total = SPLIT ? tiles * splits : tiles;
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int bid = xcd * (total >> 3) + min(xcd, total & 7) + idx;
+  int bid = xcd * (total >> 3) + min(xcd, total & 7) + idx;
+  // with K split over workgroups, part p of every tile comes before part p + 1 of any: the tiles of M under one
+  // tile of N still run side by side on one die
+  const int part = SPLIT ? bid / tiles : 0;
+  bid -= part * tiles;
   // 8 tiles of M under one tile of N at a time
   const int GROUP = 8;
   const int per_group = GROUP * tiles_n;
@@ -78,7 +85,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
   }
 #define GM_FILL(f, kt, buf)                                                                                  \
   __builtin_amdgcn_global_load_lds(                                                                         \
-      (gm_global_ptr)(reinterpret_cast<const char*>((8 * (f) * WAVES < BM) ? X : W) + (size_t)(kt) * GM_ROW_BYTES + \
+      (gm_global_ptr)(reinterpret_cast<const char*>((8 * (f) * WAVES < BM) ? X : W) + (size_t)(k_first + (kt)) * GM_ROW_BYTES + \
                       src[f]),                                                                              \
       (gm_lds_ptr)(lds + (buf) * STAGE_BYTES + 1024 * ((f) * WAVES + wave)), 16, 0, 0)
 
@@ -94,7 +101,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
 
   // stage j of LDS holds steps j, j + STAGES, ..: while step kt is worked on, step kt + STAGES - 1 is
   // fetched into the stage that step kt - 1 has left
-  const int ksteps = K / GM_BK;
+  // a part takes a run of the steps of K; the steps are dealt out evenly, the first parts one more
+  const int ksteps_all = K / GM_BK;
+  const int k_first = SPLIT ? part * (ksteps_all / splits) + min(part, ksteps_all % splits) : 0;
+  const int ksteps = SPLIT ? ksteps_all / splits + (part < ksteps_all % splits ? 1 : 0) : ksteps_all;
 #pragma unroll
   for (int j = 0; j < STAGES - 1; ++j)
 #pragma unroll
@@ -177,6 +187,34 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
   // wave's part leaves as consecutive 16-byte pieces (the accumulators hold 4 values of a row per lane, 32
   // rows apart from lane to lane).  Every wave has a region of its own, WM rows of WN values; the 16-byte
   // piece c of row m lies at position c ^ (m % CP): the lanes of a store instruction write 32 different rows.
+  if constexpr (SPLIT) {
+    // the sums of this part of K, fp32, into part `part` of P [splits, M, N]: whoever reads them adds the parts in
+    // the order of their index
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the loads asked for past the end write LDS too
+    float* const pp = P + (size_t)part * M * N;
+    const bool vec4 = (N & 3) == 0;
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+      for (int b = 0; b < TM; ++b) {
+        const int m = m0 + wm * WM + b * 32 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = n0 + wn * WN + a * 32 + 8 * g + 4 * lh;
+          float* dstp = pp + (size_t)m * N + n;
+          if (vec4 && n + 3 < N) {
+            *reinterpret_cast<float4*>(dstp) =
+                make_float4(acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2], acc[a][b][4 * g + 3]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) dstp[e] = acc[a][b][4 * g + e];
+          }
+        }
+      }
+    return;
+  }
   constexpr int CP = WN / 8;                        // 16-byte pieces per row of a wave's part
   static_assert(STAGES * STAGE_BYTES >= WAVES * WM * WN * 2, "the stages must hold the tile of C");
   if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
@@ -236,34 +274,38 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS>
-static int launch_gemm_mfma(const uint16_t* x, const uint16_t* w, uint16_t* c, int M, int N, int K,
-                            hipStream_t stream) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT>
+static int launch_gemm_mfma(const uint16_t* x, const uint16_t* w, uint16_t* c, float* parts, int M, int N, int K,
+                            int splits, hipStream_t stream) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds_bytes = (size_t)STAGES * (BM + BN) * GM_ROW_BYTES;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  if ((long long)tiles_m * tiles_n > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
-  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS><<<tiles_m * tiles_n, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
-      x, w, c, M, N, K, tiles_m, tiles_n);
+  if ((long long)tiles_m * tiles_n * splits > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
+  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT>
+      <<<tiles_m * tiles_n * splits, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(x, w, c, parts, M, N, K, tiles_m,
+                                                                                  tiles_n, splits);
   IA_LAUNCH_CHECK();
   return IA_OK;
+}
+
+static bool gemm_mfma_takes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || (K % GM_BK) != 0) return false;
+  // rows are addressed with 32-bit byte offsets
+  return (unsigned long long)M * K * 2 <= 0xffffffffULL && (unsigned long long)N * K * 2 <= 0xffffffffULL;
 }
 
 // X [M, K], W [N, K], C [M, N]: bf16, contiguous.  tile: 0 = chosen here, 1 = 256 x 256 (two stages),
 // 2 = 128 x 256 (three stages), 3 = 128 x 128 (four stages).
 extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int tile,
                             hipStream_t stream) {
-  if (M <= 0 || N <= 0 || K <= 0 || (K % GM_BK) != 0) return IA_ERR_UNSUPPORTED;
-  // rows are addressed with 32-bit byte offsets
-  if ((unsigned long long)M * K * 2 > 0xffffffffULL || (unsigned long long)N * K * 2 > 0xffffffffULL)
-    return IA_ERR_UNSUPPORTED;
+  if (!gemm_mfma_takes(M, N, K)) return IA_ERR_UNSUPPORTED;
   const uint16_t* x = (const uint16_t*)X;
   const uint16_t* w = (const uint16_t*)W;
   uint16_t* c = (uint16_t*)C;
@@ -276,12 +318,25 @@ extern "C" int ia_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
   }
   // the later stage's loads go out during the first two quarters of a step where the tile is large
   // (measured best), during the first for the small tile
-  if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2, 2>(x, w, c, M, N, K, stream);
-  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3, 2>(x, w, c, M, N, K, stream);
-  if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4, 1>(x, w, c, M, N, K, stream);
+  if (tile == 1) return launch_gemm_mfma<256, 256, 2, 2, 2, 2, false>(x, w, c, nullptr, M, N, K, 1, stream);
+  if (tile == 2) return launch_gemm_mfma<128, 256, 2, 2, 3, 2, false>(x, w, c, nullptr, M, N, K, 1, stream);
+  if (tile == 3) return launch_gemm_mfma<128, 128, 2, 2, 4, 1, false>(x, w, c, nullptr, M, N, K, 1, stream);
   return IA_ERR_BAD_ARG;
+}
+
+// The same product for a few hundred rows, where the tiles of C alone are fewer than the compute units: K is
+// split over `splits` workgroups per tile of 128 x 128, and the fp32 sums of part p go to parts[p] of
+// parts [splits, M, N] for the next kernel to add in the order of their index (the weight is then read at the
+// memory's rate, as in the product for few rows).  1 <= splits <= K / 64.
+extern "C" int ia_gemm_mfma_split(const void* X, const void* W, float* parts, int M, int N, int K, int splits,
+                                  hipStream_t stream) {
+  if (!gemm_mfma_takes(M, N, K)) return IA_ERR_UNSUPPORTED;
+  if (splits < 1 || splits > K / GM_BK || !parts) return IA_ERR_BAD_ARG;
+  return launch_gemm_mfma<128, 128, 2, 2, 4, 1, true>((const uint16_t*)X, (const uint16_t*)W, nullptr, parts, M, N, K,
+                                                      splits, stream);
 }
 
 // ---- the launchers of this file as operations of a step's program (see op_call.h) ----
 #include "op_call.h"
 IA_OP(ia_gemm_mfma)
+IA_OP(ia_gemm_mfma_split)

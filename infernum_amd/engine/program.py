@@ -455,6 +455,7 @@ class StepProgram:
             self._check(add(self._h, fn, name.encode(), A, len(flat) // 4, G, len(terms) // 5, int(if_unsupported)))
         self._check(self._lib.ia_program_finish(self._h, len(self._vars), len(self._ptrs)))
         self.num_ops = len(self._ops)
+        self.op_names = [op[1] for op in self._ops]              # the launchers, in the program's order
         self.num_python_ops = sum(1 for op in self._ops if op[1].startswith("python:"))   # parts called back into
         self._ops = []
         self._finished = True

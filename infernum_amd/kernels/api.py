@@ -357,6 +357,26 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     return out
 
 
+def gemm_mfma_split(a: torch.Tensor, w: torch.Tensor, splits: int, parts: Optional[torch.Tensor] = None) -> SplitSum:
+    """a[M, K] @ w[N, K]^T for a few hundred rows as fp32 partial sums [splits, M, N]: the LDS-tiled MFMA product
+    with tiles of 128 x 128 and K split over ``splits`` workgroups a tile, so that the launch fills the GPU where the
+    tiles alone would not and the weight comes at the memory's rate; the next kernel adds the parts."""
+    _dev(a, w, parts)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_mfma_split: shapes")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_mfma_split: bf16 operands")
+    _need(a.is_contiguous() and w.is_contiguous(), "gemm_mfma_split: contiguous operands")
+    _need(gemm_mfma_supported(M, N, K), f"gemm_mfma_split: M={M} N={N} K={K} not supported (K % 64 == 0, below 4 GiB)")
+    _need(1 <= splits <= K // 64, f"gemm_mfma_split: {splits} parts of K={K} (1 to K / 64)")
+    if parts is None:
+        parts = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+    _need(parts.dtype == torch.float32 and parts.is_contiguous() and tuple(parts.shape) == (splits, M, N),
+          f"gemm_mfma_split: parts must be contiguous fp32 [{splits}, {M}, {N}]")
+    _ok(_core().ia_gemm_mfma_split(_p(a), _p(w), _p(parts), M, N, K, splits, _stream()), "gemm_mfma_split")
+    return SplitSum(parts)
+
+
 LIBRARY_WORKSPACE_BYTES = 128 << 20
 _library_workspace: Dict[torch.device, torch.Tensor] = {}
 

@@ -14,8 +14,11 @@ bf16: up to 128 rows the hand-written MFMA kernel that streams the weight once, 
 (hipBLASLt, called directly with its choice of an algorithm kept per shape) where that is known to be faster for
 the weight's shape (:data:`KNOWN_ROUTES`, a table that is part of the source, so that two runs of one model make
 the same launches; ``INFERNUM_GEMM_ROUTE=measured`` times both when a model loads instead, ``static`` keeps to
-the rule of sizes); above 128 rows the library, as the reference uses its library there; an fp32 result of many
-rows comes 128 rows at a time from the hand-written kernel.  ``set_prefill_gemm("mfma")`` (or
+the rule of sizes); from 129 to 256 rows the LDS-tiled MFMA kernel with K split over workgroups for the weights
+of :data:`KNOWN_MID_ROWS` whose partial sums the next kernel takes (the library's kernels for so few rows leave
+most of the GPU idle); above that the library, as the reference uses its library there; an fp32 result of more
+than 128 rows comes from the LDS-tiled kernel's fp32 sums (128 rows at a time from the weight-streaming kernel where
+the tiled one does not take the size).  ``set_prefill_gemm("mfma")`` (or
 INFERNUM_PREFILL_GEMM=mfma) sends the many-row bf16 products to the hand-written LDS-tiled MFMA kernel instead,
 where it takes the size (K in steps of 64).
 
@@ -60,6 +63,18 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
     (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
 }
 
+# (N, K) of a weight whose product leaves partial sums for the next kernel -> the parts K is split into by the
+# LDS-tiled MFMA kernel from 129 to 256 rows (two tiles of 128 rows over N / 128 tiles of columns: the parts bring
+# the workgroups to about one a compute unit).  Measured on an MI355X against the library's product with cold
+# weights, microseconds at 129 / 192 / 256 rows: the 8B shape's down projection 37 / 41 / 45 against 58 / 104 / 63,
+# its output projection 17 / 18 / 19 against 22 / 34 / 23, its QKV product 23 / 24 / 26 against 40 / 35 / 42 (the
+# rotary kernel then adds the two parts).  The 8B shape's decode step at 160 / 192 / 256 requests: 19.8k / 21.4k /
+# 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
+MID_ROWS = (129, 256)
+KNOWN_MID_ROWS: Dict[Tuple[int, int], int] = {
+    (4096, 14336): 4, (4096, 4096): 4, (6144, 4096): 2,
+}
+
 ROUTES = ("table", "measured", "static")
 _route = os.environ.get("INFERNUM_GEMM_ROUTE", "table")
 if _route not in ROUTES:
@@ -96,6 +111,15 @@ def library_rows(N: int, K_: int, epilogue: Optional[str], keep_split: bool) -> 
     if mask < 0:
         mask = 0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1)
     return mask & 0xFE             # up to 16 rows the weight-streaming kernel, always
+
+
+def mid_rows_parts(N: int, K_: int, keep_split: bool) -> int:
+    """Into how many parts the LDS-tiled kernel splits K for MID_ROWS rows of a product with this weight, 0 where
+    the library takes those rows."""
+    if not keep_split or _route != "table" or _prefill_gemm != "library":
+        return 0
+    parts = KNOWN_MID_ROWS.get((N, K_), 0)
+    return parts if parts and K.gemm_mfma_supported(MID_ROWS[1], N, K_) and parts <= K_ // 64 else 0
 
 
 def tiled_copy(w: torch.Tensor, epilogue: Optional[str]) -> Optional[torch.Tensor]:
@@ -216,11 +240,16 @@ class Route:
     (fp32 multiply-adds in a fixed order), "skinny" (the weight-streaming kernel, its parts joined, the
     activation in its epilogue), "skinny_split" (the same with its partial sums left for the next kernel),
     "skinny_rows" (128 rows at a time), "library" (hipBLASLt; ``fallback`` names the kernel for a shape it
-    refuses), "mfma" (the LDS-tiled kernel)."""
+    refuses), "mfma" (the LDS-tiled kernel), "mfma_split" (the same with K split into ``parts``, its partial
+    sums left for the next kernel), "mfma_f32" (the same in one part: an fp32 result from bf16 operands).  A route
+    with ``rows`` (first, last) takes those numbers of rows only, and takes them from the routes without that stand
+    behind it."""
 
     blocks: int
     kind: str
     fallback: Optional[str] = None
+    rows: Optional[Tuple[int, int]] = None
+    parts: int = 0
 
 
 _MANY_ROWS = 65536         # the LDS-tiled kernel addresses rows with 32 bits: its fitness is judged at this many
@@ -244,25 +273,37 @@ def plan(N: int, Kdim: int, dtype: torch.dtype, out_dtype: torch.dtype, epilogue
     if out_dtype != torch.bfloat16:
         if epilogue is not None:
             raise K.KernelError("linear: an fp32 result from bf16 operands has no activation here")
-        return [Route(_UP_TO_128, own), Route(ALL_BLOCKS & ~_UP_TO_128, "skinny_rows")]
+        # more than 128 rows (the head of a step that wants the logits of many places): the LDS-tiled kernel leaving
+        # its fp32 sums (one part), which reads the weight once per 128 x 128 tile of the result where the
+        # weight-streaming kernel reads all of it for every 128 rows (the head of 128,256 x 4,096 on an MI355X:
+        # 371 against 649 us at 256 rows, 2.6 against 4.9 ms at 2,048)
+        return [Route(_UP_TO_128, own),
+                Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_f32" if tiled_fits else "skinny_rows")]
     to_library = library_rows(N, Kdim, epilogue, keep_split) if _prefill_gemm == "library" else \
         (0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1))
-    routes = [Route(_UP_TO_128 & ~to_library, own),
-              Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback)]
+    routes = [Route(_UP_TO_128 & ~to_library, own)]
+    mid = mid_rows_parts(N, Kdim, keep_split and epilogue is None)
+    if mid:
+        routes.append(Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_split", rows=MID_ROWS, parts=mid))
+    routes.append(Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback))
     return [r for r in routes if r.blocks]
 
 
 def route_of(routes: List[Route], M: int) -> Route:
     bit = 1 << min((M - 1) // 16, 8)
     for r in routes:
-        if r.blocks & bit:
+        if r.blocks & bit and (r.rows is None or r.rows[0] <= M <= r.rows[1]):
             return r
     raise K.KernelError(f"linear: no route for {M} rows")
 
 
 def _run(kind: str, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, epilogue: Optional[str],
-         fallback: Optional[str] = None):
+         fallback: Optional[str] = None, parts: int = 0):
     M, N = x.shape[0], w.shape[0]
+    if kind == "mfma_split":
+        return K.gemm_mfma_split(x, w, parts), True
+    if kind == "mfma_f32":
+        return K.gemm_mfma_split(x, w, 1).parts[0], True
     if kind == "skinny":
         return K.gemm_skinny(x, w, epilogue=epilogue, out_dtype=out_dtype, tiled=tiled_copy(w, epilogue)), True
     if kind == "skinny_split":
@@ -293,7 +334,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if not x.is_contiguous():
         x = x.contiguous()
     route = route_of(plan(N, Kdim, x.dtype, out_dtype, epilogue, keep_split, kernels), M)
-    y, activated = _run(route.kind, x, w, out_dtype, epilogue, route.fallback)
+    y, activated = _run(route.kind, x, w, out_dtype, epilogue, route.fallback, route.parts)
     if epilogue == "swiglu" and not activated:
         return K.swiglu(y, torch.empty((M, N // 2), dtype=y.dtype, device=y.device))
     return y
@@ -320,15 +361,32 @@ def emit_linear(program, x: Any, M: Any, w: torch.Tensor, out_dtype: torch.dtype
         size = T * n_out * out_bytes
         if any(r.kind == "skinny_split" for r in routes):
             size = max(size, splits * small * N * 4)
+        for r in routes:
+            if r.kind == "mfma_split":
+                size = max(size, r.parts * min(T, r.rows[1]) * N * 4)
         out = program.buffer(out, size)
     code, in_code = K.DTYPE_CODE[out_dtype], K.DTYPE_CODE[rt.dtype]
     tiled = tiled_copy(w, epilogue)
     skinny, wk = ("ia_gemm_skinny_tiled", tiled) if tiled is not None else ("ia_gemm_skinny", w)
     program.keep(w, tiled)
     alts = []
+    ranged = P.NEVER                   # the rows that routes with a range of their own have taken
     for r in routes:
         g = when & P.Guard.blocks(M, r.blocks)
+        if r.rows is not None:
+            own_rows = P.Guard.between(M, r.rows[0], r.rows[1])
+            g, ranged = g & own_rows & ~ranged, ranged | own_rows
+        else:
+            g = g & ~ranged
         if g.never:
+            continue
+        if r.kind == "mfma_split":
+            program.op("core", "ia_gemm_mfma_split", [x, w, out, M, N, Kdim, r.parts, P.STREAM], g)
+            alts.append(P.Alt(g, out, r.parts, torch.float32))
+            continue
+        if r.kind == "mfma_f32":                # one part: the fp32 matrix itself
+            program.op("core", "ia_gemm_mfma_split", [x, w, out, M, N, Kdim, 1, P.STREAM], g)
+            alts.append(P.Alt(g, out, 0, out_dtype))
             continue
         if r.kind == "skinny_split":
             program.op("core", skinny, [x, wk, None, 0, M, N, Kdim, 0, out, M * (splits * N), P.STREAM], g)

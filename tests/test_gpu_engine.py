@@ -91,6 +91,35 @@ def test_whole_with_the_hand_written_prefill_gemm(models):
     assert worst <= 2e-2 * rms, f"own and library products differ by {worst:.3e} at {where}"
 
 
+def test_steps_of_129_to_256_rows_through_the_tiled_kernel_with_k_split(models, monkeypatch):
+    """Configuration B with its output projection (and, beyond what the table of the source holds, its QKV product)
+    sent to the LDS-tiled kernel with K split in two for steps of 129 to 256 tokens: the norm and the rotary kernel
+    add the partial sums.  Whole prompts of 129 to 200 tokens are such steps; the mixed trace has them beside
+    smaller and larger ones.  Against the plain model, and the host library's program against the parts' calls."""
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    d, cfg, reqs, ref = models[("B", "bfloat16", "mixed")]
+    H, nh, nkv = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    hd = H // nh
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, (H, nh * hd), 2)
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, ((nh + 2 * nkv) * hd, H), 2)
+    kinds = {M: L.route_of(L.plan(H, nh * hd, torch.bfloat16, torch.bfloat16, None, True), M).kind for M in (128, 129, 256, 257)}
+    assert kinds == {128: "skinny", 129: "mfma_split", 256: "mfma_split", 257: "library"}      # K of 128: one part up to 128 rows
+    assert sum(129 <= len(t) <= 256 for t in reqs.values()) >= 4
+    native = _engine(d, "bfloat16", PAGE["B"], 128)
+    parts = _engine(d, "bfloat16", PAGE["B"], 128, executor="parts")
+    assert "ia_gemm_mfma_split" in native.program.op_names
+    a, b = TT.run_steps(native, TT.trace_whole(reqs)), TT.run_steps(parts, TT.trace_whole(reqs))
+    _check(a, ref, "bfloat16", "B bfloat16 whole, 129 to 256 rows on the split tiled kernel")
+    assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
+    native.program.check_guards()
+    prompt_len = {r: max(2, len(t) - 20) for r, t in reqs.items()}
+    mixed, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=5)
+    eng = _engine(d, "bfloat16", PAGE["B"], max_tokens // PAGE["B"])
+    _check(TT.run_steps(eng, mixed), ref, "bfloat16", "B bfloat16 mixed, split tiled kernel", every_place=False)
+    eng.program.check_guards()
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_tail_one_by_one_rotation_inside_attention_or_before_it(models, name):
     """Steps of single tokens rotate queries and keys and write the pages inside the attention kernel; with the

@@ -411,6 +411,60 @@ def test_gemm_mfma_picks_out_one_product():
     assert torch.equal(api.gemm_mfma(a, w).float(), want)
 
 
+@pytest.mark.parametrize("M,N,K_,S", [(129, 250, 64, 1), (256, 516, 1024, 4), (200, 1003, 448, 3), (300, 328, 448, 7),
+                                      (130, 7, 128, 2), (512, 384, 320, 5)])
+def test_gemm_mfma_split(M, N, K_, S):
+    """The LDS-tiled product with K split over workgroups: part p of the result holds the fp32 sums over its run of
+    the steps of 64 (dealt out evenly, the first parts one more), at sizes that fill no tile, with rows of N that
+    are no multiple of 4 (scalar stores), one step a part and many."""
+    api = K()
+    a, w = _rand(M, K_, dtype=torch.bfloat16, seed=8), _rand(N, K_, dtype=torch.bfloat16, scale=0.1, seed=9)
+    parts = torch.full((S, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    got = api.gemm_mfma_split(a, w, S, parts)
+    assert got.parts.data_ptr() == parts.data_ptr() and tuple(got.shape) == (M, N)
+    steps, first = K_ // 64, 0
+    for p in range(S):
+        n = steps // S + (1 if p < steps % S else 0)
+        ka, kb = 64 * first, 64 * (first + n)
+        want = a[:, ka:kb].double() @ w[:, ka:kb].double().t()
+        assert bool(((parts[p].double() - want).abs() <= 2e-6 * math.sqrt(kb - ka) * 0.1 + 2e-6 * want.abs()).all()), p
+        first += n
+    # the parts added in the order of their index and rounded once are what the whole product gives (the same
+    # sums in the same order within a part; across parts fp32 additions): within one rounding to bf16
+    whole = api.gemm_mfma(a, w, tile="128x128")
+    joined = got.joined(torch.bfloat16)
+    want = a.double() @ w.double().t()
+    assert bool(((joined.double() - want).abs() <= 2e-5 * math.sqrt(K_) * 0.1 + 2.0 ** -8 * want.abs()).all())
+    assert bool(((joined.double() - whole.double()).abs() <= 2.0 ** -7 * want.abs() + 1e-6).all())
+    # a row's sums do not depend on the rows beside it
+    last = api.gemm_mfma_split(a[M - 1:M].contiguous(), w, S)
+    assert torch.equal(last.parts[:, 0], parts[:, M - 1])
+
+
+def test_gemm_mfma_split_picks_out_one_product_and_refuses_what_it_cannot_do():
+    api = K()
+    M, N, K_, S = 200, 771, 448, 3                      # 7 steps of K: parts of 3, 2 and 2
+    a = torch.zeros(M, K_, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(N, K_, dtype=torch.bfloat16, device=DEV)
+    spots = [(0, 0, 0, 0), (M - 1, N - 1, K_ - 1, 2), (128, 255, 192, 1), (129, 513, 191, 0), (77, 2, 320, 2)]
+    for i, (m, n, k, p) in enumerate(spots):
+        a[m, k] = 1 + i
+        w[n, k] = 2
+    got = api.gemm_mfma_split(a, w, S).parts
+    want = torch.zeros(S, M, N, device=DEV)
+    for i, (m, n, k, p) in enumerate(spots):
+        want[p, m, n] = 2 * (1 + i)
+    assert torch.equal(got, want)
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_split(a, w, 8)                                                                # more parts than steps
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_split(a, w, 0)
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_split(_rand(80, 96, dtype=torch.bfloat16), _rand(32, 96, dtype=torch.bfloat16), 1)   # K % 64
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_split(a, w, S, torch.empty(S, M, N + 1, device=DEV))                           # parts' shape
+
+
 def test_gemm_mfma_refuses_what_it_cannot_do():
     api = K()
     with pytest.raises(api.KernelError):
@@ -503,6 +557,24 @@ def test_linear_fp32_result_of_many_rows_from_bf16_operands():
     assert y.dtype == torch.float32 and (y.double() - want).abs().max().item() <= 2e-5 * 10 * 0.1
     for m in (1, 128, 129, 256, 257):
         assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
+
+
+def test_linear_fp32_result_of_many_rows_by_the_tiled_kernel():
+    """Where the LDS-tiled kernel takes the size (K in steps of 64), the fp32 result of more than 128 rows is its
+    one part of fp32 sums: every row as exact as the weight-streaming kernel's, whatever rows stand beside it."""
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    x, w = _rand(300, 192, dtype=torch.bfloat16, seed=5), _rand(1003, 192, dtype=torch.bfloat16, scale=0.1, seed=6)
+    assert [r.kind for r in L.plan(1003, 192, torch.bfloat16, torch.float32, None, False)] == ["skinny", "mfma_f32"]
+    y = L.linear(x, w, out_dtype=torch.float32)
+    want = x.double() @ w.double().t()
+    assert y.dtype == torch.float32 and tuple(y.shape) == (300, 1003)
+    assert (y.double() - want).abs().max().item() <= 2e-5 * 14 * 0.1
+    for m in (129, 256, 257):
+        assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
+    few = L.linear(x[:128].contiguous(), w, out_dtype=torch.float32)           # the weight-streaming kernel
+    assert (few.double() - want[:128]).abs().max().item() <= 2e-5 * 14 * 0.1
+    assert (few - y[:128]).abs().max().item() <= 4e-6 * 14 * 0.1
 
 
 @pytest.mark.parametrize("N,Kd,epilogue", [(28672, 4096, "swiglu"), (330, 264, "swiglu"), (1000, 96, None), (6144, 512, None),

@@ -57,6 +57,7 @@ def test_the_product_plan_covers_every_number_of_rows_once(monkeypatch):
     L = importlib.import_module("infernum_amd.parts.linear")
     # the number of parts of a split product is the kernel library's to say; any rule serves here
     monkeypatch.setattr(L.K, "gemm_skinny_splits", lambda N, K: 4 if N < 8192 else 1)
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, (48, 4096), 3)      # beside the shapes the table holds
     try:
         for N, Kd in itertools.product((48, 4096, 28672, 16385), (64, 4096, 100, 14336)):
             for dtype, out, epi, keep, kernels in itertools.product(
@@ -68,8 +69,14 @@ def test_the_product_plan_covers_every_number_of_rows_once(monkeypatch):
                     L.set_gemm_route(route)
                     seen = 0
                     for r in L.plan(N, Kd, dtype, out, epi, keep, kernels):
+                        if r.rows is not None:                 # a route for a range of rows: ahead of the one it takes from
+                            assert r.blocks == 1 << 8 and 129 <= r.rows[0] <= r.rows[1] and not (seen & r.blocks)
+                            assert r.kind == "mfma_split" and r.parts >= 1 and keep and epi is None
+                            continue
                         assert r.blocks and not (seen & r.blocks)
                         seen |= r.blocks
                     assert seen == L.ALL_BLOCKS
+                    for M in (1, 16, 17, 64, 65, 128, 129, 200, 256, 257, 5000):
+                        assert L.route_of(L.plan(N, Kd, dtype, out, epi, keep, kernels), M) is not None
     finally:
         L.set_gemm_route("table")
