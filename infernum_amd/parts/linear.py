@@ -14,7 +14,7 @@ bf16: up to 128 rows the hand-written MFMA kernel that streams the weight once, 
 (hipBLASLt, called directly with its choice of an algorithm kept per shape) where that is known to be faster for
 the weight's shape (:data:`KNOWN_ROUTES`, a table that is part of the source, so that two runs of one model make
 the same launches; ``INFERNUM_GEMM_ROUTE=measured`` times both when a model loads instead, ``static`` keeps to
-the rule of sizes); from 129 to 256 rows the LDS-tiled MFMA kernel with K split over workgroups for the weights
+the rule of sizes); for a few hundred rows the LDS-tiled MFMA kernel with K split over workgroups for the weights
 of :data:`KNOWN_MID_ROWS` whose partial sums the next kernel takes (the library's kernels for so few rows leave
 most of the GPU idle); above that the library, as the reference uses its library there; an fp32 result of more
 than 128 rows comes from the LDS-tiled kernel's fp32 sums (128 rows at a time from the weight-streaming kernel where
@@ -63,16 +63,22 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
     (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
 }
 
-# (N, K) of a weight whose product leaves partial sums for the next kernel -> the parts K is split into by the
-# LDS-tiled MFMA kernel from 129 to 256 rows (two tiles of 128 rows over N / 128 tiles of columns: the parts bring
-# the workgroups to about one a compute unit).  Measured on an MI355X against the library's product with cold
-# weights, microseconds at 129 / 192 / 256 rows: the 8B shape's down projection 37 / 41 / 45 against 58 / 104 / 63,
-# its output projection 17 / 18 / 19 against 22 / 34 / 23, its QKV product 23 / 24 / 26 against 40 / 35 / 42 (the
-# rotary kernel then adds the two parts).  The 8B shape's decode step at 160 / 192 / 256 requests: 19.8k / 21.4k /
-# 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
-MID_ROWS = (129, 256)
-KNOWN_MID_ROWS: Dict[Tuple[int, int], int] = {
-    (4096, 14336): 4, (4096, 4096): 4, (6144, 4096): 2,
+# (N, K) of a weight whose product leaves partial sums for the next kernel -> (first row, last row, parts): for
+# these numbers of rows the LDS-tiled MFMA kernel takes the product with K split into so many parts (tiles of
+# 128 x 128 of the result: the parts bring the workgroups to about one a compute unit, which is what was fastest
+# for every shape).  Measured on an MI355X against the library's product with cold weights, microseconds at
+# 129 / 192 / 256 rows: the 8B shape's down projection 37 / 41 / 45 against 58 / 104 / 63, its output projection
+# 17 / 18 / 19 against 22 / 34 / 23, its QKV product 23 / 24 / 26 against 40 / 35 / 42 (the rotary kernel then adds
+# the two parts); the 13B shape's down projection 43 / 47 / 53 against 54 / 100 / 120, the 70B shape's 165 / 155 /
+# 163 against 298 / 231 / 312, the 1B shape's 16 / 17 / 18 against 27 / 27 / 27.  At 384 rows: the 8B shape's down
+# projection 73 against 79, the 13B shape's 72 against 91, the 1B shape's 22 against 34.  Shapes whose QKV or output
+# projection came out even with the library's stay with it.  The 8B shape's decode step at 160 / 192 / 256 requests:
+# 19.8k / 21.4k / 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
+KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
+    (2048, 8192): ((129, 256, 8), (257, 384, 5), (385, 512, 4)),
+    (4096, 14336): ((129, 256, 4), (257, 384, 2)), (4096, 4096): ((129, 256, 4),), (6144, 4096): ((129, 256, 2),),
+    (5120, 13824): ((129, 256, 3), (257, 384, 2)), (5120, 5120): ((129, 256, 3), (257, 384, 2)),
+    (8192, 28672): ((129, 256, 2),), (8192, 8192): ((129, 256, 2),),
 }
 
 ROUTES = ("table", "measured", "static")
@@ -113,13 +119,13 @@ def library_rows(N: int, K_: int, epilogue: Optional[str], keep_split: bool) -> 
     return mask & 0xFE             # up to 16 rows the weight-streaming kernel, always
 
 
-def mid_rows_parts(N: int, K_: int, keep_split: bool) -> int:
-    """Into how many parts the LDS-tiled kernel splits K for MID_ROWS rows of a product with this weight, 0 where
-    the library takes those rows."""
+def mid_rows(N: int, K_: int, keep_split: bool) -> Tuple[Tuple[int, int, int], ...]:
+    """(first row, last row, parts) for which the LDS-tiled kernel, K split into ``parts``, takes the product with
+    this weight; none where the library takes every number of rows above 128."""
     if not keep_split or _route != "table" or _prefill_gemm != "library":
-        return 0
-    parts = KNOWN_MID_ROWS.get((N, K_), 0)
-    return parts if parts and K.gemm_mfma_supported(MID_ROWS[1], N, K_) and parts <= K_ // 64 else 0
+        return ()
+    return tuple((lo, hi, parts) for lo, hi, parts in KNOWN_MID_ROWS.get((N, K_), ())
+                 if lo > K.SKINNY_MAX_M and K.gemm_mfma_supported(hi, N, K_) and 1 <= parts <= K_ // 64)
 
 
 def tiled_copy(w: torch.Tensor, epilogue: Optional[str]) -> Optional[torch.Tensor]:
@@ -282,9 +288,8 @@ def plan(N: int, Kdim: int, dtype: torch.dtype, out_dtype: torch.dtype, epilogue
     to_library = library_rows(N, Kdim, epilogue, keep_split) if _prefill_gemm == "library" else \
         (0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1))
     routes = [Route(_UP_TO_128 & ~to_library, own)]
-    mid = mid_rows_parts(N, Kdim, keep_split and epilogue is None)
-    if mid:
-        routes.append(Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_split", rows=MID_ROWS, parts=mid))
+    for lo, hi, parts in mid_rows(N, Kdim, keep_split and epilogue is None):
+        routes.append(Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_split", rows=(lo, hi), parts=parts))
     routes.append(Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback))
     return [r for r in routes if r.blocks]
 

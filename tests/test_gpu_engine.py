@@ -101,8 +101,8 @@ def test_steps_of_129_to_256_rows_through_the_tiled_kernel_with_k_split(models, 
     d, cfg, reqs, ref = models[("B", "bfloat16", "mixed")]
     H, nh, nkv = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
     hd = H // nh
-    monkeypatch.setitem(L.KNOWN_MID_ROWS, (H, nh * hd), 2)
-    monkeypatch.setitem(L.KNOWN_MID_ROWS, ((nh + 2 * nkv) * hd, H), 2)
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, (H, nh * hd), ((129, 256, 2),))
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, ((nh + 2 * nkv) * hd, H), ((129, 160, 2), (161, 256, 1)))
     kinds = {M: L.route_of(L.plan(H, nh * hd, torch.bfloat16, torch.bfloat16, None, True), M).kind for M in (128, 129, 256, 257)}
     assert kinds == {128: "skinny", 129: "mfma_split", 256: "mfma_split", 257: "library"}      # K of 128: one part up to 128 rows
     assert sum(129 <= len(t) <= 256 for t in reqs.values()) >= 4

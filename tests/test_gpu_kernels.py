@@ -559,6 +559,36 @@ def test_linear_fp32_result_of_many_rows_from_bf16_operands():
         assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
 
 
+def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split():
+    """Every band of the table is a route of its weight's plan, ahead of the library's, for products that leave
+    partial sums; a product that wants a tensor, or a route switched to the rule of sizes, stays with the library."""
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    assert L.KNOWN_MID_ROWS[(4096, 14336)][0] == (129, 256, 4)
+    for (N, Kd), bands in L.KNOWN_MID_ROWS.items():
+        routes = L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True)
+        last = 128
+        for lo, hi, parts in bands:
+            assert lo == last + 1 and hi >= lo and 1 <= parts <= Kd // 64       # bands follow each other from 129 on
+            for M in (lo, hi):
+                r = L.route_of(routes, M)
+                assert (r.kind, r.parts) == ("mfma_split", parts), (N, Kd, M)
+            last = hi
+        assert L.route_of(routes, last + 1).kind == "library"
+        assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False), 200).kind == "library"
+        previous = L.set_gemm_route("static")
+        try:
+            assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True), 200).kind == "library"
+        finally:
+            L.set_gemm_route(previous)
+    # the product through the route is the product: 8B shape's output projection at 200 rows
+    x, w = _rand(200, 4096, dtype=torch.bfloat16, seed=5), _rand(4096, 4096, dtype=torch.bfloat16, scale=0.02, seed=6)
+    y = L.linear(x, w, keep_split=True)
+    assert isinstance(y, K().SplitSum) and tuple(y.parts.shape) == (4, 200, 4096)
+    want = x.double() @ w.double().t()
+    assert (y.parts.double().sum(0) - want).abs().max().item() <= 2e-5 * 64 * 0.02
+
+
 def test_linear_fp32_result_of_many_rows_by_the_tiled_kernel():
     """Where the LDS-tiled kernel takes the size (K in steps of 64), the fp32 result of more than 128 rows is its
     one part of fp32 sums: every row as exact as the weight-streaming kernel's, whatever rows stand beside it."""

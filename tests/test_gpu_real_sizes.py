@@ -49,7 +49,7 @@ SHAPES = {
             "num_hidden_layers": 1, "num_attention_heads": 64, "num_key_value_heads": 8, "rope_theta": 500000.0,
             "max_position_embeddings": 131072, "rms_norm_eps": 1e-5, "rope_scaling": dict(_LLAMA3, factor=8.0)},
 }
-LENGTHS = (200, 61, 130)
+LENGTHS = (300, 61, 130)
 
 
 def _ratio(a: torch.Tensor, ref: torch.Tensor) -> float:

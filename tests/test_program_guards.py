@@ -57,7 +57,7 @@ def test_the_product_plan_covers_every_number_of_rows_once(monkeypatch):
     L = importlib.import_module("infernum_amd.parts.linear")
     # the number of parts of a split product is the kernel library's to say; any rule serves here
     monkeypatch.setattr(L.K, "gemm_skinny_splits", lambda N, K: 4 if N < 8192 else 1)
-    monkeypatch.setitem(L.KNOWN_MID_ROWS, (48, 4096), 3)      # beside the shapes the table holds
+    monkeypatch.setitem(L.KNOWN_MID_ROWS, (48, 4096), ((129, 256, 3), (257, 300, 2)))      # beside the shapes the table holds
     try:
         for N, Kd in itertools.product((48, 4096, 28672, 16385), (64, 4096, 100, 14336)):
             for dtype, out, epi, keep, kernels in itertools.product(
