@@ -72,13 +72,14 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
 # the two parts); the 13B shape's down projection 43 / 47 / 53 against 54 / 100 / 120, the 70B shape's 165 / 155 /
 # 163 against 298 / 231 / 312, the 1B shape's 16 / 17 / 18 against 27 / 27 / 27.  At 384 rows: the 8B shape's down
 # projection 73 against 79, the 13B shape's 72 against 91, the 1B shape's 22 against 34.  Shapes whose QKV or output
-# projection came out even with the library's stay with it.  The 8B shape's decode step at 160 / 192 / 256 requests:
+# projection came out even with the library's stay with it (an entry without bands).  The 8B shape's decode step at 160 / 192 / 256 requests:
 # 19.8k / 21.4k / 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
 KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
     (2048, 8192): ((129, 256, 8), (257, 384, 5), (385, 512, 4)),
     (4096, 14336): ((129, 256, 4), (257, 384, 2)), (4096, 4096): ((129, 256, 4),), (6144, 4096): ((129, 256, 2),),
     (5120, 13824): ((129, 256, 3), (257, 384, 2)), (5120, 5120): ((129, 256, 3), (257, 384, 2)),
     (8192, 28672): ((129, 256, 2),), (8192, 8192): ((129, 256, 2),),
+    (3072, 2048): (), (2048, 2048): (), (15360, 5120): (), (10240, 8192): (),
 }
 
 ROUTES = ("table", "measured", "static")
@@ -119,12 +120,34 @@ def library_rows(N: int, K_: int, epilogue: Optional[str], keep_split: bool) -> 
     return mask & 0xFE             # up to 16 rows the weight-streaming kernel, always
 
 
+MID_ROWS_WORKGROUPS = 256      # the MI355X's compute units: the workgroups a launch of the split tiled kernel aims at
+MID_ROWS_MOST_PARTS = 8        # as far as measured
+
+
+def _mid_rows_by_size(N: int, K_: int) -> Tuple[Tuple[int, int, int], ...]:
+    """For shapes the table does not hold: per band of 128 rows (129 to 256, 257 to 384) as many parts as bring the
+    tiles of 128 x 128 to one workgroup a compute unit, while those are at least two (with one part the library was
+    as fast or faster for every shape measured) and a part keeps at least 8 steps of K."""
+    bands = []
+    tiles_n = -(-N // 128)
+    for tiles_m in (2, 3):
+        parts = min(MID_ROWS_WORKGROUPS // (tiles_m * tiles_n), K_ // 64 // 8, MID_ROWS_MOST_PARTS)
+        if parts < 2:
+            break
+        bands.append((128 * (tiles_m - 1) + 1, 128 * tiles_m, parts))
+    return tuple(bands)
+
+
 def mid_rows(N: int, K_: int, keep_split: bool) -> Tuple[Tuple[int, int, int], ...]:
     """(first row, last row, parts) for which the LDS-tiled kernel, K split into ``parts``, takes the product with
-    this weight; none where the library takes every number of rows above 128."""
-    if not keep_split or _route != "table" or _prefill_gemm != "library":
+    this weight; none where the library takes every number of rows above 128.  By the table, then by the rule of
+    sizes ("static": by the rule alone)."""
+    if not keep_split or _prefill_gemm != "library" or K_ % 64:
         return ()
-    return tuple((lo, hi, parts) for lo, hi, parts in KNOWN_MID_ROWS.get((N, K_), ())
+    bands = KNOWN_MID_ROWS.get((N, K_)) if _route == "table" else None
+    if bands is None:
+        bands = _mid_rows_by_size(N, K_)
+    return tuple((lo, hi, parts) for lo, hi, parts in bands
                  if lo > K.SKINNY_MAX_M and K.gemm_mfma_supported(hi, N, K_) and 1 <= parts <= K_ // 64)
 
 

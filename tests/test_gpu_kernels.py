@@ -561,7 +561,7 @@ def test_linear_fp32_result_of_many_rows_from_bf16_operands():
 
 def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split():
     """Every band of the table is a route of its weight's plan, ahead of the library's, for products that leave
-    partial sums; a product that wants a tensor, or a route switched to the rule of sizes, stays with the library."""
+    partial sums; a product that wants a tensor stays with the library; shapes outside the table follow a rule."""
     import importlib
     L = importlib.import_module("infernum_amd.parts.linear")
     assert L.KNOWN_MID_ROWS[(4096, 14336)][0] == (129, 256, 4)
@@ -576,11 +576,16 @@ def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split
             last = hi
         assert L.route_of(routes, last + 1).kind == "library"
         assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False), 200).kind == "library"
-        previous = L.set_gemm_route("static")
+        previous = L.set_gemm_route("static")            # the rule of sizes alone
         try:
-            assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True), 200).kind == "library"
+            by_size = L._mid_rows_by_size(N, Kd)
+            r = L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True), 200)
+            assert (r.kind, r.parts) == (("mfma_split", by_size[0][2]) if by_size else ("library", 0))
         finally:
             L.set_gemm_route(previous)
+    # a shape the table does not hold: as many parts as bring the tiles to a workgroup a compute unit, at least two
+    assert L.mid_rows(4096, 11008, True) == ((129, 256, 4), (257, 384, 2)) and L.mid_rows(4096, 11008, False) == ()
+    assert L.mid_rows(22016, 4096, True) == () and L.mid_rows(4096, 1000, True) == () and L.mid_rows(64, 448, True) == ()
     # the product through the route is the product: 8B shape's output projection at 200 rows
     x, w = _rand(200, 4096, dtype=torch.bfloat16, seed=5), _rand(4096, 4096, dtype=torch.bfloat16, scale=0.02, seed=6)
     y = L.linear(x, w, keep_split=True)
