@@ -72,8 +72,8 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
 # the two parts); the 13B shape's down projection 43 / 47 / 53 against 54 / 100 / 120, the 70B shape's 165 / 155 /
 # 163 against 298 / 231 / 312, the 1B shape's 16 / 17 / 18 against 27 / 27 / 27.  At 384 rows: the 8B shape's down
 # projection 73 against 79, the 13B shape's 72 against 91, the 1B shape's 22 against 34.  Shapes whose QKV or output
-# projection came out even with the library's stay with it (an entry without bands).  The 8B shape's decode step at 160 / 192 / 256 requests:
-# 19.8k / 21.4k / 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
+# projection came out even with the library's stay with it (an entry without bands).  The 8B shape's decode step at
+# 160 / 192 / 256 requests: 19.8k / 21.4k / 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
 KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
     (2048, 8192): ((129, 256, 8), (257, 384, 5), (385, 512, 4)),
     (4096, 14336): ((129, 256, 4), (257, 384, 2)), (4096, 4096): ((129, 256, 4),), (6144, 4096): ((129, 256, 2),),
