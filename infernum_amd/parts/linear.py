@@ -14,9 +14,10 @@ bf16: up to 128 rows the hand-written MFMA kernel that streams the weight once, 
 (hipBLASLt, called directly with its choice of an algorithm kept per shape) where that is known to be faster for
 the weight's shape (:data:`KNOWN_ROUTES`, a table that is part of the source, so that two runs of one model make
 the same launches; ``INFERNUM_GEMM_ROUTE=measured`` times both when a model loads instead, ``static`` keeps to
-the rule of sizes); for a few hundred rows the LDS-tiled MFMA kernel with K split over workgroups for the weights
-of :data:`KNOWN_MID_ROWS` whose partial sums the next kernel takes (the library's kernels for so few rows leave
-most of the GPU idle); above that the library, as the reference uses its library there; an fp32 result of more
+the rule of sizes); for the bands of rows of :data:`KNOWN_MID_ROWS` (up to a few hundred rows) the LDS-tiled MFMA
+kernel with K split over workgroups, for products whose partial sums the next kernel takes (the library's kernels
+for so few rows leave most of the GPU idle, and from some tens of rows on the tiled kernel streams a weight faster
+than the weight-streaming one); above that the library, as the reference uses its library there; an fp32 result of more
 than 128 rows comes from the LDS-tiled kernel's fp32 sums (128 rows at a time from the weight-streaming kernel where
 the tiled one does not take the size).  ``set_prefill_gemm("mfma")`` (or
 INFERNUM_PREFILL_GEMM=mfma) sends the many-row bf16 products to the hand-written LDS-tiled MFMA kernel instead,
@@ -63,23 +64,34 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
     (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
 }
 
-# (N, K) of a weight whose product leaves partial sums for the next kernel -> (first row, last row, parts): for
+# (N, K) of a weight whose product leaves partial sums for the next kernel -> bands (first row, last row, parts): for
 # these numbers of rows the LDS-tiled MFMA kernel takes the product with K split into so many parts (tiles of
 # 128 x 128 of the result: the parts bring the workgroups to about one a compute unit, which is what was fastest
-# for every shape).  Measured on an MI355X against the library's product with cold weights, microseconds at
-# 129 / 192 / 256 rows: the 8B shape's down projection 37 / 41 / 45 against 58 / 104 / 63, its output projection
-# 17 / 18 / 19 against 22 / 34 / 23, its QKV product 23 / 24 / 26 against 40 / 35 / 42 (the rotary kernel then adds
-# the two parts); the 13B shape's down projection 43 / 47 / 53 against 54 / 100 / 120, the 70B shape's 165 / 155 /
-# 163 against 298 / 231 / 312, the 1B shape's 16 / 17 / 18 against 27 / 27 / 27.  At 384 rows: the 8B shape's down
-# projection 73 against 79, the 13B shape's 72 against 91, the 1B shape's 22 against 34.  Shapes whose QKV or output
-# projection came out even with the library's stay with it (an entry without bands).  The 8B shape's decode step at
-# 160 / 192 / 256 requests: 19.8k / 21.4k / 24.3k tokens/s against 15.7k / 16.3k / 21.7k with the library's products.
+# for nearly every shape).  Measured on an MI355X with cold weights, in microseconds.
+# Above 128 rows, against the library's product, at 129 / 192 / 256 rows: the 8B shape's down projection 37 / 41 / 45
+# against 58 / 104 / 63, its output projection 17 / 18 / 19 against 22 / 34 / 23, its QKV product 23 / 24 / 26 against
+# 40 / 35 / 42 (the rotary kernel then adds the two parts); the 13B shape's down projection 43 / 47 / 53 against
+# 54 / 100 / 120, the 70B shape's 165 / 155 / 163 against 298 / 231 / 312, the 1B shape's 16 / 17 / 18 against 27 / 27 /
+# 27.  At 384 rows: the 8B shape's down projection 73 against 79, the 13B shape's 72 against 91, the 1B shape's 22
+# against 34.  The 8B shape's decode step at 160 / 192 / 256 requests: 19.8k / 21.4k / 24.3k tokens/s against 15.7k /
+# 16.3k / 21.7k with the library's products.
+# Up to 128 rows, against the weight-streaming kernel (or the library where KNOWN_ROUTES has it), at 32 / 64 / 128
+# rows: the 8B shape's down projection 25 / 26 / 30 against 29 / 32 / 40, its QKV product 13 / 14 / 17 against 15 / 17 /
+# 24, its output projection 10.5 / 11.5 / 14 against 10 / 12 / 15.5; the 13B shape's down projection 28 / 30 / 34
+# against 33 / 37 / 46, its output projection 14 / 16 / 19 against 16 / 19 / 23; the 70B shape's down projection 84 /
+# 90 / 105 against 94 / 111 / 139, its QKV product 36 / 35 / 39 against 38 / 41 / 52; at 8 rows the 70B shape's output
+# projection 29 against 35.  The 8B shape's decode step at 32 / 64 / 128 requests: 7.34k / 11.93k / 17.84k tokens/s
+# against 7.08k / 11.52k / 17.03k.  A band begins where the tiled kernel was ahead; a shape whose product came out
+# even stays where it was (an entry without bands).
 KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
-    (2048, 8192): ((129, 256, 8), (257, 384, 5), (385, 512, 4)),
-    (4096, 14336): ((129, 256, 4), (257, 384, 2)), (4096, 4096): ((129, 256, 4),), (6144, 4096): ((129, 256, 2),),
-    (5120, 13824): ((129, 256, 3), (257, 384, 2)), (5120, 5120): ((129, 256, 3), (257, 384, 2)),
-    (8192, 28672): ((129, 256, 2),), (8192, 8192): ((129, 256, 2),),
-    (3072, 2048): (), (2048, 2048): (), (15360, 5120): (), (10240, 8192): (),
+    (2048, 8192): ((17, 128, 16), (129, 256, 8), (257, 384, 5), (385, 512, 4)),
+    (3072, 2048): (), (2048, 2048): (),
+    (4096, 14336): ((17, 128, 8), (129, 256, 4), (257, 384, 2)), (4096, 4096): ((49, 128, 8), (129, 256, 4)),
+    (6144, 4096): ((25, 128, 5), (129, 256, 2)),
+    (5120, 13824): ((17, 128, 6), (129, 256, 3), (257, 384, 2)), (5120, 5120): ((1, 128, 6), (129, 256, 3), (257, 384, 2)),
+    (15360, 5120): ((1, 16, 2), (97, 128, 2)),
+    (8192, 28672): ((17, 128, 4), (129, 256, 2)), (8192, 8192): ((1, 16, 8), (81, 128, 4), (129, 256, 2)),
+    (10240, 8192): ((17, 128, 3),),
 }
 
 ROUTES = ("table", "measured", "static")
@@ -148,7 +160,7 @@ def mid_rows(N: int, K_: int, keep_split: bool) -> Tuple[Tuple[int, int, int], .
     if bands is None:
         bands = _mid_rows_by_size(N, K_)
     return tuple((lo, hi, parts) for lo, hi, parts in bands
-                 if lo > K.SKINNY_MAX_M and K.gemm_mfma_supported(hi, N, K_) and 1 <= parts <= K_ // 64)
+                 if 1 <= lo <= hi and K.gemm_mfma_supported(hi, N, K_) and 1 <= parts <= K_ // 64)
 
 
 def tiled_copy(w: torch.Tensor, epilogue: Optional[str]) -> Optional[torch.Tensor]:
@@ -310,9 +322,10 @@ def plan(N: int, Kdim: int, dtype: torch.dtype, out_dtype: torch.dtype, epilogue
                 Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_f32" if tiled_fits else "skinny_rows")]
     to_library = library_rows(N, Kdim, epilogue, keep_split) if _prefill_gemm == "library" else \
         (0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1))
-    routes = [Route(_UP_TO_128 & ~to_library, own)]
-    for lo, hi, parts in mid_rows(N, Kdim, keep_split and epilogue is None):
-        routes.append(Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_split", rows=(lo, hi), parts=parts))
+    # the bands of rows of the split tiled kernel stand first: they take their rows from the routes behind them
+    routes = [Route(ALL_BLOCKS, "mfma_split", rows=(lo, hi), parts=parts)
+              for lo, hi, parts in mid_rows(N, Kdim, keep_split and epilogue is None)]
+    routes.append(Route(_UP_TO_128 & ~to_library, own))
     routes.append(Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback))
     return [r for r in routes if r.blocks]
 
@@ -398,14 +411,23 @@ def emit_linear(program, x: Any, M: Any, w: torch.Tensor, out_dtype: torch.dtype
     skinny, wk = ("ia_gemm_skinny_tiled", tiled) if tiled is not None else ("ia_gemm_skinny", w)
     program.keep(w, tiled)
     alts = []
-    ranged = P.NEVER                   # the rows that routes with a range of their own have taken
+    taken: List[Tuple[int, int]] = []          # the rows that routes with a range of their own have taken
+
+    def not_taken():
+        """Holds for the numbers of rows in none of the ranges taken so far: the gaps between them."""
+        g, first = P.NEVER, None
+        for lo, hi in sorted(taken) + [(None, None)]:
+            last = None if lo is None else lo - 1
+            if first is None or last is None or first <= last:
+                g = g | P.Guard.between(M, first, last)
+            first = None if hi is None else (hi + 1 if first is None else max(first, hi + 1))
+        return g
+
     for r in routes:
-        g = when & P.Guard.blocks(M, r.blocks)
+        g = when & P.Guard.blocks(M, r.blocks) & not_taken()
         if r.rows is not None:
-            own_rows = P.Guard.between(M, r.rows[0], r.rows[1])
-            g, ranged = g & own_rows & ~ranged, ranged | own_rows
-        else:
-            g = g & ~ranged
+            g = g & P.Guard.between(M, r.rows[0], r.rows[1])
+            taken.append(r.rows)
         if g.never:
             continue
         if r.kind == "mfma_split":

@@ -564,17 +564,21 @@ def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split
     partial sums; a product that wants a tensor stays with the library; shapes outside the table follow a rule."""
     import importlib
     L = importlib.import_module("infernum_amd.parts.linear")
-    assert L.KNOWN_MID_ROWS[(4096, 14336)][0] == (129, 256, 4)
+    assert (129, 256, 4) in L.KNOWN_MID_ROWS[(4096, 14336)]
     for (N, Kd), bands in L.KNOWN_MID_ROWS.items():
         routes = L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True)
-        last = 128
+        last = 0
         for lo, hi, parts in bands:
-            assert lo == last + 1 and hi >= lo and 1 <= parts <= Kd // 64       # bands follow each other from 129 on
+            assert lo > last and hi >= lo and 1 <= parts <= Kd // 64           # bands follow each other
             for M in (lo, hi):
                 r = L.route_of(routes, M)
                 assert (r.kind, r.parts) == ("mfma_split", parts), (N, Kd, M)
+            if lo > 1:
+                assert L.route_of(routes, lo - 1).kind != "mfma_split" or lo - 1 == last
             last = hi
-        assert L.route_of(routes, last + 1).kind == "library"
+        assert L.route_of(routes, max(last, 128) + 1).kind == "library"
+        if not any(lo <= 8 <= hi for lo, hi, _ in bands):                       # few rows: the weight-streaming kernel
+            assert L.route_of(routes, 8).kind in ("skinny", "skinny_split")
         assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False), 200).kind == "library"
         previous = L.set_gemm_route("static")            # the rule of sizes alone
         try:
@@ -672,7 +676,15 @@ def test_known_routes_send_rows_to_the_library_where_the_table_says():
     assert L.KNOWN_ROUTES[key] == 0b11111110
     kinds = lambda: {m: L.route_of(L.plan(15360, 5120, torch.bfloat16, torch.bfloat16, None, True), m).kind
                      for m in (1, 16, 17, 64, 128, 129)}
-    assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "library", 64: "library", 128: "library", 129: "library"}
+    # (the bands of KNOWN_MID_ROWS stand in front: up to 16 rows and from 97 to 128 the split tiled kernel for this shape)
+    assert L.KNOWN_MID_ROWS[(15360, 5120)] == ((1, 16, 2), (97, 128, 2))
+    assert kinds() == {1: "mfma_split", 16: "mfma_split", 17: "library", 64: "library", 128: "mfma_split", 129: "library"}
+    saved = L.KNOWN_MID_ROWS.pop((15360, 5120))
+    try:
+        assert L.mid_rows(15360, 5120, True) == ()           # the rule of sizes has none for so wide a weight
+        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "library", 64: "library", 128: "library", 129: "library"}
+    finally:
+        L.KNOWN_MID_ROWS[(15360, 5120)] = saved
     previous = L.set_gemm_route("static")
     try:
         assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "skinny_split", 64: "skinny_split",

@@ -70,7 +70,7 @@ def test_the_product_plan_covers_every_number_of_rows_once(monkeypatch):
                     seen = 0
                     for r in L.plan(N, Kd, dtype, out, epi, keep, kernels):
                         if r.rows is not None:                 # a route for a range of rows: ahead of the one it takes from
-                            assert r.blocks == 1 << 8 and 129 <= r.rows[0] <= r.rows[1] and not (seen & r.blocks)
+                            assert r.blocks == L.ALL_BLOCKS and 1 <= r.rows[0] <= r.rows[1] and not seen
                             assert r.kind == "mfma_split" and r.parts >= 1 and keep and epi is None
                             continue
                         assert r.blocks and not (seen & r.blocks)
