@@ -30,7 +30,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef const __attribute__((address_space(1))) void* gm_global_ptr;
 typedef __attribute__((address_space(3))) void* gm_lds_ptr;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT, bool GLU = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X,
                                                                            const uint16_t* __restrict__ W,
                                                                            uint16_t* __restrict__ C,
@@ -80,7 +80,19 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
   for (int f = 0; f < FPW; ++f) {
     const int row = 8 * (f * WAVES + wave) + (lane >> 3);
     const int piece = (lane & 7) ^ (row & 7);
-    const int r = (8 * f * WAVES < BM) ? min(m0 + row, M - 1) : min(n0 + row - BM, N - 1);
+    int r;
+    if (8 * f * WAVES < BM) {
+      r = min(m0 + row, M - 1);
+    } else if (GLU) {
+      // the rows of W of a wave's part alternate in groups of 32 between the first half of W (gate) and the
+      // second (up), for the same 32 columns of the result: accumulator tiles 2 p and 2 p + 1 of a wave meet
+      // lane by lane in the epilogue
+      const int rw = row - BM, q = (rw % WN) / 32;
+      const int col = tn * (BN / 2) + (rw / WN) * (WN / 2) + (q >> 1) * 32 + (rw & 31);
+      r = (q & 1) * (N / 2) + min(col, N / 2 - 1);
+    } else {
+      r = min(n0 + row - BM, N - 1);
+    }
     src[f] = ((uint32_t)r * (uint32_t)K + (uint32_t)piece * 8u) * 2u;
   }
 #define GM_FILL(f, kt, buf)                                                                                  \
@@ -215,6 +227,41 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
       }
     return;
   }
+  if constexpr (GLU) {
+    // C [M, N / 2] = silu(X W_first^T) * (X W_second^T), from the fp32 sums, rounded once
+    static_assert(!SPLIT && TN % 2 == 0, "the activation needs whole sums and pairs of accumulator tiles");
+    const int NO = N / 2;
+    const bool vec4 = (NO & 3) == 0;
+#pragma unroll
+    for (int p = 0; p < TN / 2; ++p)
+#pragma unroll
+      for (int b = 0; b < TM; ++b) {
+        const int m = m0 + wm * WM + b * 32 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = tn * (BN / 2) + wn * (WN / 2) + p * 32 + 8 * g + 4 * lh;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float gate = acc[2 * p][b][4 * g + e], up = acc[2 * p + 1][b][4 * g + e];
+            v[e] = gate / (1.0f + expf(-gate)) * up;
+          }
+          uint16_t* dstp = C + (size_t)m * NO + n;
+          if (vec4 && n + 3 < NO) {
+            uint2 o;
+            o.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+            o.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+            *reinterpret_cast<uint2*>(dstp) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < NO) dstp[e] = float_to_bf16_bits(v[e]);
+          }
+        }
+      }
+    return;
+  }
   constexpr int CP = WN / 8;                        // 16-byte pieces per row of a wave's part
   static_assert(STAGES * STAGE_BYTES >= WAVES * WM * WN * 2, "the stages must hold the tile of C");
   if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
@@ -274,21 +321,22 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT, bool GLU = false>
 static int launch_gemm_mfma(const uint16_t* x, const uint16_t* w, uint16_t* c, float* parts, int M, int N, int K,
                             int splits, hipStream_t stream) {
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  // with the activation a tile of BN rows of W gives BN / 2 columns of the result
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = GLU ? (N / 2 + BN / 2 - 1) / (BN / 2) : (N + BN - 1) / BN;
   const size_t lds_bytes = (size_t)STAGES * (BM + BN) * GM_ROW_BYTES;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT, GLU>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
   if ((long long)tiles_m * tiles_n * splits > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
-  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT>
+  gemm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, FILL_STEPS, SPLIT, GLU>
       <<<tiles_m * tiles_n * splits, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(x, w, c, parts, M, N, K, tiles_m,
                                                                                   tiles_n, splits);
   IA_LAUNCH_CHECK();
@@ -336,7 +384,17 @@ extern "C" int ia_gemm_mfma_split(const void* X, const void* W, float* parts, in
                                                       splits, stream);
 }
 
+// C [M, N / 2] = silu(X W[:N/2]^T) * (X W[N/2:]^T), bf16, the activation on the fp32 sums in the epilogue: for up
+// to some hundred rows, where the launch's N / 128 tiles of 128 x 128 stream the weight once.
+extern "C" int ia_gemm_mfma_swiglu(const void* X, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
+  if (!gemm_mfma_takes(M, N, K)) return IA_ERR_UNSUPPORTED;
+  if (N & 1) return IA_ERR_BAD_ARG;
+  return launch_gemm_mfma<128, 128, 2, 2, 4, 1, false, true>((const uint16_t*)X, (const uint16_t*)W, (uint16_t*)C,
+                                                             nullptr, M, N, K, 1, stream);
+}
+
 // ---- the launchers of this file as operations of a step's program (see op_call.h) ----
 #include "op_call.h"
 IA_OP(ia_gemm_mfma)
 IA_OP(ia_gemm_mfma_split)
+IA_OP(ia_gemm_mfma_swiglu)

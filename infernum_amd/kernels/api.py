@@ -357,6 +357,25 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     return out
 
 
+def gemm_mfma_swiglu(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(a @ w[:N/2]^T) * (a @ w[N/2:]^T) as bf16 [M, N/2]: the LDS-tiled MFMA product (tiles of 128 x 128) with
+    the activation on its fp32 sums in the epilogue, for up to some hundred rows."""
+    _dev(a, w, out)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_mfma_swiglu: shapes")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_mfma_swiglu: bf16 operands")
+    _need(a.is_contiguous() and w.is_contiguous(), "gemm_mfma_swiglu: contiguous operands")
+    _need(N % 2 == 0 and gemm_mfma_supported(M, N, K),
+          f"gemm_mfma_swiglu: M={M} N={N} K={K} not supported (N even, K % 64 == 0, below 4 GiB)")
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=a.device)
+    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N // 2),
+          f"gemm_mfma_swiglu: out must be contiguous bf16 [{M}, {N // 2}]")
+    _ok(_core().ia_gemm_mfma_swiglu(_p(a), _p(w), _p(out), M, N, K, _stream()), "gemm_mfma_swiglu")
+    return out
+
+
 def gemm_mfma_split(a: torch.Tensor, w: torch.Tensor, splits: int, parts: Optional[torch.Tensor] = None) -> SplitSum:
     """a[M, K] @ w[N, K]^T for a few hundred rows as fp32 partial sums [splits, M, N]: the LDS-tiled MFMA product
     with tiles of 128 x 128 and K split over ``splits`` workgroups a tile, so that the launch fills the GPU where the

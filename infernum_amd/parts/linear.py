@@ -94,6 +94,12 @@ KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
     (10240, 8192): ((17, 128, 3),),
 }
 
+# (N, K) of a gate+up weight -> bands (first row, last row) in which the LDS-tiled kernel with the activation in
+# its epilogue takes the product (the same bits as the weight-streaming kernel's epilogue gives).
+KNOWN_GLU_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int], ...]] = {
+    (28672, 4096): ((49, 128),), (27648, 5120): ((33, 128),), (57344, 8192): ((49, 128),),
+}
+
 ROUTES = ("table", "measured", "static")
 _route = os.environ.get("INFERNUM_GEMM_ROUTE", "table")
 if _route not in ROUTES:
@@ -282,7 +288,8 @@ class Route:
     activation in its epilogue), "skinny_split" (the same with its partial sums left for the next kernel),
     "skinny_rows" (128 rows at a time), "library" (hipBLASLt; ``fallback`` names the kernel for a shape it
     refuses), "mfma" (the LDS-tiled kernel), "mfma_split" (the same with K split into ``parts``, its partial
-    sums left for the next kernel), "mfma_f32" (the same in one part: an fp32 result from bf16 operands).  A route
+    sums left for the next kernel), "mfma_f32" (the same in one part: an fp32 result from bf16 operands), "mfma_swiglu" (the tiled kernel with the
+    activation in its epilogue).  A route
     with ``rows`` (first, last) takes those numbers of rows only, and takes them from the routes without that stand
     behind it."""
 
@@ -293,6 +300,7 @@ class Route:
     parts: int = 0
 
 
+FP32_TILED_FROM_ROWS = (49, 81)     # an fp32 result goes to the tiled kernel from so many rows on: K >= 4,096; shorter K
 _MANY_ROWS = 65536         # the LDS-tiled kernel addresses rows with 32 bits: its fitness is judged at this many
 
 
@@ -314,17 +322,23 @@ def plan(N: int, Kdim: int, dtype: torch.dtype, out_dtype: torch.dtype, epilogue
     if out_dtype != torch.bfloat16:
         if epilogue is not None:
             raise K.KernelError("linear: an fp32 result from bf16 operands has no activation here")
-        # more than 128 rows (the head of a step that wants the logits of many places): the LDS-tiled kernel leaving
-        # its fp32 sums (one part), which reads the weight once per 128 x 128 tile of the result where the
-        # weight-streaming kernel reads all of it for every 128 rows (the head of 128,256 x 4,096 on an MI355X:
-        # 371 against 649 us at 256 rows, 2.6 against 4.9 ms at 2,048)
-        return [Route(_UP_TO_128, own),
-                Route(ALL_BLOCKS & ~_UP_TO_128, "mfma_f32" if tiled_fits else "skinny_rows")]
+        # many rows (the head of a step that wants the logits of many places): the LDS-tiled kernel leaving its fp32
+        # sums (one part), which reads the weight once per 128 x 128 tile of the result where the weight-streaming
+        # kernel reads all of it for every 128 rows (the head of 128,256 x 4,096 on an MI355X: 371 against 649 us at
+        # 256 rows, 2.6 against 4.9 ms at 2,048) and all of X for every 64 rows of the weight (201 against 229 us at
+        # 64 rows, 226 against 314 at 128; with K of 2,048 even at 64 rows, 150 against 181 at 128).  The same bits.
+        routes = [Route(_UP_TO_128, own), Route(ALL_BLOCKS & ~_UP_TO_128, "skinny_rows")]
+        if tiled_fits:
+            first = FP32_TILED_FROM_ROWS[0] if Kdim >= 4096 else FP32_TILED_FROM_ROWS[1]
+            routes.insert(0, Route(ALL_BLOCKS, "mfma_f32", rows=(first, (2 ** 32 - 1) // (2 * Kdim) - 1)))
+        return routes
     to_library = library_rows(N, Kdim, epilogue, keep_split) if _prefill_gemm == "library" else \
         (0 if N < SKINNY_WIDE else 0xFF & ~((1 << (SKINNY_ROWS_ANY_WIDTH // 16)) - 1))
     # the bands of rows of the split tiled kernel stand first: they take their rows from the routes behind them
     routes = [Route(ALL_BLOCKS, "mfma_split", rows=(lo, hi), parts=parts)
               for lo, hi, parts in mid_rows(N, Kdim, keep_split and epilogue is None)]
+    if epilogue == "swiglu" and _route == "table" and _prefill_gemm == "library" and tiled_fits:
+        routes += [Route(ALL_BLOCKS, "mfma_swiglu", rows=(lo, hi)) for lo, hi in KNOWN_GLU_ROWS.get((N, Kdim), ())]
     routes.append(Route(_UP_TO_128 & ~to_library, own))
     routes.append(Route((ALL_BLOCKS & ~_UP_TO_128) | to_library, many.kind, many.fallback))
     return [r for r in routes if r.blocks]
@@ -345,6 +359,8 @@ def _run(kind: str, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, ep
         return K.gemm_mfma_split(x, w, parts), True
     if kind == "mfma_f32":
         return K.gemm_mfma_split(x, w, 1).parts[0], True
+    if kind == "mfma_swiglu":
+        return K.gemm_mfma_swiglu(x, w), True
     if kind == "skinny":
         return K.gemm_skinny(x, w, epilogue=epilogue, out_dtype=out_dtype, tiled=tiled_copy(w, epilogue)), True
     if kind == "skinny_split":
@@ -433,6 +449,10 @@ def emit_linear(program, x: Any, M: Any, w: torch.Tensor, out_dtype: torch.dtype
         if r.kind == "mfma_split":
             program.op("core", "ia_gemm_mfma_split", [x, w, out, M, N, Kdim, r.parts, P.STREAM], g)
             alts.append(P.Alt(g, out, r.parts, torch.float32))
+            continue
+        if r.kind == "mfma_swiglu":
+            program.op("core", "ia_gemm_mfma_swiglu", [x, w, out, M, N, Kdim, P.STREAM], g)
+            alts.append(P.Alt(g, out, 0, out_dtype))
             continue
         if r.kind == "mfma_f32":                # one part: the fp32 matrix itself
             program.op("core", "ia_gemm_mfma_split", [x, w, out, M, N, Kdim, 1, P.STREAM], g)

@@ -103,12 +103,16 @@ def test_steps_of_129_to_256_rows_through_the_tiled_kernel_with_k_split(models, 
     hd = H // nh
     monkeypatch.setitem(L.KNOWN_MID_ROWS, (H, nh * hd), ((129, 256, 2),))
     monkeypatch.setitem(L.KNOWN_MID_ROWS, ((nh + 2 * nkv) * hd, H), ((129, 160, 2), (161, 256, 1)))
+    # and gate+up on the tiled kernel with the activation in its epilogue from 20 to 150 rows
+    monkeypatch.setitem(L.KNOWN_GLU_ROWS, (2 * cfg["intermediate_size"], H), ((20, 150),))
+    glu = L.plan(2 * cfg["intermediate_size"], H, torch.bfloat16, torch.bfloat16, "swiglu", False)
+    assert {M: L.route_of(glu, M).kind for M in (19, 20, 150, 151)} == {19: "skinny", 20: "mfma_swiglu", 150: "mfma_swiglu", 151: "library"}
     kinds = {M: L.route_of(L.plan(H, nh * hd, torch.bfloat16, torch.bfloat16, None, True), M).kind for M in (128, 129, 256, 257)}
     assert kinds == {128: "skinny", 129: "mfma_split", 256: "mfma_split", 257: "library"}      # K of 128: one part up to 128 rows
     assert sum(129 <= len(t) <= 256 for t in reqs.values()) >= 4
     native = _engine(d, "bfloat16", PAGE["B"], 128)
     parts = _engine(d, "bfloat16", PAGE["B"], 128, executor="parts")
-    assert "ia_gemm_mfma_split" in native.program.op_names
+    assert "ia_gemm_mfma_split" in native.program.op_names and "ia_gemm_mfma_swiglu" in native.program.op_names
     a, b = TT.run_steps(native, TT.trace_whole(reqs)), TT.run_steps(parts, TT.trace_whole(reqs))
     _check(a, ref, "bfloat16", "B bfloat16 whole, 129 to 256 rows on the split tiled kernel")
     assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)

@@ -465,6 +465,36 @@ def test_gemm_mfma_split_picks_out_one_product_and_refuses_what_it_cannot_do():
         api.gemm_mfma_split(a, w, S, torch.empty(S, M, N + 1, device=DEV))                           # parts' shape
 
 
+@pytest.mark.parametrize("M,N,K_", [(64, 1000, 192), (1, 66, 64), (128, 330, 256), (200, 2048, 448), (37, 254, 448),
+                                    (130, 260, 1024)])
+def test_gemm_mfma_swiglu(M, N, K_):
+    """The LDS-tiled product with the activation in its epilogue: silu(first half) * second half from the fp32 sums,
+    rounded once; tiles of 64 columns of the result at sizes that fill none, half widths that are no multiple of 4
+    (scalar stores), more rows than a tile.  Up to 128 rows the weight-streaming kernel's epilogue gives the same
+    bits (the same sums in the same order, the same formula)."""
+    api = K()
+    a, w = _rand(M, K_, dtype=torch.bfloat16, seed=8), _rand(N, K_, dtype=torch.bfloat16, scale=0.1, seed=9)
+    out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert api.gemm_mfma_swiglu(a, w, out).data_ptr() == out.data_ptr()
+    y = a.double() @ w.double().t()
+    gate, up = y[:, :N // 2], y[:, N // 2:]
+    want = torch.nn.functional.silu(gate) * up
+    # the sums carry fp32 rounding (2e-5 sqrt(K) 0.1 each); silu has slope at most 1.1
+    e = 2e-5 * math.sqrt(K_) * 0.1
+    bound = 2.0 ** -8 * want.abs() + e * (1.1 * up.abs() + gate.abs() + e)
+    assert bool(((out.double() - want).abs() <= bound).all())
+    if M <= 128:
+        assert torch.equal(api.gemm_skinny(a, w, epilogue="swiglu"), out)
+    # a row's result does not depend on the rows beside it
+    assert torch.equal(api.gemm_mfma_swiglu(a[M - 1:M].contiguous(), w)[0], out[M - 1])
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_swiglu(a, w[:N - 1].contiguous())                                             # an odd number of rows
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_swiglu(a, w, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))             # out's shape
+    with pytest.raises(api.KernelError):
+        api.gemm_mfma_swiglu(_rand(8, 96, dtype=torch.bfloat16), _rand(32, 96, dtype=torch.bfloat16))   # K % 64
+
+
 def test_gemm_mfma_refuses_what_it_cannot_do():
     api = K()
     with pytest.raises(api.KernelError):
@@ -587,6 +617,13 @@ def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split
             assert (r.kind, r.parts) == (("mfma_split", by_size[0][2]) if by_size else ("library", 0))
         finally:
             L.set_gemm_route(previous)
+    # gate+up products: the tiled kernel with the activation in its epilogue for the bands of its table
+    for (N, Kd), bands in L.KNOWN_GLU_ROWS.items():
+        routes = L.plan(N, Kd, torch.bfloat16, torch.bfloat16, "swiglu", False)
+        for lo, hi in bands:
+            assert L.route_of(routes, lo).kind == L.route_of(routes, hi).kind == "mfma_swiglu"
+            assert L.route_of(routes, lo - 1).kind != "mfma_swiglu" and L.route_of(routes, hi + 1).kind != "mfma_swiglu"
+        assert all(r.kind != "mfma_swiglu" for r in L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False))
     # a shape the table does not hold: as many parts as bring the tiles to a workgroup a compute unit, at least two
     assert L.mid_rows(4096, 11008, True) == ((129, 256, 4), (257, 384, 2)) and L.mid_rows(4096, 11008, False) == ()
     assert L.mid_rows(22016, 4096, True) == () and L.mid_rows(4096, 1000, True) == () and L.mid_rows(64, 448, True) == ()
@@ -604,16 +641,21 @@ def test_linear_fp32_result_of_many_rows_by_the_tiled_kernel():
     import importlib
     L = importlib.import_module("infernum_amd.parts.linear")
     x, w = _rand(300, 192, dtype=torch.bfloat16, seed=5), _rand(1003, 192, dtype=torch.bfloat16, scale=0.1, seed=6)
-    assert [r.kind for r in L.plan(1003, 192, torch.bfloat16, torch.float32, None, False)] == ["skinny", "mfma_f32"]
+    assert [r.kind for r in L.plan(1003, 192, torch.bfloat16, torch.float32, None, False)] == ["mfma_f32", "skinny", "skinny_rows"]
+    first = L.FP32_TILED_FROM_ROWS[1]
+    assert L.route_of(L.plan(1003, 192, torch.bfloat16, torch.float32, None, False), first).kind == "mfma_f32"
+    assert L.route_of(L.plan(1003, 192, torch.bfloat16, torch.float32, None, False), first - 1).kind == "skinny"
+    assert L.route_of(L.plan(1003, 4096, torch.bfloat16, torch.float32, None, False), L.FP32_TILED_FROM_ROWS[0]).kind == "mfma_f32"
     y = L.linear(x, w, out_dtype=torch.float32)
     want = x.double() @ w.double().t()
     assert y.dtype == torch.float32 and tuple(y.shape) == (300, 1003)
     assert (y.double() - want).abs().max().item() <= 2e-5 * 14 * 0.1
     for m in (129, 256, 257):
         assert torch.equal(L.linear(x[:m].contiguous(), w, out_dtype=torch.float32), y[:m])
-    few = L.linear(x[:128].contiguous(), w, out_dtype=torch.float32)           # the weight-streaming kernel
-    assert (few.double() - want[:128]).abs().max().item() <= 2e-5 * 14 * 0.1
-    assert (few - y[:128]).abs().max().item() <= 4e-6 * 14 * 0.1
+    few = L.linear(x[:first - 1].contiguous(), w, out_dtype=torch.float32)     # the weight-streaming kernel
+    assert (few.double() - want[:first - 1]).abs().max().item() <= 2e-5 * 14 * 0.1
+    assert (few - y[:first - 1]).abs().max().item() <= 4e-6 * 14 * 0.1
+    assert torch.equal(L.linear(x[:first].contiguous(), w, out_dtype=torch.float32), y[:first])
 
 
 @pytest.mark.parametrize("N,Kd,epilogue", [(28672, 4096, "swiglu"), (330, 264, "swiglu"), (1000, 96, None), (6144, 512, None),

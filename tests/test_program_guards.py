@@ -71,7 +71,9 @@ def test_the_product_plan_covers_every_number_of_rows_once(monkeypatch):
                     for r in L.plan(N, Kd, dtype, out, epi, keep, kernels):
                         if r.rows is not None:                 # a route for a range of rows: ahead of the one it takes from
                             assert r.blocks == L.ALL_BLOCKS and 1 <= r.rows[0] <= r.rows[1] and not seen
-                            assert r.kind == "mfma_split" and r.parts >= 1 and keep and epi is None
+                            assert (r.kind == "mfma_split" and r.parts >= 1 and keep and epi is None) or \
+                                (r.kind == "mfma_f32" and out == torch.float32 and dtype == torch.bfloat16) or \
+                                (r.kind == "mfma_swiglu" and epi == "swiglu")
                             continue
                         assert r.blocks and not (seen & r.blocks)
                         seen |= r.blocks
