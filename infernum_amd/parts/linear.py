@@ -95,9 +95,10 @@ KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
 }
 
 # (N, K) of a gate+up weight -> bands (first row, last row) in which the LDS-tiled kernel with the activation in
-# its epilogue takes the product (the same bits as the weight-streaming kernel's epilogue gives).
+# its epilogue takes the product (the 8B shape's at 32 / 64 / 128 rows: 43 / 45 / 51 us against the weight-streaming
+# kernel's 47 / 56 / 73 and the library's with the activation's launch 54 / 54 / 57).
 KNOWN_GLU_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int], ...]] = {
-    (28672, 4096): ((49, 128),), (27648, 5120): ((33, 128),), (57344, 8192): ((49, 128),),
+    (28672, 4096): ((17, 128),), (27648, 5120): ((33, 128),), (57344, 8192): ((17, 128),), (16384, 2048): ((129, 256),),
 }
 
 ROUTES = ("table", "measured", "static")

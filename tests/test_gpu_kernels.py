@@ -471,7 +471,7 @@ def test_gemm_mfma_swiglu(M, N, K_):
     """The LDS-tiled product with the activation in its epilogue: silu(first half) * second half from the fp32 sums,
     rounded once; tiles of 64 columns of the result at sizes that fill none, half widths that are no multiple of 4
     (scalar stores), more rows than a tile.  Up to 128 rows the weight-streaming kernel's epilogue gives the same
-    bits (the same sums in the same order, the same formula)."""
+    values but for the order of the fp32 additions (a tile of columns starts its walk over K at a step of its own)."""
     api = K()
     a, w = _rand(M, K_, dtype=torch.bfloat16, seed=8), _rand(N, K_, dtype=torch.bfloat16, scale=0.1, seed=9)
     out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
@@ -484,7 +484,8 @@ def test_gemm_mfma_swiglu(M, N, K_):
     bound = 2.0 ** -8 * want.abs() + e * (1.1 * up.abs() + gate.abs() + e)
     assert bool(((out.double() - want).abs() <= bound).all())
     if M <= 128:
-        assert torch.equal(api.gemm_skinny(a, w, epilogue="swiglu"), out)
+        other = api.gemm_skinny(a, w, epilogue="swiglu").double()
+        assert bool(((out.double() - other).abs() <= 2.0 ** -7 * want.abs() + 2 * e * (1.1 * up.abs() + gate.abs() + e)).all())
     # a row's result does not depend on the rows beside it
     assert torch.equal(api.gemm_mfma_swiglu(a[M - 1:M].contiguous(), w)[0], out[M - 1])
     with pytest.raises(api.KernelError):
