@@ -60,7 +60,7 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
     (4096, 14336, None, True): 0,
     (15360, 5120, None, True): 0b11111110, (5120, 5120, None, True): 0,
     (27648, 5120, "swiglu", False): 0b11111010, (5120, 13824, None, True): 0,
-    (10240, 8192, None, True): 0b01001110, (8192, 8192, None, True): 0b01011110,
+    (10240, 8192, None, True): 0, (8192, 8192, None, True): 0,
     (57344, 8192, "swiglu", False): 0b11111110, (8192, 28672, None, True): 0,
 }
 
@@ -79,19 +79,18 @@ KNOWN_ROUTES: Dict[Tuple[int, int, Optional[str], bool], int] = {
 # rows: the 8B shape's down projection 25 / 26 / 30 against 29 / 32 / 40, its QKV product 13 / 14 / 17 against 15 / 17 /
 # 24, its output projection 10.5 / 11.5 / 14 against 10 / 12 / 15.5; the 13B shape's down projection 28 / 30 / 34
 # against 33 / 37 / 46, its output projection 14 / 16 / 19 against 16 / 19 / 23; the 70B shape's down projection 84 /
-# 90 / 105 against 94 / 111 / 139, its QKV product 36 / 35 / 39 against 38 / 41 / 52; at 8 rows the 70B shape's output
-# projection 29 against 35.  The 8B shape's decode step at 32 / 64 / 128 requests: 7.34k / 11.93k / 17.84k tokens/s
+# 90 / 105 against 94 / 111 / 139, its QKV product 36 / 35 / 39 against 38 / 41 / 52.  The 8B shape's decode step at 32 / 64 / 128 requests: 7.34k / 11.93k / 17.84k tokens/s
 # against 7.08k / 11.52k / 17.03k.  A band begins where the tiled kernel was ahead; a shape whose product came out
 # even stays where it was (an entry without bands).
 KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
     (2048, 8192): ((17, 128, 16), (129, 256, 8), (257, 384, 5), (385, 512, 4)),
     (3072, 2048): (), (2048, 2048): (),
     (4096, 14336): ((17, 128, 8), (129, 256, 4), (257, 384, 2)), (4096, 4096): ((49, 128, 8), (129, 256, 4)),
-    (6144, 4096): ((25, 128, 5), (129, 256, 2)),
+    (6144, 4096): ((17, 128, 5), (129, 256, 2)),
     (5120, 13824): ((17, 128, 6), (129, 256, 3), (257, 384, 2)), (5120, 5120): ((1, 128, 6), (129, 256, 3), (257, 384, 2)),
     (15360, 5120): ((1, 16, 2), (97, 128, 2)),
-    (8192, 28672): ((17, 128, 4), (129, 256, 2)), (8192, 8192): ((1, 16, 8), (81, 128, 4), (129, 256, 2)),
-    (10240, 8192): ((17, 128, 3),),
+    (8192, 28672): ((17, 128, 4), (129, 256, 2)), (8192, 8192): ((25, 128, 4), (129, 256, 2)),
+    (10240, 8192): ((33, 128, 3),),
 }
 
 # (N, K) of a gate+up weight -> bands (first row, last row) in which the LDS-tiled kernel with the activation in
