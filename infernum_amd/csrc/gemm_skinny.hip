@@ -127,14 +127,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(const uint16
   };
 
   // Workgroups that walk K in step read rows of W one row's length apart at the same moment, and such addresses
-  // crowd on few memory channels where that length is a power of two.  A product that leaves partial sums (which
-  // the next kernel adds in fp32 anyway) lets every tile of rows start its walk over its chunks at a chunk of its
-  // own (a hash of the tile's number) and wrap: the 70B shape's output projection (K = 8,192) 26.3 against 36.1 us at
-  // 1 to 16 rows, its QKV product 31.7 against 34.2, the 8B shape's down projection 23.6 against 24.2; a weight whose
-  // rows are no power of two long neither gains nor loses.  The start depends on the tile of rows of W alone.
-  // (counted in chunks of SK_KC, so that the order of the sums does not depend on the length of the pieces)
+  // crowd on few memory channels where that length is a power of two.  Every tile of rows therefore starts its walk
+  // over its chunks at a chunk of its own (a hash of the tile's number) and wraps: the 70B shape's output projection
+  // (K = 8,192) 26.3 against 36.1 us at 1 to 16 rows, its QKV product 31.7 against 34.2, the 8B shape's gate+up product
+  // from the file's layout 43.4 against 47.5 (41.8 from the copy laid out for this kernel), its head 187 either way;
+  // a weight whose rows are no power of two long neither gains nor loses.  The start depends on the tile of rows of W
+  // alone, and is counted in chunks of SK_KC, so that the order of the sums does not depend on the length of the pieces.
   const int span = c1 - c0, span_chunks = (span + PER_CHUNK - 1) / PER_CHUNK;
-  const int rot = (part != nullptr && span_chunks > 1)
+  const int rot = (span_chunks > 1)
                       ? (int)((((unsigned)blockIdx.x * 0x9E3779B1u) >> 8) % (unsigned)span_chunks) * PER_CHUNK : 0;
   auto ce = [&](int c) {
     const int k = c + rot;

@@ -192,15 +192,16 @@ def _room_for_copy(w: torch.Tensor) -> bool:
 def prepare_weights(rt, uses) -> None:
     """``uses``: (weight, epilogue, keep_split) of a part that has just been loaded.  On a GPU, in bfloat16 with the
     fast kernels: a weight with so many rows that the weight-streaming kernel gives every workgroup all of K (no
-    split: the gate+up matrix, the head) gets a second copy laid out for that kernel, in which a workgroup's 64
-    rows x 256 values of a chunk are consecutive, so that the workgroup reads one stretch of memory front to back
+    split: the gate+up matrix) gets a second copy laid out for that kernel, in which a workgroup's 64 rows x 256
+    values of a chunk are consecutive, so that the workgroup reads one stretch of memory front to back
     (``kernels.api.tile_weight``; the same bits).  Rows of the matrix as the file holds it lie K values apart, and a
-    workgroup that walks 64 of them side by side gets less out of the memory: measured on an MI355X, the head of
-    128,256 rows 177 against 194 us at one row, the 8B shape's decode step 3.83 against 3.98 ms at 8 requests (267
-    against 256 tokens/s at one), for 8.5 GB more memory (the 70B shape: 77 GB beside 141 GB of weights; copies are
-    made while COPIES_LEAVE_FREE of the device's memory stays free); weights whose K is split over workgroups gain
-    nothing (3.84 ms with copies of all).  The copy in the file's layout stays: the library's product for many rows reads
-    it.  With the measured route switched on, each use's shape is timed as well (once a process)."""
+    workgroup that walks 64 of them side by side gets less out of the memory: measured on an MI355X, the 8B shape's
+    gate+up product at 8 rows 41.8 against 43.4 us, the 13B shape's 53.2 against 57.5, the 70B shape's 168 against 175
+    (before the kernel's tiles of rows walked K from starts of their own the gap was twice that, and the head, which
+    is even now and gets no copy any more, gained 9 %), for 7.5 GB more memory (the 70B shape: 75 GB beside 141 GB of
+    weights; copies are made while COPIES_LEAVE_FREE of the device's memory stays free); weights whose K is split over
+    workgroups gain nothing.  The copy in the file's layout stays: the products for more rows read it.  With the
+    measured route switched on, each use's shape is timed as well (once a process)."""
     if not (rt.device.type == "cuda" and rt.dtype == torch.bfloat16 and rt.kernels == "auto"):
         return
     for w, epilogue, keep_split in uses:

@@ -340,9 +340,13 @@ def test_gemm_skinny_partial_sums_and_swiglu(M, N, K_):
     else:
         assert torch.equal(kept, plain.bfloat16())
     act = api.gemm_skinny(a, w, epilogue="swiglu", out_dtype=torch.float32)
-    g, u = plain[:, :N // 2].double(), plain[:, N // 2:].double()
     assert tuple(act.shape) == (M, N // 2)
-    assert torch.allclose(act.double(), g / (1 + torch.exp(-g)) * u, atol=1e-6, rtol=1e-5)
+    # against the activation of the exact sums: the kernel's sums carry fp32 rounding (a tile of columns walks K from
+    # a start of its own, so they are not the sums of the product without the activation bit for bit); silu has a
+    # slope of at most 1.1
+    g, u = want[:, :N // 2], want[:, N // 2:]
+    e = 2e-5 * math.sqrt(K_) * 0.05 + 1e-6 * want.abs().max().item()
+    assert bool(((act.double() - g / (1 + torch.exp(-g)) * u).abs() <= e * (1.1 * u.abs() + g.abs() + e) + 1e-6).all())
     actb = api.gemm_skinny(a, w, epilogue="swiglu")
     assert torch.equal(actb, act.bfloat16())
 
