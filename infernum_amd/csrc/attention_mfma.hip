@@ -75,6 +75,14 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 // loads of keys and values wait for no other global load, and a wave's next tile is in flight while it
 // works on this one.
 #define DEC_WAVES 4
+// A launch with no more workgroups than the GPU has compute units (few requests) gives a workgroup eight waves
+// instead of four: its keys are then read by twice the loads in flight (the 8B shape's decode step at 8 requests
+// 2,151 against 2,130 tokens/s, at one 274.5 against 271.9; with more workgroups than compute units four waves are
+// ahead: 12,620 against 12,274 tokens/s at 64 requests).  Head sizes above 128 keep four (the waves' partial results
+// would not fit the LDS twice).
+#define DEC_WAVES_FEW (IA_HEAD_DIM <= 128 ? 8 : 4)
+#define DEC_COMPUTE_UNITS 256
+static bool dec_wide(int B, int groups, int splits) { return (long long)B * groups * splits <= DEC_COMPUTE_UNITS; }
 #define DEC_BT_LDS 2048          // block-table entries kept in LDS (a longer slice is read from global memory)
 
 struct DecTile {                 // 16 keys as they come from memory: operands of the two products
@@ -220,14 +228,14 @@ struct DecFused {
 // FUSED: q is not read; every workgroup rotates the queries of its heads into LDS, the workgroups whose keys
 // include the token's own also make its key and value, use them from LDS (the loads from the page are replaced
 // in registers) and one of them (the first tile of heads) writes them to the page.
-template <bool FUSED, typename TS, bool POW2>
-__global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_decode_kernel(
+template <bool FUSED, typename TS, bool POW2, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, ((WAVES == 4 && HD <= 128) ? 3 : 1)) void attn_decode_kernel(
     const uint16_t* __restrict__ q, int q_row_stride, uint16_t* k_pages, uint16_t* v_pages,
     uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int bt_stride, int nh, int nkv, int ps,
     int num_pages, float scale_log2, int window, int num_splits, DecFused F) {
-  __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
-  __shared__ f32x4 s_o[DEC_WAVES][NS][64];
+  __shared__ float s_m[WAVES][16], s_l[WAVES][16];
+  __shared__ f32x4 s_o[WAVES][NS][64];
   __shared__ int s_bt[DEC_BT_LDS];
   __shared__ __attribute__((aligned(16))) uint16_t s_q[FUSED ? 16 : 1][HD];
   __shared__ __attribute__((aligned(16))) uint16_t s_newk[HD], s_newv[HD];
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
   const int G = nh / nkv, HT = (G + 15) / 16;
   const int g = blockIdx.y / HT, ht = blockIdx.y - g * HT;
   const int split = blockIdx.z;
-  constexpr int NT = DEC_WAVES * 64;
+  constexpr int NT = WAVES * 64;
   const int tid = threadIdx.x;
   const int hj = ht * 16 + j;
   const bool col_ok = hj < G;
@@ -371,17 +379,17 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
   }
   // two tiles in flight: the loads of the next tile of this wave are issued before this one is worked on
   while (t < tb) {
-    const bool more1 = t + DEC_WAVES < tb;
-    if (more1) dec_load<POW2>(geo, (t + DEC_WAVES) * 16, j, qd, B);
+    const bool more1 = t + WAVES < tb;
+    if (more1) dec_load<POW2>(geo, (t + WAVES) * 16, j, qd, B);
     dec_finish(geo, t * 16, j, qd, A);
     dec_compute(t * 16, A, qreg, pos, lo0, qd, scale_log2, o, m, l);
-    t += DEC_WAVES;
+    t += WAVES;
     if (!more1) break;
-    const bool more2 = t + DEC_WAVES < tb;
-    if (more2) dec_load<POW2>(geo, (t + DEC_WAVES) * 16, j, qd, A);
+    const bool more2 = t + WAVES < tb;
+    if (more2) dec_load<POW2>(geo, (t + WAVES) * 16, j, qd, A);
     dec_finish(geo, t * 16, j, qd, B);
     dec_compute(t * 16, B, qreg, pos, lo0, qd, scale_log2, o, m, l);
-    t += DEC_WAVES;
+    t += WAVES;
     if (!more2) break;
   }
   if (FUSED && own_key && ht == 0) {                         // to the page, for the steps to come
@@ -401,10 +409,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
   __syncthreads();
   float M = s_m[0][j];
 #pragma unroll
-  for (int w = 1; w < DEC_WAVES; ++w) M = fmaxf(M, s_m[w][j]);
+  for (int w = 1; w < WAVES; ++w) M = fmaxf(M, s_m[w][j]);
   float L = 0.f;
 #pragma unroll
-  for (int w = 0; w < DEC_WAVES; ++w) {
+  for (int w = 0; w < WAVES; ++w) {
     const float mw = s_m[w][j];
     L += (mw == -INFINITY ? 0.f : exp2f(mw - M)) * s_l[w][j];
   }
@@ -414,10 +422,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64, (HD <= 128 ? 3 : 1)) void attn_deco
   __syncthreads();
   if (!col_ok) return;
   // wave w finishes the slices n = w, w + 4, ... of the head
-  for (int n = wave; n < NS; n += DEC_WAVES) {
+  for (int n = wave; n < NS; n += WAVES) {
     f32x4 acc = s_o[0][n][lane];
 #pragma unroll
-    for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w][n][lane];
+    for (int w = 1; w < WAVES; ++w) acc += s_o[w][n][lane];
     if (num_splits == 1) {
       const float inv = 1.0f / L;
       uint2 wv;
@@ -887,12 +895,18 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
   const int G = nh / nkv, HT = (G + 15) / 16;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(B, nkv * HT, num_splits);
-#define DEC_LAUNCH(P2)                                                                                             \
-  attn_decode_kernel<false, bf16_t, P2><<<grid, DEC_WAVES * 64, 0, stream>>>(                                        \
+#define DEC_LAUNCH(P2, W)                                                                                          \
+  attn_decode_kernel<false, bf16_t, P2, W><<<grid, W * 64, 0, stream>>>(                                             \
       (const uint16_t*)q, q_row_stride, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, \
       part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{})
-  if ((ps & (ps - 1)) == 0) DEC_LAUNCH(true);
-  else DEC_LAUNCH(false);
+  const bool wide = dec_wide(B, nkv * HT, num_splits);
+  if ((ps & (ps - 1)) == 0) {
+    if (wide) DEC_LAUNCH(true, DEC_WAVES_FEW);
+    else DEC_LAUNCH(true, DEC_WAVES);
+  } else {
+    if (wide) DEC_LAUNCH(false, DEC_WAVES_FEW);
+    else DEC_LAUNCH(false, DEC_WAVES);
+  }
 #undef DEC_LAUNCH
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
@@ -933,18 +947,24 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
   F.freq_f64 = freq_f64;
   F.rot = rot;
   dim3 grid(B, nkv * HT, num_splits);
-#define DEC_FUSED_LAUNCH(TS, P2)                                                                                    \
-  attn_decode_kernel<true, TS, P2><<<grid, DEC_WAVES * 64, 0, stream>>>(                                            \
+#define DEC_FUSED_LAUNCH(TS, P2, W)                                                                                 \
+  attn_decode_kernel<true, TS, P2, W><<<grid, W * 64, 0, stream>>>(                                                 \
       nullptr, 0, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, part_ml, positions, \
       block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, F)
-  const bool pow2 = (ps & (ps - 1)) == 0;
+#define DEC_FUSED_WAVES(TS, P2)                       \
+  do {                                                \
+    if (wide) DEC_FUSED_LAUNCH(TS, P2, DEC_WAVES_FEW); \
+    else DEC_FUSED_LAUNCH(TS, P2, DEC_WAVES);         \
+  } while (0)
+  const bool pow2 = (ps & (ps - 1)) == 0, wide = dec_wide(B, nkv * HT, num_splits);
   if (src_dtype == IA_F32) {
-    if (pow2) DEC_FUSED_LAUNCH(float, true);
-    else DEC_FUSED_LAUNCH(float, false);
+    if (pow2) DEC_FUSED_WAVES(float, true);
+    else DEC_FUSED_WAVES(float, false);
   } else {
-    if (pow2) DEC_FUSED_LAUNCH(bf16_t, true);
-    else DEC_FUSED_LAUNCH(bf16_t, false);
+    if (pow2) DEC_FUSED_WAVES(bf16_t, true);
+    else DEC_FUSED_WAVES(bf16_t, false);
   }
+#undef DEC_FUSED_WAVES
 #undef DEC_FUSED_LAUNCH
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {

@@ -1041,6 +1041,51 @@ def test_attention_decode_rotating_equals_rotation_then_attention(nh, nkv, d, ps
     assert torch.equal(kp3.view(torch.int16), kp1.view(torch.int16)) and torch.equal(vp3.view(torch.int16), vp1.view(torch.int16))
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps,window,rot", [(8, 2, 128, 16, 0, 128), (6, 3, 48, 4, 0, 48), (40, 2, 64, 8, 0, 32),
+                                                    (5, 5, 16, 16, 0, 0), (2, 1, 256, 64, 0, 256), (4, 1, 96, 4, 17, 96),
+                                                    (3, 1, 80, 12, 0, 80)])
+def test_attention_decode_of_many_requests(nh, nkv, d, ps, window, rot):
+    """A launch with more workgroups than the GPU has compute units gives a workgroup four waves, one with fewer
+    eight (up to a head size of 128): the tests above are mostly of the second kind, this one, with 42 requests and
+    as many parts of the keys as it takes, is of the first.  Against the plain reference, and the launch that rotates
+    and writes the token's key and value against the two kernels one after the other, bit for bit."""
+    lens = [70, 1, 331, 64, 150, 16, 17] * 6
+    B = len(lens)
+    groups = nkv * (-(-(nh // nkv) // 16))
+    splits = 256 // (B * groups) + 1
+    assert B * groups * splits > 256
+    case = _paged_case(nh, nkv, d, ps, lens, [1] * B, torch.bfloat16, seed=d + nh + 3)
+    scale = 1.0 / math.sqrt(d)
+    out = torch.full((B, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K().attention_decode(case["q"], case["kp"], case["vp"], out, case["positions"], case["bt"], nh, nkv, d, scale,
+                         window, max(lens), num_splits=splits)
+    want = _ref_attention(case, nh, nkv, d, scale, window)
+    assert (out.double().cpu() - want).abs().max().item() <= 2e-2
+    # the same keys in few workgroups (one part, the first seven requests): eight waves a workgroup up to d = 128
+    few = torch.full((7, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K().attention_decode(case["q"][:7], case["kp"], case["vp"], few, case["positions"][:7], case["bt"][:7], nh, nkv, d,
+                         scale, window, max(lens), num_splits=1)
+    assert (few.double().cpu() - want[:7]).abs().max().item() <= 2e-2
+    # rotation inside the launch
+    g = torch.Generator().manual_seed(5)
+    W = (nh + 2 * nkv) * d
+    qkv = K().SplitSum(torch.randn(3, B, W, generator=g).to(DEV))
+    inv_freq = (10000.0 ** (-torch.arange(0, rot, 2, dtype=torch.float64) / rot)).to(DEV) if rot else None
+    pos = case["positions"]
+    slots = torch.tensor([int(case["bt"][b, (L - 1) // ps]) * ps + (L - 1) % ps for b, L in enumerate(lens)],
+                         dtype=torch.int32, device=DEV)
+    kp1, vp1 = case["kp"].clone(), case["vp"].clone()
+    q = K().rope_kv_append(qkv, pos, inv_freq, nh, nkv, d, rot, slots, kp1, vp1)
+    two = torch.full((B, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K().attention_decode(q, kp1, vp1, two, pos, case["bt"], nh, nkv, d, scale, window, max(lens), num_splits=splits)
+    kp2, vp2 = case["kp"].clone(), case["vp"].clone()
+    one = torch.full_like(two, float("nan"))
+    K().attention_decode_rotating(qkv, pos, inv_freq, rot, slots, kp2, vp2, one, case["bt"], nh, nkv, d, scale, window,
+                                  max(lens), num_splits=splits)
+    assert not two.isnan().any() and torch.equal(one, two)
+    assert torch.equal(kp2.view(torch.int16), kp1.view(torch.int16)) and torch.equal(vp2.view(torch.int16), vp1.view(torch.int16))
+
+
 @pytest.mark.parametrize("splits", [1, 3])
 def test_attention_mfma_decode_block_table_longer_than_its_lds_slice(splits):
     """18,000 keys in pages of 4: 4,500 block-table entries, more than the 2,048 the decode kernel keeps in LDS;
