@@ -380,10 +380,12 @@ def long_contexts(a) -> int:
 
 
 def decode_kernels_alone(a) -> int:
-    """The two kernels that a decode step of the 8B shape spends its time in, alone, on operands of the step's
-    sizes at batch 8 (what is in the operands does not change what the kernels do): the weight-streaming product
-    with each of a layer's four weights (the gate+up matrix in the layout made for it), and the attention over
-    527 cached tokens with the rotation and the write of the token's key and value inside.  For hardware counters
+    """The kernels that a decode step of the 8B shape spends its time in, alone, on operands of the step's sizes
+    at ``--batch`` requests (8 by default; what is in the operands does not change what the kernels do): the
+    product with each of a layer's four weights by the kernel that the routes of ``parts/linear.py`` give these
+    rows (at 8 rows the weight-streaming kernel, the gate+up matrix in the layout made for it; at 64 the LDS-tiled
+    kernel with K split over workgroups, or with the activation in its epilogue), and the attention over 527
+    cached tokens with the rotation and the write of the token's key and value inside.  For hardware counters
     (``rocprofv3 --pmc ... -- python3 bench.py --decode-kernels``): nothing else runs on the GPU, no library kernel
     either (the operands are uninitialised memory; tables and positions come from the host by copies)."""
     import math
@@ -404,15 +406,19 @@ def decode_kernels_alone(a) -> int:
     inv_freq = (500000.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)).to(dev)
     out = torch.empty((B, nh * d), **bf)
     times = {}
+    import importlib
+    L = importlib.import_module("infernum_amd.parts.linear")
+    from infernum_amd.parts.base import Runtime
+    rt = Runtime(torch.device(dev), torch.bfloat16)
     for name, N, Kd, epilogue in weights:
         w = torch.empty((N, Kd), **bf)
-        tiled = K.tile_weight(w, epilogue) if K.gemm_skinny_splits(N, Kd) == 1 else None
+        L.prepare_weights(rt, [(w, epilogue, epilogue is None)])        # the copy in the weight-streaming kernel's layout
         for _ in range(a.warmup):
-            K.gemm_skinny(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None, tiled=tiled)
+            L.linear(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None)
         sync()
         t0 = time.perf_counter()
         for _ in range(a.steps):
-            y = K.gemm_skinny(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None, tiled=tiled)
+            y = L.linear(x[Kd], w, epilogue=epilogue, keep_split=epilogue is None)
         sync()
         times[name] = round((time.perf_counter() - t0) / a.steps * 1e6, 1)
         if name == "qkv":
