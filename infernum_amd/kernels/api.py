@@ -357,10 +357,12 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     return out
 
 
-def gemm_mfma_swiglu(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def gemm_mfma_swiglu(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+                     tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(a @ w[:N/2]^T) * (a @ w[N/2:]^T) as bf16 [M, N/2]: the LDS-tiled MFMA product (tiles of 128 x 128) with
-    the activation on its fp32 sums in the epilogue, for up to some hundred rows."""
-    _dev(a, w, out)
+    the activation on its fp32 sums in the epilogue, for up to some hundred rows.  ``tiled``: the copy of ``w`` that
+    :func:`tile_weight` made with the "swiglu" epilogue, read instead of ``w`` (the same bits)."""
+    _dev(a, w, out, tiled)
     _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_mfma_swiglu: shapes")
     M, K = a.shape
     N = w.shape[0]
@@ -372,7 +374,13 @@ def gemm_mfma_swiglu(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tenso
         out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=a.device)
     _need(out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N // 2),
           f"gemm_mfma_swiglu: out must be contiguous bf16 [{M}, {N // 2}]")
-    _ok(_core().ia_gemm_mfma_swiglu(_p(a), _p(w), _p(out), M, N, K, _stream()), "gemm_mfma_swiglu")
+    if tiled is not None:
+        _core().ia_gemm_skinny_tiled_elements.restype = ctypes.c_size_t
+        _need(tiled.dtype == torch.bfloat16 and tiled.is_contiguous() and gemm_skinny_splits(N, K) == 1 and
+              tiled.numel() == int(_core().ia_gemm_skinny_tiled_elements(N, K, EPILOGUE["swiglu"])),
+              "gemm_mfma_swiglu: tiled is not the copy, made for the swiglu epilogue, of a weight that is not split over K")
+    _ok(_core().ia_gemm_mfma_swiglu(_p(a), _p(tiled if tiled is not None else w), int(tiled is not None), _p(out),
+                                    M, N, K, _stream()), "gemm_mfma_swiglu")
     return out
 
 

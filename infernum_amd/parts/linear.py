@@ -361,7 +361,7 @@ def _run(kind: str, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, ep
     if kind == "mfma_f32":
         return K.gemm_mfma_split(x, w, 1).parts[0], True
     if kind == "mfma_swiglu":
-        return K.gemm_mfma_swiglu(x, w), True
+        return K.gemm_mfma_swiglu(x, w, tiled=tiled_copy(w, "swiglu")), True
     if kind == "skinny":
         return K.gemm_skinny(x, w, epilogue=epilogue, out_dtype=out_dtype, tiled=tiled_copy(w, epilogue)), True
     if kind == "skinny_split":
@@ -452,7 +452,7 @@ def emit_linear(program, x: Any, M: Any, w: torch.Tensor, out_dtype: torch.dtype
             alts.append(P.Alt(g, out, r.parts, torch.float32))
             continue
         if r.kind == "mfma_swiglu":
-            program.op("core", "ia_gemm_mfma_swiglu", [x, w, out, M, N, Kdim, P.STREAM], g)
+            program.op("core", "ia_gemm_mfma_swiglu", [x, wk, int(tiled is not None), out, M, N, Kdim, P.STREAM], g)
             alts.append(P.Alt(g, out, 0, out_dtype))
             continue
         if r.kind == "mfma_f32":                # one part: the fp32 matrix itself

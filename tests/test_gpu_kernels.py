@@ -470,7 +470,7 @@ def test_gemm_mfma_split_picks_out_one_product_and_refuses_what_it_cannot_do():
 
 
 @pytest.mark.parametrize("M,N,K_", [(64, 1000, 192), (1, 66, 64), (128, 330, 256), (200, 2048, 448), (37, 254, 448),
-                                    (130, 260, 1024)])
+                                    (130, 260, 1024), (70, 16446, 448), (9, 28672, 512)])
 def test_gemm_mfma_swiglu(M, N, K_):
     """The LDS-tiled product with the activation in its epilogue: silu(first half) * second half from the fp32 sums,
     rounded once; tiles of 64 columns of the result at sizes that fill none, half widths that are no multiple of 4
@@ -492,6 +492,12 @@ def test_gemm_mfma_swiglu(M, N, K_):
         assert bool(((out.double() - other).abs() <= 2.0 ** -7 * want.abs() + 2 * e * (1.1 * up.abs() + gate.abs() + e)).all())
     # a row's result does not depend on the rows beside it
     assert torch.equal(api.gemm_mfma_swiglu(a[M - 1:M].contiguous(), w)[0], out[M - 1])
+    # from the copy laid out for the weight-streaming kernel (where that kernel does not split K): the same bits
+    if api.gemm_skinny_splits(N, K_) == 1:
+        assert torch.equal(api.gemm_mfma_swiglu(a, w, tiled=api.tile_weight(w, "swiglu")), out)
+    else:
+        with pytest.raises(api.KernelError):
+            api.gemm_mfma_swiglu(a, w, tiled=api.tile_weight(w, "swiglu"))
     with pytest.raises(api.KernelError):
         api.gemm_mfma_swiglu(a, w[:N - 1].contiguous())                                             # an odd number of rows
     with pytest.raises(api.KernelError):
