@@ -19,6 +19,13 @@
 // K must be a multiple of 64; M and N are arbitrary (rows beyond them are read from the last valid row and
 // not stored).  A result row depends on its own row of X only; how rows are grouped into tiles does not
 // change it.
+//
+// Three forms of the one kernel: the product as bf16 (the sums of the library's product, bit for bit, on the
+// shapes tried); SPLIT, for steps of some tens to some hundreds of rows, where the tiles of C alone would not fill
+// the GPU: K is dealt out over `splits` workgroups a tile and the fp32 sums of part p go to parts[p] for the next
+// kernel to add (one part: an fp32 result); GLU, silu(X W_first^T) * (X W_second^T) from the fp32 sums in the
+// epilogue, the rows of W of a wave's part alternating between the two halves of W.  In the last two a tile of
+// columns walks K from a step of its own (see ROTATE below).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
