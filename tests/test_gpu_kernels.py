@@ -772,6 +772,52 @@ def test_rope_from_partial_sums():
     assert torch.allclose(kp1.float(), kp3.float(), atol=6e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps,rot", [(6, 2, 48, 8, 48), (32, 8, 128, 16, 128), (5, 5, 16, 16, 8), (4, 1, 96, 4, 64), (3, 1, 80, 12, 80)])
+@pytest.mark.parametrize("S", [1, 2, 5])
+def test_rope_of_many_tokens_from_partial_sums(nh, nkv, d, ps, rot, S):
+    """From 32 tokens on, a product that comes as one part is rotated by another kernel (a workgroup a token, all
+    heads, 16-byte loads; the values to their transposed pages by a launch of their own where pages take eight tokens
+    at a time); a stack of partial sums stays with the kernel for few tokens, which adds the parts in the order of
+    their index.  Either way the first 9 of 40 tokens alone (the kernel for few tokens) give the same queries and
+    the same slots of the pages, bit for bit, and all 40 agree with plain arithmetic on the joined sums."""
+    api = K()
+    N = 40
+    row = (nh + 2 * nkv) * d
+    parts = _rand(S, N, row, seed=4 + S)
+    pos = torch.arange(3, 3 + N, dtype=torch.int32, device=DEV)
+    slots = torch.cat([torch.arange(16, 16 + 24), torch.randperm(16)[:16]]).to(torch.int32).to(DEV)   # a run, then scattered
+    num_pages = -(-56 // ps) + 1
+    inv = (1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    kp1 = torch.zeros(num_pages, nkv, ps, d, dtype=torch.bfloat16, device=DEV)
+    vp1 = torch.zeros(num_pages, nkv, d, ps, dtype=torch.bfloat16, device=DEV)
+    q1 = api.rope_kv_append(api.SplitSum(parts), pos, inv, nh, nkv, d, rot, slots, kp1, vp1)
+    kp2, vp2 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    few = api.SplitSum(parts[:, :9].contiguous())
+    q2 = api.rope_kv_append(few, pos[:9].contiguous(), inv, nh, nkv, d, rot, slots[:9].contiguous(), kp2, vp2)
+    assert torch.equal(q1[:9], q2)
+    for n in range(9):
+        pg, off = int(slots[n]) // ps, int(slots[n]) % ps
+        assert torch.equal(kp1[pg, :, off], kp2[pg, :, off]) and torch.equal(vp1[pg, :, :, off], vp2[pg, :, :, off])
+    # and against plain arithmetic on the joined sums
+    x = parts.double().sum(0).cpu()
+    ang = pos.cpu().double()[:, None] * inv.cpu().double()[None, :]
+    cs, sn = torch.cos(ang), torch.sin(ang)
+    half = rot // 2
+    for h in range(nh + nkv):
+        v = x[:, h * d:(h + 1) * d].clone()
+        a, b = v[:, :half].clone(), v[:, half:rot].clone()
+        v[:, :half], v[:, half:rot] = a * cs - b * sn, b * cs + a * sn
+        if h < nh:
+            got = q1[:, h * d:(h + 1) * d].double().cpu()
+        else:
+            got = torch.stack([kp1[int(slots[n]) // ps, h - nh, int(slots[n]) % ps] for n in range(N)]).double().cpu()
+        assert (got - v).abs().max().item() <= 2.0 ** -7 * v.abs().max().item() + 1e-3
+    for g in range(nkv):
+        v = x[:, (nh + nkv + g) * d:(nh + nkv + g + 1) * d]
+        got = torch.stack([vp1[int(slots[n]) // ps, g, :, int(slots[n]) % ps] for n in range(N)]).double().cpu()
+        assert (got - v).abs().max().item() <= 2.0 ** -7 * v.abs().max().item() + 1e-3
+
+
 # ------------------------------------------------------------------- attention
 def _paged_case(nh, nkv, d, ps, lens, q_lens, dtype, seed=0, scale_one=None, loud=(), q_lift=0.0):
     """Random queries/keys/values of several requests laid out into shuffled pages.
