@@ -95,9 +95,12 @@ KNOWN_MID_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int, int], ...]] = {
 
 # (N, K) of a gate+up weight -> bands (first row, last row) in which the LDS-tiled kernel with the activation in
 # its epilogue takes the product (the 8B shape's at 32 / 64 / 128 rows: 43 / 45 / 51 us against the weight-streaming
-# kernel's 47 / 56 / 73 and the library's with the activation's launch 54 / 54 / 57).
+# kernel's 47 / 56 / 73 and the library's with the activation's launch 54 / 54 / 57).  No rule of sizes stands behind
+# this table: 22,016 x 4,096 gains as the 8B shape does (38 / 42 / 48 us against 45 / 53 / 71 and 46 / 48 / 50), while for
+# 16,384 x 3,072 and 37,888 x 3,584 the library's product with the activation's launch is ahead from 32 rows on.
 KNOWN_GLU_ROWS: Dict[Tuple[int, int], Tuple[Tuple[int, int], ...]] = {
     (28672, 4096): ((17, 128),), (27648, 5120): ((33, 128),), (57344, 8192): ((17, 128),), (16384, 2048): ((129, 256),),
+    (22016, 4096): ((17, 128),),
 }
 
 ROUTES = ("table", "measured", "static")
@@ -143,16 +146,19 @@ MID_ROWS_MOST_PARTS = 8        # as far as measured
 
 
 def _mid_rows_by_size(N: int, K_: int) -> Tuple[Tuple[int, int, int], ...]:
-    """For shapes the table does not hold: per band of 128 rows (129 to 256, 257 to 384) as many parts as bring the
-    tiles of 128 x 128 to one workgroup a compute unit, while those are at least two (with one part the library was
-    as fast or faster for every shape measured) and a part keeps at least 8 steps of K."""
+    """For shapes the table does not hold: per band of rows (33 to 128, 129 to 256, 257 to 384: one, two and three
+    tiles of 128 rows) as many parts as bring the tiles of 128 x 128 to one workgroup a compute unit, while those are
+    at least two (with one part the library was as fast or faster for every shape measured) and a part keeps at
+    least 8 steps of K.  Measured beside the table's shapes on those of other models of the family (4,096 x 11,008,
+    12,288 x 4,096, 3,072 x 8,192, 5,120 x 3,072, 3,584 x 18,944, ...): ahead of the weight-streaming kernel and of the
+    library, or even with the better of them, from 32 rows on."""
     bands = []
     tiles_n = -(-N // 128)
-    for tiles_m in (2, 3):
+    for tiles_m in (1, 2, 3):
         parts = min(MID_ROWS_WORKGROUPS // (tiles_m * tiles_n), K_ // 64 // 8, MID_ROWS_MOST_PARTS)
         if parts < 2:
             break
-        bands.append((128 * (tiles_m - 1) + 1, 128 * tiles_m, parts))
+        bands.append((33 if tiles_m == 1 else 128 * (tiles_m - 1) + 1, 128 * tiles_m, parts))
     return tuple(bands)
 
 

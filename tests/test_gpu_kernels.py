@@ -623,9 +623,9 @@ def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split
         assert L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False), 200).kind == "library"
         previous = L.set_gemm_route("static")            # the rule of sizes alone
         try:
-            by_size = L._mid_rows_by_size(N, Kd)
+            at_200 = [parts for lo, hi, parts in L._mid_rows_by_size(N, Kd) if lo <= 200 <= hi]
             r = L.route_of(L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, True), 200)
-            assert (r.kind, r.parts) == (("mfma_split", by_size[0][2]) if by_size else ("library", 0))
+            assert (r.kind, r.parts) == (("mfma_split", at_200[0]) if at_200 else ("library", 0))
         finally:
             L.set_gemm_route(previous)
     # gate+up products: the tiled kernel with the activation in its epilogue for the bands of its table
@@ -636,7 +636,7 @@ def test_known_mid_rows_send_a_few_hundred_rows_to_the_tiled_kernel_with_k_split
             assert L.route_of(routes, lo - 1).kind != "mfma_swiglu" and L.route_of(routes, hi + 1).kind != "mfma_swiglu"
         assert all(r.kind != "mfma_swiglu" for r in L.plan(N, Kd, torch.bfloat16, torch.bfloat16, None, False))
     # a shape the table does not hold: as many parts as bring the tiles to a workgroup a compute unit, at least two
-    assert L.mid_rows(4096, 11008, True) == ((129, 256, 4), (257, 384, 2)) and L.mid_rows(4096, 11008, False) == ()
+    assert L.mid_rows(4096, 11008, True) == ((33, 128, 8), (129, 256, 4), (257, 384, 2)) and L.mid_rows(4096, 11008, False) == ()
     assert L.mid_rows(22016, 4096, True) == () and L.mid_rows(4096, 1000, True) == () and L.mid_rows(64, 448, True) == ()
     # the product through the route is the product: 8B shape's output projection at 200 rows
     x, w = _rand(200, 4096, dtype=torch.bfloat16, seed=5), _rand(4096, 4096, dtype=torch.bfloat16, scale=0.02, seed=6)
@@ -734,14 +734,14 @@ def test_known_routes_send_rows_to_the_library_where_the_table_says():
     assert kinds() == {1: "mfma_split", 16: "mfma_split", 17: "library", 64: "library", 128: "mfma_split", 129: "library"}
     saved = L.KNOWN_MID_ROWS.pop((15360, 5120))
     try:
-        assert L.mid_rows(15360, 5120, True) == ()           # the rule of sizes has none for so wide a weight
-        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "library", 64: "library", 128: "library", 129: "library"}
+        assert L.mid_rows(15360, 5120, True) == ((33, 128, 2),)      # the rule of sizes: 120 tiles of columns, two parts
+        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "library", 64: "mfma_split", 128: "mfma_split", 129: "library"}
     finally:
         L.KNOWN_MID_ROWS[(15360, 5120)] = saved
     previous = L.set_gemm_route("static")
     try:
-        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "skinny_split", 64: "skinny_split",
-                           128: "skinny_split", 129: "library"}
+        assert kinds() == {1: "skinny_split", 16: "skinny_split", 17: "skinny_split", 64: "mfma_split",
+                           128: "mfma_split", 129: "library"}
     finally:
         L.set_gemm_route(previous)
 
